@@ -1,0 +1,16 @@
+"""MI355X (gfx950) implementation of ArcticInference's ``csrc/custom_ops`` hot path.
+
+``arcticinference_amd.py_custom_ops`` is the drop-in counterpart of the
+reference's ``arctic_inference/py_custom_ops.py``: it loads the HIP library
+through its C ABI and registers the ``torch.ops.arctic_inference`` operators.
+"""
+__version__ = "0.1.0"
+
+from . import py_custom_ops  # noqa: F401
+from .py_custom_ops import (  # noqa: F401
+    reshape_and_cache_flash_bulk,
+    speculator_ln,
+    sum_lstm,
+    try_load_jit_library,
+    try_load_torch_library,
+)

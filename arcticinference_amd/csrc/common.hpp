@@ -1,0 +1,151 @@
+// Shared device helpers for the gfx950 kernels: 16-bit float conversion,
+// 16-byte vector access, wave64 DPP reductions and the error channel of the C ABI.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/arctic_mi355x.h"
+
+namespace arctic {
+
+// ---- error channel ---------------------------------------------------------
+int fail(int code, const char *fmt, ...);
+int check_launch(const char *what);
+
+// ---- 16-bit floats ---------------------------------------------------------
+// Activation element types. to_float is exact; from_float rounds to nearest
+// even (what __float2bfloat16 / __float2half do in the reference,
+// csrc/custom_ops/dtype_common.cuh:13-35).
+struct BF16 {
+  static constexpr int kCode = ARCTIC_DTYPE_BF16;
+  __device__ static __forceinline__ float lo(uint32_t w) {
+    return __uint_as_float(w << 16);
+  }
+  __device__ static __forceinline__ float hi(uint32_t w) {
+    return __uint_as_float(w & 0xffff0000u);
+  }
+  __device__ static __forceinline__ uint32_t round_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    return (f != f) ? 0x7fffu : r;
+  }
+  __device__ static __forceinline__ uint32_t pack(float a, float b) {
+    return round_bits(a) | (round_bits(b) << 16);
+  }
+  // value of the rounded 16-bit number, as fp32
+  __device__ static __forceinline__ float requant(float f) {
+    return __uint_as_float(round_bits(f) << 16);
+  }
+};
+
+struct F16 {
+  static constexpr int kCode = ARCTIC_DTYPE_F16;
+  __device__ static __forceinline__ float lo(uint32_t w) {
+    return __half2float(__ushort_as_half((unsigned short)(w & 0xffffu)));
+  }
+  __device__ static __forceinline__ float hi(uint32_t w) {
+    return __half2float(__ushort_as_half((unsigned short)(w >> 16)));
+  }
+  __device__ static __forceinline__ uint32_t round_bits(float f) {
+    return (uint32_t)__half_as_ushort(__float2half_rn(f));
+  }
+  __device__ static __forceinline__ uint32_t pack(float a, float b) {
+    return round_bits(a) | (round_bits(b) << 16);
+  }
+  __device__ static __forceinline__ float requant(float f) {
+    return __half2float(__float2half_rn(f));
+  }
+};
+
+// Eight 16-bit elements (one 16-byte lane access) unpacked to fp32 and back.
+template <typename T>
+__device__ __forceinline__ void unpack8(const uint4 &v, float (&f)[8]) {
+  f[0] = T::lo(v.x);
+  f[1] = T::hi(v.x);
+  f[2] = T::lo(v.y);
+  f[3] = T::hi(v.y);
+  f[4] = T::lo(v.z);
+  f[5] = T::hi(v.z);
+  f[6] = T::lo(v.w);
+  f[7] = T::hi(v.w);
+}
+
+template <typename T>
+__device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
+  uint4 v;
+  v.x = T::pack(f[0], f[1]);
+  v.y = T::pack(f[2], f[3]);
+  v.z = T::pack(f[4], f[5]);
+  v.w = T::pack(f[6], f[7]);
+  return v;
+}
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// Every tensor on these paths lives in device (global) memory.  Saying so keeps
+// the compiler from falling back to flat_* instructions when a pointer has been
+// round-tripped through LDS or a struct.
+#define ARCTIC_GLOBAL __attribute__((address_space(1)))
+
+__device__ __forceinline__ uint4 load16(const void *p) {
+  const u32x4 v = *(const ARCTIC_GLOBAL u32x4 *)p;
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+// streaming variants: every byte on these paths is touched exactly once
+__device__ __forceinline__ uint4 load16_stream(const void *p) {
+  const u32x4 v = __builtin_nontemporal_load((const ARCTIC_GLOBAL u32x4 *)p);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void store16_stream(void *p, const uint4 &v) {
+  const u32x4 t = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(t, (ARCTIC_GLOBAL u32x4 *)p);
+}
+__device__ __forceinline__ void store8_stream(void *p, const uint2 &v) {
+  const u32x2 t = {v.x, v.y};
+  __builtin_nontemporal_store(t, (ARCTIC_GLOBAL u32x2 *)p);
+}
+__device__ __forceinline__ void store4_stream(void *p, uint32_t v) {
+  __builtin_nontemporal_store(v, (ARCTIC_GLOBAL uint32_t *)p);
+}
+
+// ---- wave64 / workgroup reductions ------------------------------------------
+// DPP butterfly inside each row of 16 lanes, then the four row totals are read
+// with v_readlane.  Every lane returns the same wave total.
+template <int kCtrl>
+__device__ __forceinline__ float dpp_add(float v) {
+  int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xf, 0xf, true);
+  return v + __int_as_float(moved);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+  v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+  v = dpp_add<0x141>(v);  // row_half_mirror
+  v = dpp_add<0x140>(v);  // row_mirror
+  const int b = __float_as_int(v);
+  float r0 = __int_as_float(__builtin_amdgcn_readlane(b, 0));
+  float r1 = __int_as_float(__builtin_amdgcn_readlane(b, 16));
+  float r2 = __int_as_float(__builtin_amdgcn_readlane(b, 32));
+  float r3 = __int_as_float(__builtin_amdgcn_readlane(b, 48));
+  return (r0 + r1) + (r2 + r3);
+}
+
+// Sum over the whole workgroup (blockDim.x a multiple of 64, at most 1024).
+// `slots` is LDS for 16 floats, private to this call site; all threads get the
+// same value because all of them add the partials in the same order.
+__device__ __forceinline__ float block_sum(float v, float *slots) {
+  v = wave_sum(v);
+  const int nwaves = blockDim.x >> 6;
+  if (nwaves == 1) return v;
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) slots[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < nwaves; ++w) total += slots[w];
+  return total;
+}
+
+}  // namespace arctic

@@ -1,0 +1,378 @@
+// SwiftKV bulk KV-cache write for gfx950.
+//
+// Replaces reshape_and_cache_flash_bulk (host launcher and kernel,
+// csrc/custom_ops/reshape_and_cache_flash_bulk.cu:12-144 in the reference).
+//
+// Work decomposition
+// ------------------
+// One workgroup owns one token and a run of consecutive layers.  The token's
+// slot is looked up once; a prologue turns (slot, layer, K|V) into a table of
+// row descriptors in LDS - destination address of the token's row in that
+// layer's cache and the fp64 reciprocal of that layer's scale - with one lane per
+// row, so the per-layer pointer and scale reads are issued together instead of
+// one dependent pair per layer.  The main loop then streams the token's source
+// rows: every lane moves 16 bytes per access (8 bf16/fp16 or 4 fp32 elements),
+// consecutive lanes cover consecutive addresses along head_size, and the cache
+// row is written with 16-byte (copy) or 8-byte (fp8, 8 codes) stores.  Source
+// and destination are each touched exactly once, so both use streaming
+// (non-temporal) accesses.
+//
+// The four per-layer pointer tables travel in the kernel-argument segment, so a
+// call uploads nothing and can be recorded into a HIP graph.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <type_traits>
+
+#include "common.hpp"
+#include "fp8_convert.hpp"
+
+namespace arctic {
+
+constexpr int kBulkThreads = 256;
+constexpr int kLayersPerLaunch = 64;  // 4 tables x 64 pointers = 2 KiB of kernel arguments
+
+struct LayerTables {
+  const void *key_cache[kLayersPerLaunch];
+  const void *value_cache[kLayersPerLaunch];
+  const float *k_scale[kLayersPerLaunch];
+  const float *v_scale[kLayersPerLaunch];
+};
+
+struct BulkParams {
+  const char *keys;    // already offset to the first layer of this launch
+  const char *values;
+  const int64_t *slot_mapping;
+  int64_t key_stride_bytes;
+  int64_t value_stride_bytes;
+  int64_t block_stride;  // elements
+  int num_layers;        // layers in this launch
+  int layers_per_group;  // consecutive layers owned by one workgroup
+  int groups_per_token;
+  int n;                 // num_heads * head_size
+  int block_size;
+  int chunks_per_row;    // 16-byte source chunks per (token, layer) row
+  int chunk_shift;       // log2(chunks_per_row) or -1
+};
+
+struct __align__(16) RowDesc {
+  char *dst;    // first byte of this token's row in the layer's K or V cache
+  double inv;   // RN64(1 / scale); unused by the copy path
+};
+
+// ---- element-type plumbing ---------------------------------------------------
+struct SrcBF16 {
+  static constexpr int kElemsPerChunk = 8;
+  static constexpr int kBytes = 2;
+  __device__ static __forceinline__ void to_float(const uint4 &v, float (&f)[8]) { unpack8<BF16>(v, f); }
+};
+struct SrcF16 {
+  static constexpr int kElemsPerChunk = 8;
+  static constexpr int kBytes = 2;
+  __device__ static __forceinline__ void to_float(const uint4 &v, float (&f)[8]) { unpack8<F16>(v, f); }
+};
+struct SrcF32 {
+  static constexpr int kElemsPerChunk = 4;
+  static constexpr int kBytes = 4;
+};
+
+struct Copy {};  // ARCTIC_KV_AUTO
+
+template <typename F8>
+__device__ __forceinline__ void quantize_store(char *dst, const float (&f)[8], double inv) {
+  uint2 out;
+  out.x = encode4<F8>(div_by_scale(f[0], inv), div_by_scale(f[1], inv),
+                      div_by_scale(f[2], inv), div_by_scale(f[3], inv));
+  out.y = encode4<F8>(div_by_scale(f[4], inv), div_by_scale(f[5], inv),
+                      div_by_scale(f[6], inv), div_by_scale(f[7], inv));
+  store8_stream(dst, out);
+}
+
+// One 16-byte source chunk -> cache.  `col` is the chunk's index inside its row.
+template <typename Src, typename Dst>
+__device__ __forceinline__ void emit_chunk(const uint4 &v, const RowDesc &d, int col) {
+  if constexpr (std::is_same<Dst, Copy>::value) {
+    store16_stream(d.dst + (int64_t)col * 16, v);
+  } else if constexpr (Src::kElemsPerChunk == 8) {
+    float f[8];
+    Src::to_float(v, f);
+    quantize_store<Dst>(d.dst + (int64_t)col * 8, f, d.inv);
+  } else {
+    const uint32_t w = encode4<Dst>(div_by_scale(__uint_as_float(v.x), d.inv),
+                                    div_by_scale(__uint_as_float(v.y), d.inv),
+                                    div_by_scale(__uint_as_float(v.z), d.inv),
+                                    div_by_scale(__uint_as_float(v.w), d.inv));
+    store4_stream(d.dst + (int64_t)col * 4, w);
+  }
+}
+
+template <typename Src, typename Dst, bool kPow2>
+__global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
+    const BulkParams p, const LayerTables tab) {
+  constexpr bool kCopy = std::is_same<Dst, Copy>::value;
+  constexpr int kDstElemBytes = kCopy ? Src::kBytes : 1;
+  constexpr int kUnroll = 4;
+
+  __shared__ RowDesc rows[2 * kLayersPerLaunch];
+
+  const int64_t token = blockIdx.x / p.groups_per_token;
+  const int group = blockIdx.x - (int)(token * p.groups_per_token);
+  const int layer0 = group * p.layers_per_group;
+  const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
+
+  const int64_t slot = p.slot_mapping[token];
+  if (slot < 0) return;  // padding token: uniform exit, before any barrier
+
+  int64_t blk, off;
+  if (slot < 0x7fffffffLL) {
+    const uint32_t s32 = (uint32_t)slot, bs = (uint32_t)p.block_size;
+    blk = s32 / bs;
+    off = s32 - (uint32_t)blk * bs;
+  } else {
+    blk = slot / p.block_size;
+    off = slot - blk * p.block_size;
+  }
+  const int64_t row_elem = blk * p.block_stride + off * (int64_t)p.n;
+
+  // prologue: one lane per (layer, K|V) row of this token
+  for (int r = threadIdx.x; r < 2 * nlayers; r += kBulkThreads) {
+    const int layer = layer0 + (r >> 1);
+    const bool is_v = r & 1;
+    const void *base = is_v ? tab.value_cache[layer] : tab.key_cache[layer];
+    RowDesc d;
+    d.dst = (char *)base + row_elem * kDstElemBytes;
+    d.inv = 0.0;
+    if constexpr (!kCopy) {
+      const float *sp = is_v ? tab.v_scale[layer] : tab.k_scale[layer];
+      d.inv = 1.0 / (double)(*sp);
+    }
+    rows[r] = d;
+  }
+  __syncthreads();
+
+  const char *ksrc = p.keys + token * p.key_stride_bytes + (int64_t)layer0 * p.n * Src::kBytes;
+  const char *vsrc = p.values + token * p.value_stride_bytes + (int64_t)layer0 * p.n * Src::kBytes;
+  const int cpr = p.chunks_per_row;
+  const int total = 2 * nlayers * cpr;  // chunks this workgroup moves
+
+  auto locate = [&](int c, int &r, int &col) {
+    if constexpr (kPow2) {
+      r = c >> p.chunk_shift;
+      col = c & (cpr - 1);
+    } else {
+      r = c / cpr;
+      col = c - r * cpr;
+    }
+  };
+  auto src_of = [&](int r, int col) -> const char * {
+    const char *base = (r & 1) ? vsrc : ksrc;
+    return base + ((int64_t)(r >> 1) * cpr + col) * 16;
+  };
+
+  int c = threadIdx.x;
+  // main loop: kUnroll independent 16-byte loads in flight per lane
+  for (; c + (kUnroll - 1) * kBulkThreads < total; c += kUnroll * kBulkThreads) {
+    uint4 v[kUnroll];
+    int r[kUnroll], col[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      locate(c + u * kBulkThreads, r[u], col[u]);
+      v[u] = load16_stream(src_of(r[u], col[u]));
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) emit_chunk<Src, Dst>(v[u], rows[r[u]], col[u]);
+  }
+  for (; c < total; c += kBulkThreads) {
+    int r, col;
+    locate(c, r, col);
+    const uint4 v = load16_stream(src_of(r, col));
+    emit_chunk<Src, Dst>(v, rows[r], col);
+  }
+}
+
+// Fallback for shapes or addresses that do not allow 16-byte accesses: one
+// element per lane per step, any alignment.  Same arithmetic, no vector access.
+template <typename SrcElem, typename Dst>
+__global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_scalar_kernel(
+    const BulkParams p, const LayerTables tab, const int src_dtype) {
+  constexpr bool kCopy = std::is_same<Dst, Copy>::value;
+  const int64_t token = blockIdx.x / p.groups_per_token;
+  const int group = blockIdx.x - (int)(token * p.groups_per_token);
+  const int layer0 = group * p.layers_per_group;
+  const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
+  const int64_t slot = p.slot_mapping[token];
+  if (slot < 0) return;
+  const int64_t blk = slot / p.block_size;
+  const int64_t off = slot - blk * p.block_size;
+  const int64_t row_elem = blk * p.block_stride + off * (int64_t)p.n;
+  const SrcElem *ks = reinterpret_cast<const SrcElem *>(p.keys + token * p.key_stride_bytes);
+  const SrcElem *vs = reinterpret_cast<const SrcElem *>(p.values + token * p.value_stride_bytes);
+
+  for (int l = layer0; l < layer0 + nlayers; ++l) {
+    double kinv = 0.0, vinv = 0.0;
+    if constexpr (!kCopy) {
+      kinv = 1.0 / (double)(*tab.k_scale[l]);
+      vinv = 1.0 / (double)(*tab.v_scale[l]);
+    }
+    for (int i = threadIdx.x; i < p.n; i += kBulkThreads) {
+      const SrcElem k = ks[(int64_t)l * p.n + i];
+      const SrcElem v = vs[(int64_t)l * p.n + i];
+      if constexpr (kCopy) {
+        ((SrcElem *)tab.key_cache[l])[row_elem + i] = k;
+        ((SrcElem *)tab.value_cache[l])[row_elem + i] = v;
+      } else {
+        float kf, vf;
+        if constexpr (sizeof(SrcElem) == 4) {
+          kf = __uint_as_float((uint32_t)k);
+          vf = __uint_as_float((uint32_t)v);
+        } else if (src_dtype == ARCTIC_DTYPE_BF16) {
+          kf = BF16::lo((uint32_t)k);
+          vf = BF16::lo((uint32_t)v);
+        } else {
+          kf = F16::lo((uint32_t)k);
+          vf = F16::lo((uint32_t)v);
+        }
+        const uint32_t wk = encode4<Dst>(div_by_scale(kf, kinv), 0.f, 0.f, 0.f);
+        const uint32_t wv = encode4<Dst>(div_by_scale(vf, vinv), 0.f, 0.f, 0.f);
+        ((uint8_t *)tab.key_cache[l])[row_elem + i] = (uint8_t)(wk & 0xffu);
+        ((uint8_t *)tab.value_cache[l])[row_elem + i] = (uint8_t)(wv & 0xffu);
+      }
+    }
+  }
+}
+
+template <typename Src, typename Dst>
+static void launch_vec(const BulkParams &p, const LayerTables &tab, int64_t grid, hipStream_t s) {
+  if (p.chunk_shift >= 0)
+    hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true>), dim3((unsigned)grid), dim3(kBulkThreads), 0, s, p, tab);
+  else
+    hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, false>), dim3((unsigned)grid), dim3(kBulkThreads), 0, s, p, tab);
+}
+template <typename SrcElem, typename Dst>
+static void launch_scalar(const BulkParams &p, const LayerTables &tab, int64_t grid, int src_dtype,
+                          hipStream_t s) {
+  hipLaunchKernelGGL((kv_write_bulk_scalar_kernel<SrcElem, Dst>), dim3((unsigned)grid),
+                     dim3(kBulkThreads), 0, s, p, tab, src_dtype);
+}
+
+template <typename Dst>
+static void dispatch_src(bool vec, int src_dtype, const BulkParams &p, const LayerTables &tab,
+                         int64_t grid, hipStream_t s) {
+  if (vec) {
+    switch (src_dtype) {
+      case ARCTIC_DTYPE_BF16: launch_vec<SrcBF16, Dst>(p, tab, grid, s); break;
+      case ARCTIC_DTYPE_F16: launch_vec<SrcF16, Dst>(p, tab, grid, s); break;
+      default: launch_vec<SrcF32, Dst>(p, tab, grid, s); break;
+    }
+  } else {
+    if (src_dtype == ARCTIC_DTYPE_F32)
+      launch_scalar<uint32_t, Dst>(p, tab, grid, src_dtype, s);
+    else
+      launch_scalar<uint16_t, Dst>(p, tab, grid, src_dtype, s);
+  }
+}
+
+static inline bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p % a) == 0; }
+
+}  // namespace arctic
+
+using namespace arctic;
+
+extern "C" int arctic_reshape_and_cache_flash_bulk(
+    const void *keys, const void *values, int64_t key_stride, int64_t value_stride,
+    const void *const *key_cache_ptrs, const void *const *value_cache_ptrs,
+    const float *const *k_scale_ptrs, const float *const *v_scale_ptrs,
+    const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads,
+    int head_size, int block_size, int64_t block_stride, int src_dtype, int kv_cache_dtype,
+    void *stream) {
+  const char *fn = "reshape_and_cache_flash_bulk";
+  if (num_layers == 0 || num_tokens == 0) return ARCTIC_OK;  // reference :87-89
+  if (num_layers < 0 || num_layers > ARCTIC_MAX_LAYERS)
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: num_layers=%d outside [0, %d]", fn, num_layers,
+                ARCTIC_MAX_LAYERS);
+  if (num_tokens < 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: num_tokens=%lld < 0", fn, (long long)num_tokens);
+  if (num_heads <= 0 || head_size <= 0 || block_size <= 0)
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: num_heads, head_size and block_size must be positive", fn);
+  if (src_dtype != ARCTIC_DTYPE_F32 && src_dtype != ARCTIC_DTYPE_F16 && src_dtype != ARCTIC_DTYPE_BF16)
+    return fail(ARCTIC_ERR_UNSUPPORTED, "%s: Unsupported input type of kv cache: %d", fn, src_dtype);
+  if (kv_cache_dtype != ARCTIC_KV_AUTO && kv_cache_dtype != ARCTIC_KV_FP8_E4M3 &&
+      kv_cache_dtype != ARCTIC_KV_FP8_E5M2)
+    return fail(ARCTIC_ERR_UNSUPPORTED, "%s: Unsupported data type of kv cache: %d", fn, kv_cache_dtype);
+  if (!keys || !values || !slot_mapping || !key_cache_ptrs || !value_cache_ptrs)
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
+  const bool quant = kv_cache_dtype != ARCTIC_KV_AUTO;
+  if (quant && (!k_scale_ptrs || !v_scale_ptrs))
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: fp8 cache needs k_scales and v_scales", fn);
+  const int64_t n64 = (int64_t)num_heads * head_size;
+  if (n64 > (1 << 24)) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: num_heads*head_size too large", fn);
+  const int n = (int)n64;
+  for (int l = 0; l < num_layers; ++l) {
+    if (!key_cache_ptrs[l] || !value_cache_ptrs[l])
+      return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null cache pointer for layer %d", fn, l);
+    if (quant && (!k_scale_ptrs[l] || !v_scale_ptrs[l]))
+      return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null scale pointer for layer %d", fn, l);
+  }
+
+  const int es = src_dtype == ARCTIC_DTYPE_F32 ? 4 : 2;
+  const int des = quant ? 1 : es;
+  const int epc = 16 / es;  // elements per 16-byte chunk
+  // 16-byte loads need aligned rows; stores are 16 B (copy), 8 B (fp8 from 16-bit) or 4 B (fp8 from fp32)
+  const int store_bytes = quant ? epc : 16;
+  bool vec = (n % epc == 0) && aligned(keys, 16) && aligned(values, 16) &&
+             ((key_stride * es) % 16 == 0 || num_tokens == 1) &&
+             ((value_stride * es) % 16 == 0 || num_tokens == 1) && ((block_stride * des) % store_bytes == 0);
+  for (int l = 0; vec && l < num_layers; ++l)
+    vec = aligned(key_cache_ptrs[l], store_bytes) && aligned(value_cache_ptrs[l], store_bytes);
+
+  hipStream_t s = (hipStream_t)stream;
+  for (int first = 0; first < num_layers; first += kLayersPerLaunch) {
+    const int count = std::min(kLayersPerLaunch, num_layers - first);
+    LayerTables tab;
+    for (int l = 0; l < kLayersPerLaunch; ++l) {
+      const bool in = l < count;
+      tab.key_cache[l] = in ? key_cache_ptrs[first + l] : nullptr;
+      tab.value_cache[l] = in ? value_cache_ptrs[first + l] : nullptr;
+      tab.k_scale[l] = (in && quant) ? k_scale_ptrs[first + l] : nullptr;
+      tab.v_scale[l] = (in && quant) ? v_scale_ptrs[first + l] : nullptr;
+    }
+    BulkParams p;
+    p.keys = (const char *)keys + (int64_t)first * n * es;
+    p.values = (const char *)values + (int64_t)first * n * es;
+    p.slot_mapping = slot_mapping;
+    p.key_stride_bytes = key_stride * es;
+    p.value_stride_bytes = value_stride * es;
+    p.block_stride = block_stride;
+    p.num_layers = count;
+    p.n = n;
+    p.block_size = block_size;
+    p.chunks_per_row = vec ? n / epc : 0;
+    p.chunk_shift = -1;
+    if (vec && (p.chunks_per_row & (p.chunks_per_row - 1)) == 0) p.chunk_shift = __builtin_ctz(p.chunks_per_row);
+
+    // Split a token's layers over several workgroups when there are too few
+    // tokens to fill the 256 CUs, but keep every workgroup at >= 4 steps of work.
+    const int64_t want_groups = 8192;
+    int groups = (int)std::min<int64_t>(count, (want_groups + num_tokens - 1) / num_tokens);
+    if (vec) {
+      const int64_t chunks_per_layer = 2LL * p.chunks_per_row;
+      const int min_layers = (int)std::max<int64_t>(1, (4LL * kBulkThreads + chunks_per_layer - 1) / chunks_per_layer);
+      groups = std::min(groups, std::max(1, count / min_layers));
+    }
+    groups = std::max(groups, 1);
+    p.layers_per_group = (count + groups - 1) / groups;
+    p.groups_per_token = (count + p.layers_per_group - 1) / p.layers_per_group;
+    const int64_t grid = num_tokens * p.groups_per_token;
+    if (grid > 0x7fffffffLL)
+      return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: too many tokens (%lld)", fn, (long long)num_tokens);
+
+    switch (kv_cache_dtype) {
+      case ARCTIC_KV_AUTO: dispatch_src<Copy>(vec, src_dtype, p, tab, grid, s); break;
+      case ARCTIC_KV_FP8_E4M3: dispatch_src<E4M3>(vec, src_dtype, p, tab, grid, s); break;
+      default: dispatch_src<E5M2>(vec, src_dtype, p, tab, grid, s); break;
+    }
+    const int rc = check_launch(fn);
+    if (rc) return rc;
+  }
+  return ARCTIC_OK;
+}

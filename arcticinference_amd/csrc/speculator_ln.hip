@@ -1,0 +1,145 @@
+// Speculator "LayerNorm" (RMS norm with optional scale and shift) for gfx950.
+//
+// Replaces speculator_ln_cuda and its kernels
+// (csrc/custom_ops/speculator_ln.cu:21-252 in the reference).
+//
+// One workgroup per row.  On the vector path every lane keeps its 16-byte
+// chunks of the row in registers between the sum of squares and the scaling, so
+// the row is read from HBM once (the reference reads it twice); the sum is a DPP
+// wave reduction followed by a small LDS combine.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+
+#include "common.hpp"
+
+namespace arctic {
+
+template <typename T, int kChunksPerThread>
+__global__ __launch_bounds__(1024) void spec_ln_vec_kernel(
+    char *__restrict__ out, const char *__restrict__ in, const char *__restrict__ weight,
+    const char *__restrict__ bias, int64_t in_row_stride_bytes, int hidden, float eps) {
+  __shared__ float slots[16];
+  const int chunks = hidden >> 3;
+  const char *row_in = in + (int64_t)blockIdx.x * in_row_stride_bytes;
+  char *row_out = out + (int64_t)blockIdx.x * hidden * 2;
+
+  uint4 raw[kChunksPerThread];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < kChunksPerThread; ++k) {
+    const int c = threadIdx.x + k * blockDim.x;
+    raw[k] = make_uint4(0, 0, 0, 0);
+    if (c < chunks) raw[k] = load16_stream(row_in + (int64_t)c * 16);
+  }
+#pragma unroll
+  for (int k = 0; k < kChunksPerThread; ++k) {
+    float x[8];
+    unpack8<T>(raw[k], x);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss += x[j] * x[j];
+  }
+  const float total = block_sum(ss, slots);
+  const float inv = rsqrtf(total / (float)hidden + eps);
+
+#pragma unroll
+  for (int k = 0; k < kChunksPerThread; ++k) {
+    const int c = threadIdx.x + k * blockDim.x;
+    if (c >= chunks) continue;
+    float x[8];
+    unpack8<T>(raw[k], x);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] *= inv;
+    if (weight) {
+      float w[8];
+      unpack8<T>(load16(weight + (int64_t)c * 16), w);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[j] *= w[j];
+    }
+    if (bias) {
+      float b[8];
+      unpack8<T>(load16(bias + (int64_t)c * 16), b);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[j] += b[j];
+    }
+    store16_stream(row_out + (int64_t)c * 16, pack8<T>(x));
+  }
+}
+
+// Any hidden size, any alignment: element-wise, two passes over the row.
+template <typename T>
+__global__ __launch_bounds__(256) void spec_ln_scalar_kernel(
+    uint16_t *__restrict__ out, const uint16_t *__restrict__ in, const uint16_t *__restrict__ weight,
+    const uint16_t *__restrict__ bias, int64_t in_row_stride, int hidden, float eps) {
+  __shared__ float slots[16];
+  const uint16_t *row_in = in + (int64_t)blockIdx.x * in_row_stride;
+  uint16_t *row_out = out + (int64_t)blockIdx.x * hidden;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
+    const float x = T::lo(row_in[j]);
+    ss += x * x;
+  }
+  const float total = block_sum(ss, slots);
+  const float inv = rsqrtf(total / (float)hidden + eps);
+  for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
+    float y = T::lo(row_in[j]) * inv;
+    if (weight) y *= T::lo(weight[j]);
+    if (bias) y += T::lo(bias[j]);
+    row_out[j] = (uint16_t)T::round_bits(y);
+  }
+}
+
+static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+template <typename T>
+static void launch_ln(void *out, const void *in, const void *w, const void *b, int64_t rows, int hidden,
+                      int64_t in_row_stride, float eps, hipStream_t s) {
+  const int chunks = hidden / 8;
+  const bool vec = (hidden % 8 == 0) && (in_row_stride % 8 == 0 || rows == 1) && aligned16(in) &&
+                   aligned16(out) && (!w || aligned16(w)) && (!b || aligned16(b)) && chunks <= 8 * 1024;
+  const dim3 grid((unsigned)rows);
+  if (vec) {
+    int cpt = 1;
+    while (cpt < 8 && (chunks + cpt - 1) / cpt > 1024) cpt *= 2;
+    int threads = (chunks + cpt - 1) / cpt;
+    threads = std::max(64, (threads + 63) & ~63);
+    const int64_t stride_bytes = in_row_stride * 2;
+#define ARCTIC_LN_LAUNCH(CPT)                                                                         \
+  hipLaunchKernelGGL((spec_ln_vec_kernel<T, CPT>), grid, dim3(threads), 0, s, (char *)out,             \
+                     (const char *)in, (const char *)w, (const char *)b, stride_bytes, hidden, eps)
+    switch (cpt) {
+      case 1: ARCTIC_LN_LAUNCH(1); break;
+      case 2: ARCTIC_LN_LAUNCH(2); break;
+      case 4: ARCTIC_LN_LAUNCH(4); break;
+      default: ARCTIC_LN_LAUNCH(8); break;
+    }
+#undef ARCTIC_LN_LAUNCH
+  } else {
+    hipLaunchKernelGGL((spec_ln_scalar_kernel<T>), grid, dim3(256), 0, s, (uint16_t *)out,
+                       (const uint16_t *)in, (const uint16_t *)w, (const uint16_t *)b, in_row_stride, hidden,
+                       eps);
+  }
+}
+
+}  // namespace arctic
+
+using namespace arctic;
+
+extern "C" int arctic_speculator_ln(void *out, const void *in, const void *weight, const void *bias,
+                                    int64_t rows, int hidden, int64_t in_row_stride, float eps, int dtype,
+                                    void *stream) {
+  const char *fn = "speculator_ln";
+  if (dtype != ARCTIC_DTYPE_F16 && dtype != ARCTIC_DTYPE_BF16)
+    return fail(ARCTIC_ERR_UNSUPPORTED, "%s: only fp16 and bf16 are supported.", fn);
+  if (hidden <= 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: hidden size must be > 0", fn);
+  if (rows < 0 || rows > 0x7fffffffLL) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: bad row count", fn);
+  if (rows == 0) return ARCTIC_OK;
+  if (!out || !in) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == ARCTIC_DTYPE_BF16)
+    launch_ln<BF16>(out, in, weight, bias, rows, hidden, in_row_stride, eps, s);
+  else
+    launch_ln<F16>(out, in, weight, bias, rows, hidden, in_row_stride, eps, s);
+  return check_launch(fn);
+}

@@ -1,0 +1,411 @@
+"""Drop-in ``torch.ops.arctic_inference.*`` surface backed by gfx950 HIP kernels.
+
+Mirrors the operator boundary of the reference
+(``arctic_inference/py_custom_ops.py:9-118`` and the schemas in
+``csrc/custom_ops/torch_bindings.cpp:6-51``): same namespace, same schema
+strings, same wrapper names and argument meaning, the same argument checks with
+the same message prefixes.  The reference registers compiled C++ functions from
+a pybind extension; here the schemas are defined from Python and the ``CUDA``
+dispatch key (HIP tensors under PyTorch-ROCm) is bound to thin shims that unwrap
+tensors into pointers, sizes and strides and call the C ABI of
+``libarctic_mi355x.so`` on the current stream.
+
+There is no fallback: without the shared object ``try_load_torch_library()``
+returns ``False`` (as the reference does) and every operator raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import logging
+from typing import List, Optional, Tuple
+
+import torch
+
+from . import _native
+
+logger = logging.getLogger(__name__)
+
+_NAMESPACE = "arctic_inference"
+
+# Schemas as registered by the reference (csrc/custom_ops/torch_bindings.cpp:7-49).
+_SCHEMAS = {
+    "reshape_and_cache_flash_bulk":
+        "reshape_and_cache_flash_bulk(Tensor keys, Tensor values, Tensor(c!)[] key_caches, "
+        "Tensor(d!)[] value_caches, Tensor slot_mapping, str kv_cache_dtype, Tensor(e)[] k_scales, "
+        "Tensor(f)[] v_scales, int num_heads, int head_size) -> ()",
+    "reshape_and_cache_flash_fp4":
+        "reshape_and_cache_flash_fp4(Tensor key, Tensor value, Tensor(c!) key_cache, "
+        "Tensor(d!) value_cache, Tensor slot_mapping, str kv_cache_dtype, Tensor k_scale, "
+        "Tensor v_scale, Tensor(e!) key_scale_cache, Tensor(f!) value_scale_cache) -> ()",
+    "speculator_ln_cuda":
+        "speculator_ln_cuda(Tensor input, Tensor? weight, Tensor? bias, float eps) -> Tensor",
+    "sum_lstm_cuda":
+        "sum_lstm_cuda(Tensor states_4d, Tensor z4_4d, Tensor prev_cell_d, Tensor? w_cell, "
+        "Tensor? b_cell, Tensor? w_state, Tensor? b_state, float alpha, float eps_cell, "
+        "float eps_state, bool use_fast_gelu) -> (Tensor, Tensor)",
+}
+
+_SRC_DTYPES = {
+    torch.float32: _native.DTYPE_F32,
+    torch.float16: _native.DTYPE_F16,
+    torch.bfloat16: _native.DTYPE_BF16,
+}
+_HALF_DTYPES = {torch.float16: _native.DTYPE_F16, torch.bfloat16: _native.DTYPE_BF16}
+
+_torch_lib: Optional[torch.library.Library] = None
+_registered = False
+
+
+def _check(cond: bool, msg: str) -> None:
+    # TORCH_CHECK raises c10::Error, which Python sees as RuntimeError.
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _lib() -> ctypes.CDLL:
+    if not _native.is_loaded():
+        raise RuntimeError(
+            "arctic_inference custom ops are not loaded: call try_load_torch_library() "
+            "and check that it returned True (libarctic_mi355x.so must be built)")
+    return _native.load()
+
+
+def _stream_of(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _on_device_of:
+    """OptionalCUDAGuard: make the tensor's device current for the launch."""
+
+    def __init__(self, t: torch.Tensor):
+        self.idx = t.device.index
+        self.prev = None
+
+    def __enter__(self):
+        cur = torch.cuda.current_device()
+        if self.idx is not None and self.idx != cur:
+            self.prev = cur
+            torch.cuda.set_device(self.idx)
+
+    def __exit__(self, *exc):
+        if self.prev is not None:
+            torch.cuda.set_device(self.prev)
+        return False
+
+
+# --------------------------------------------------------------------------- #
+# operator implementations (CUDA dispatch key)
+# --------------------------------------------------------------------------- #
+def _kv_dtype_code(src_dtype: torch.dtype, kv_cache_dtype: str) -> Tuple[int, int]:
+    # DISPATCH_BY_KV_CACHE_DTYPE, csrc/custom_ops/quant_utils.cuh:532-567
+    if kv_cache_dtype == "auto":
+        kv = _native.KV_AUTO
+    elif kv_cache_dtype in ("fp8", "fp8_e4m3"):
+        kv = _native.KV_FP8_E4M3
+    elif kv_cache_dtype == "fp8_e5m2":
+        kv = _native.KV_FP8_E5M2
+    else:
+        raise RuntimeError(f"Unsupported data type of kv cache: {kv_cache_dtype}")
+    if src_dtype not in _SRC_DTYPES:
+        raise RuntimeError(f"Unsupported input type of kv cache: {src_dtype}")
+    return _SRC_DTYPES[src_dtype], kv
+
+
+def _ptr_table(tensors: List[torch.Tensor]):
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+def _reshape_and_cache_flash_bulk_impl(
+    keys: torch.Tensor,
+    values: torch.Tensor,
+    key_caches: List[torch.Tensor],
+    value_caches: List[torch.Tensor],
+    slot_mapping: torch.Tensor,
+    kv_cache_dtype: str,
+    k_scales: List[torch.Tensor],
+    v_scales: List[torch.Tensor],
+    num_heads: int,
+    head_size: int,
+) -> None:
+    """Host side of the bulk KV write; follows the reference's launcher
+    (csrc/custom_ops/reshape_and_cache_flash_bulk.cu:77-144) up to the point
+    where it would copy four pointer tables to the device: here the tables ride
+    in the kernel arguments instead."""
+    lib = _lib()
+    num_layers = len(key_caches)
+    if num_layers == 0:
+        return
+    _check(num_layers == len(value_caches), "Expected num_layers == value_caches.size() to be true")
+    _check(num_layers == len(k_scales), "Expected num_layers == k_scales.size() to be true")
+    _check(num_layers == len(v_scales), "Expected num_layers == v_scales.size() to be true")
+    src_code, kv_code = _kv_dtype_code(keys.dtype, kv_cache_dtype)
+
+    num_tokens = slot_mapping.size(0)
+    block_size = key_caches[0].size(1)
+    key_stride = keys.stride(0)
+    value_stride = values.stride(0)
+    block_stride = key_caches[0].stride(0)
+    _check(block_stride == value_caches[0].stride(0),
+           "Expected block_stride == value_caches[0].stride(0) to be true")
+    _check(slot_mapping.dtype == torch.int64,
+           f"expected scalar type Long but found {slot_mapping.dtype}")
+    # Not checked by the reference (it reinterprets the pointers); a mismatch
+    # there corrupts memory, here it is an error.
+    _check(values.dtype == keys.dtype, "reshape_and_cache_flash_bulk: keys and values dtype differ")
+    _check(keys.stride(-1) == 1 and values.stride(-1) == 1,
+           "reshape_and_cache_flash_bulk: last dimension of keys/values must be contiguous")
+    _check(slot_mapping.dim() == 1 and (num_tokens <= 1 or slot_mapping.stride(0) == 1),
+           "reshape_and_cache_flash_bulk: slot_mapping must be 1-D and contiguous")
+    cache_elem = key_caches[0].element_size()
+    want_elem = keys.element_size() if kv_code == _native.KV_AUTO else 1
+    _check(cache_elem == want_elem and value_caches[0].element_size() == want_elem,
+           f"reshape_and_cache_flash_bulk: cache element size {cache_elem} does not match "
+           f"kv_cache_dtype '{kv_cache_dtype}' (expected {want_elem})")
+    if kv_code != _native.KV_AUTO:
+        _check(all(s.dtype == torch.float32 for s in k_scales) and
+               all(s.dtype == torch.float32 for s in v_scales),
+               "reshape_and_cache_flash_bulk: k_scales / v_scales must be float32")
+    dev = keys.device
+    _check(all(t.device == dev for t in (values, slot_mapping, *key_caches, *value_caches)),
+           "reshape_and_cache_flash_bulk: all tensors must be on the same device")
+
+    with _on_device_of(keys):
+        rc = lib.arctic_reshape_and_cache_flash_bulk(
+            keys.data_ptr(), values.data_ptr(), key_stride, value_stride,
+            _ptr_table(key_caches), _ptr_table(value_caches),
+            _ptr_table(k_scales), _ptr_table(v_scales),
+            slot_mapping.data_ptr(), num_tokens, num_layers, int(num_heads), int(head_size),
+            int(block_size), int(block_stride), src_code, kv_code, _stream_of(keys))
+    _native.check(rc)
+
+
+def _reshape_and_cache_flash_fp4_impl(*args, **kwargs) -> None:
+    raise NotImplementedError(
+        "arctic_inference::reshape_and_cache_flash_fp4 is not part of this library "
+        "(only the bulk KV write and the speculator ops are)")
+
+
+def _speculator_ln_impl(input: torch.Tensor, weight: Optional[torch.Tensor],
+                        bias: Optional[torch.Tensor], eps: float) -> torch.Tensor:
+    """Host side of speculator_ln_cuda (csrc/custom_ops/speculator_ln.cu:152-252)."""
+    lib = _lib()
+    _check(input.dtype in _HALF_DTYPES, "speculator_ln: only fp16 and bf16 are supported.")
+    _check(input.is_cuda, "speculator_ln: input must be CUDA")
+    dtype = input.dtype
+    hidden = input.size(-1)
+    _check(hidden > 0, "speculator_ln: hidden size must be > 0")
+    _check(input.stride(-1) == 1,
+           "speculator_ln: last dimension must be contiguous (stride -1 == 1)")
+    if weight is not None:
+        _check(weight.is_cuda, "weight must be CUDA")
+        _check(weight.dtype == dtype, "weight dtype must match input dtype")
+        _check(weight.dim() == 1 and weight.numel() == hidden, "weight must be 1D of size hidden")
+        _check(weight.is_contiguous(), "weight must be contiguous")
+    if bias is not None:
+        _check(bias.is_cuda, "bias must be CUDA")
+        _check(bias.dtype == dtype, "bias dtype must match input dtype")
+        _check(bias.dim() == 1 and bias.numel() == hidden, "bias must be 1D of size hidden")
+        _check(bias.is_contiguous(), "bias must be contiguous")
+
+    in_2d = input.view(-1, hidden)
+    rows = in_2d.size(0)
+    row_stride = in_2d.stride(0)
+    out = torch.empty_like(input)
+    out_2d = out.view(-1, hidden)  # rows are written dense, `hidden` apart
+    if rows == 0:
+        return out
+    _check(out_2d.stride(0) == hidden or rows == 1, "speculator_ln: internal - output rows must be dense")
+    with _on_device_of(input):
+        rc = lib.arctic_speculator_ln(
+            out_2d.data_ptr(), in_2d.data_ptr(),
+            weight.data_ptr() if weight is not None else None,
+            bias.data_ptr() if bias is not None else None,
+            rows, hidden, row_stride, float(eps), _HALF_DTYPES[dtype], _stream_of(input))
+    _native.check(rc)
+    return out
+
+
+def _sum_lstm_impl(
+    states_4d: torch.Tensor,
+    z4_4d: torch.Tensor,
+    prev_cell_d: torch.Tensor,
+    w_cell: Optional[torch.Tensor],
+    b_cell: Optional[torch.Tensor],
+    w_state: Optional[torch.Tensor],
+    b_state: Optional[torch.Tensor],
+    alpha: float,
+    eps_cell: float,
+    eps_state: float,
+    use_fast_gelu: bool,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Host side of sum_lstm_cuda (csrc/custom_ops/sum_lstm.cu:293-473)."""
+    lib = _lib()
+    dtype = states_4d.dtype
+    _check(dtype in _HALF_DTYPES, "sum_lstm: only fp16 and bf16 are supported.")
+    _check(states_4d.is_cuda and z4_4d.is_cuda and prev_cell_d.is_cuda,
+           "sum_lstm: inputs must be CUDA tensors")
+    _check(z4_4d.dtype == dtype and prev_cell_d.dtype == dtype,
+           "sum_lstm: all input dtypes must match")
+    hidden4 = states_4d.size(-1)
+    _check(hidden4 > 0 and hidden4 % 4 == 0, "sum_lstm: last dim of states must be 4*D_gate")
+    d_gate = hidden4 // 4
+    _check(z4_4d.size(-1) == hidden4, "sum_lstm: z4 must have last dim 4*D_gate")
+    d_cell = prev_cell_d.size(-1)
+    _check(d_cell == d_gate,
+           f"sum_lstm: prev_cell last dim must equal D_gate. Got {d_cell} vs expected {d_gate}.")
+    _check(states_4d.stride(-1) == 1 and z4_4d.stride(-1) == 1 and prev_cell_d.stride(-1) == 1,
+           "sum_lstm: last dimension must be contiguous (stride -1 == 1)")
+    for t, name in ((w_cell, "w_cell"), (b_cell, "b_cell"), (w_state, "w_state"), (b_state, "b_state")):
+        if t is not None:
+            _check(t.is_cuda, f"sum_lstm: {name} must be CUDA")
+            _check(t.dtype == dtype, f"sum_lstm: {name} dtype mismatch")
+            _check(t.numel() >= d_gate, f"sum_lstm: {name} must have length >= D_eff")
+            _check(t.is_contiguous(), f"sum_lstm: {name} must be contiguous")
+
+    s2 = states_4d.view(-1, hidden4)
+    z2 = z4_4d.view(-1, hidden4)
+    p2 = prev_cell_d.view(-1, d_cell)
+    rows = s2.size(0)
+    _check(z2.size(0) == rows and p2.size(0) == rows, "sum_lstm: row counts of the inputs differ")
+    # outputs inherit prev_cell's row pitch (reference :356-365)
+    out_cell = torch.empty_strided(p2.size(), p2.stride(), dtype=dtype, device=p2.device)
+    out_state = torch.empty_strided(p2.size(), p2.stride(), dtype=dtype, device=p2.device)
+    _check(out_cell.stride(0) == out_state.stride(0), "sum_lstm: internal - output strides mismatch")
+    out_cell_orig = out_cell.view(prev_cell_d.size())
+    out_state_orig = out_state.view(prev_cell_d.size())
+    if rows == 0:
+        return out_state_orig, out_cell_orig
+
+    def ptr(t):
+        return t.data_ptr() if t is not None else None
+
+    with _on_device_of(states_4d):
+        rc = lib.arctic_sum_lstm(
+            out_state.data_ptr(), out_cell.data_ptr(), s2.data_ptr(), z2.data_ptr(), p2.data_ptr(),
+            ptr(w_cell), ptr(b_cell), ptr(w_state), ptr(b_state),
+            rows, d_gate, s2.stride(0), z2.stride(0), p2.stride(0), out_cell.stride(0),
+            float(alpha), float(eps_cell), float(eps_state), int(bool(use_fast_gelu)),
+            _HALF_DTYPES[dtype], _stream_of(states_4d))
+    _native.check(rc)
+    return out_state_orig, out_cell_orig
+
+
+_IMPLS = {
+    "reshape_and_cache_flash_bulk": _reshape_and_cache_flash_bulk_impl,
+    "reshape_and_cache_flash_fp4": _reshape_and_cache_flash_fp4_impl,
+    "speculator_ln_cuda": _speculator_ln_impl,
+    "sum_lstm_cuda": _sum_lstm_impl,
+}
+
+
+def _register_ops() -> None:
+    """Define the four schemas and bind the CUDA key (the only key the reference
+    binds, torch_bindings.cpp:17,32,37,50)."""
+    global _torch_lib, _registered
+    if _registered:
+        return
+    lib = torch.library.Library(_NAMESPACE, "DEF")
+    for name, schema in _SCHEMAS.items():
+        lib.define(schema)
+        lib.impl(name, _IMPLS[name], "CUDA")
+    _torch_lib = lib  # keep alive: dropping the Library object unregisters the ops
+    _registered = True
+
+
+# --------------------------------------------------------------------------- #
+# public surface (names and meaning as in arctic_inference/py_custom_ops.py)
+# --------------------------------------------------------------------------- #
+def try_load_torch_library() -> bool:
+    """Load ``libarctic_mi355x*.so`` from the package directory and register the
+    ``torch.ops.arctic_inference`` operators.  True iff the operators are usable
+    (reference: arctic_inference/py_custom_ops.py:9-37)."""
+    path = _native.library_path()
+    if path is None:
+        logger.info("Could not find compiled %s library in package.", _native.LIB_BASENAME)
+        return False
+    try:
+        _native.load()
+        _register_ops()
+        logger.info("Successfully loaded custom ops from %s.", path)
+        return True
+    except Exception as e:  # missing ROCm runtime, ABI mismatch, duplicate registration ...
+        logger.info("Unable to load custom library from %s. %s: %s.", path, type(e).__name__, e)
+        return False
+
+
+def try_load_jit_library() -> bool:
+    """Build the library with hipcc on the spot, then load it.  Counterpart of the
+    reference's JIT route (arctic_inference/py_custom_ops.py:40-56)."""
+    try:
+        _native.build(force=False)
+    except Exception as e:
+        logger.info("Unable to build %s. %s: %s.", _native.LIB_BASENAME, type(e).__name__, e)
+        return False
+    return try_load_torch_library()
+
+
+def _ops():
+    if not _registered:
+        raise RuntimeError(
+            "arctic_inference custom ops are not loaded: call try_load_torch_library() "
+            "and check that it returned True (libarctic_mi355x.so must be built)")
+    return torch.ops.arctic_inference
+
+
+def reshape_and_cache_flash_bulk(
+    keys: torch.Tensor,
+    values: torch.Tensor,
+    key_caches: List[torch.Tensor],
+    value_caches: List[torch.Tensor],
+    slot_mapping: torch.Tensor,
+    kv_cache_dtype: str,
+    k_scales: List[torch.Tensor],
+    v_scales: List[torch.Tensor],
+    num_heads: int,
+    head_size: int,
+) -> None:
+    _ops().reshape_and_cache_flash_bulk(keys, values, key_caches, value_caches, slot_mapping,
+                                        kv_cache_dtype, k_scales, v_scales, num_heads, head_size)
+
+
+def reshape_and_cache_flash_fp4(
+    keys: torch.Tensor,
+    values: torch.Tensor,
+    key_cache: torch.Tensor,
+    value_cache: torch.Tensor,
+    key_cache_scales: torch.Tensor,
+    value_cache_scales: torch.Tensor,
+    slot_mapping: torch.Tensor,
+    kv_cache_dtype: str,
+    k_scale: torch.Tensor,
+    v_scale: torch.Tensor,
+) -> None:
+    _ops().reshape_and_cache_flash_fp4(keys, values, key_cache, value_cache, slot_mapping,
+                                       kv_cache_dtype, k_scale, v_scale, key_cache_scales,
+                                       value_cache_scales)
+
+
+def speculator_ln(
+    input: torch.Tensor,
+    weight: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor],
+    eps: float,
+) -> torch.Tensor:
+    return _ops().speculator_ln_cuda(input, weight, bias, eps)
+
+
+def sum_lstm(
+    states_4d: torch.Tensor,
+    z4_4d: torch.Tensor,
+    prev_cell_d: torch.Tensor,
+    w_cell: Optional[torch.Tensor],
+    b_cell: Optional[torch.Tensor],
+    w_state: Optional[torch.Tensor],
+    b_state: Optional[torch.Tensor],
+    alpha: float,
+    eps_cell: float,
+    eps_state: float,
+    use_fast_gelu: bool,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    return _ops().sum_lstm_cuda(states_4d, z4_4d, prev_cell_d, w_cell, b_cell, w_state, b_state,
+                                alpha, eps_cell, eps_state, use_fast_gelu)

@@ -1,0 +1,148 @@
+/*
+ * arctic_mi355x.h - C ABI of libarctic_mi355x.so
+ *
+ * MI355X (gfx950) replacement for the native half of ArcticInference's
+ * csrc/custom_ops library: the SwiftKV bulk KV-cache write and the Arctic
+ * speculator's fused element-wise operators.  Plain pointers and sizes only; no
+ * torch, ATen or pybind types cross this boundary.  Every pointer named "device"
+ * is an address in the current HIP device's memory; `stream` is a hipStream_t
+ * passed as void* (NULL = the default stream).
+ *
+ * All entry points are asynchronous with respect to the host: they enqueue work
+ * on `stream` and return.  They never allocate, free or synchronise, so they can
+ * be recorded into a HIP graph.  They return 0 on success and a non-zero
+ * ARCTIC_ERR_* code on failure; arctic_last_error() then holds a message for the
+ * calling thread.  The library keeps no reference to any argument after return.
+ *
+ * Reference paths below are relative to the ArcticInference source tree.
+ */
+#ifndef ARCTIC_MI355X_H
+#define ARCTIC_MI355X_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ARCTIC_ABI_VERSION 1
+
+/* element types of source / activation tensors */
+#define ARCTIC_DTYPE_F32 0
+#define ARCTIC_DTYPE_F16 1
+#define ARCTIC_DTYPE_BF16 2
+
+/* KV-cache storage types: the reference's Fp8KVCacheDataType
+ * (csrc/custom_ops/dtype_fp8.cuh:14-18) selected from the strings
+ * "auto" | "fp8" / "fp8_e4m3" | "fp8_e5m2" (csrc/custom_ops/quant_utils.cuh:532-567). */
+#define ARCTIC_KV_AUTO 0
+#define ARCTIC_KV_FP8_E4M3 1
+#define ARCTIC_KV_FP8_E5M2 2
+
+#define ARCTIC_OK 0
+#define ARCTIC_ERR_INVALID_ARGUMENT 1
+#define ARCTIC_ERR_UNSUPPORTED 2
+#define ARCTIC_ERR_LAUNCH 3
+
+/* Largest num_layers one call accepts. */
+#define ARCTIC_MAX_LAYERS 512
+
+int arctic_abi_version(void);
+
+/* Message of the last failure on the calling thread ("" if none). The pointer
+ * stays valid until the next failing call on the same thread. */
+const char *arctic_last_error(void);
+
+/*
+ * Bulk KV-cache write.  Replaces the host launcher + kernel
+ *   reshape_and_cache_flash_bulk()            csrc/custom_ops/reshape_and_cache_flash_bulk.cu:77-144
+ *   reshape_and_cache_flash_bulk_kernel<>     csrc/custom_ops/reshape_and_cache_flash_bulk.cu:12-60
+ *   fp8::scaled_convert<>                     csrc/custom_ops/quant_utils.cuh:456-489,515-526
+ * (declared in csrc/custom_ops/custom_ops.h:9-17, bound at torch_bindings.cpp:7-18).
+ *
+ * For every layer l < num_layers and token t < num_tokens with
+ * slot = slot_mapping[t] >= 0 (negative slots are padding and are skipped):
+ *   dst = cache_l + (slot / block_size) * block_stride + (slot % block_size) * n
+ *   dst[i] = cvt(src[t * stride + l * n + i])   for i < n = num_heads * head_size
+ * for both (keys, key_cache_ptrs, k_scale_ptrs) and (values, value_cache_ptrs,
+ * v_scale_ptrs).  cvt is a raw copy for ARCTIC_KV_AUTO (cache element type ==
+ * src_dtype) and fp8(float(x) / *scale_l) otherwise: IEEE fp32 division, round to
+ * nearest even into OCP e4m3fn / e5m2, saturating to the largest finite value.
+ *
+ *   keys, values        device; [num_tokens, >= num_layers*n], row strides
+ *                       key_stride / value_stride in ELEMENTS, inner dim dense
+ *   key_cache_ptrs ...  HOST arrays of num_layers DEVICE pointers (the reference
+ *                       builds the same four tables on its host stack, :104-118);
+ *                       they are copied into the kernel arguments, so nothing is
+ *                       uploaded separately and they may be freed on return.
+ *                       Scale pointers address one fp32 each; they are read on the
+ *                       device at execution time.  May be NULL for ARCTIC_KV_AUTO.
+ *   slot_mapping        device int64[num_tokens]
+ *   block_stride        ELEMENTS between consecutive cache blocks (same for K and
+ *                       V); inside a block the layout is [block_size][n] dense
+ * Distinct valid slots are required for a deterministic result (as in the
+ * reference).  num_layers == 0 or num_tokens == 0 is a successful no-op.
+ */
+int arctic_reshape_and_cache_flash_bulk(
+    const void *keys, const void *values, int64_t key_stride,
+    int64_t value_stride, const void *const *key_cache_ptrs,
+    const void *const *value_cache_ptrs, const float *const *k_scale_ptrs,
+    const float *const *v_scale_ptrs, const int64_t *slot_mapping,
+    int64_t num_tokens, int num_layers, int num_heads, int head_size,
+    int block_size, int64_t block_stride, int src_dtype, int kv_cache_dtype,
+    void *stream);
+
+/*
+ * Speculator "LayerNorm" (an RMS norm with optional scale and shift).  Replaces
+ *   speculator_ln_cuda()                      csrc/custom_ops/speculator_ln.cu:152-252
+ *   spec_ln_vec_kernel<> / spec_ln_scalar_kernel<>   csrc/custom_ops/speculator_ln.cu:21-150
+ * (custom_ops.h:29-32, torch_bindings.cpp:33-37).
+ *
+ *   y = x * rsqrt(mean(x^2) + eps);  if (weight) y *= weight;  if (bias) y += bias
+ * in fp32, rounded to nearest even into `dtype` (F16 or BF16).
+ *
+ *   in       device; rows of `hidden` elements, in_row_stride ELEMENTS apart
+ *   out      device; rows * hidden elements, dense
+ *   weight, bias   device [hidden] or NULL
+ */
+int arctic_speculator_ln(void *out, const void *in, const void *weight,
+                         const void *bias, int64_t rows, int hidden,
+                         int64_t in_row_stride, float eps, int dtype,
+                         void *stream);
+
+/*
+ * Fused LSTM-style gate / cell / state update.  Replaces
+ *   sum_lstm_cuda()                           csrc/custom_ops/sum_lstm.cu:293-473
+ *   sum_lstm_vec_kernel<> / sum_lstm_scalar_kernel<>   csrc/custom_ops/sum_lstm.cu:28-291
+ * (custom_ops.h:34-41, torch_bindings.cpp:39-50).
+ *
+ * Per row, with gate order f | i | o | c along the 4*D dimension:
+ *   pre_g    = states_g + alpha * z4_g
+ *   c_new    = prev_cell * sigmoid(pre_f)
+ *              + gelu(rmsnorm(pre_c; w_cell, b_cell, eps_cell)) * sigmoid(pre_i)
+ *   out_cell = round(c_new)
+ *   out_state = round(gelu(rmsnorm(out_cell; w_state, b_state, eps_state)) * sigmoid(pre_o))
+ * where rmsnorm(v; w, b, eps) = v * rsqrt(mean(v^2) + eps) [* w] [+ b]; the mean
+ * for the state norm is taken over the unrounded c_new while the normalised
+ * values are the rounded out_cell, as in the reference (:136-137,:163,:174).
+ * gelu is the exact erf form, or the tanh form when fast_gelu != 0.
+ *
+ *   states, z4     device; rows of 4*D elements, s_stride / z_stride apart
+ *   prev_cell      device; rows of D elements, pc_stride apart
+ *   out_state, out_cell   device; rows of D elements, out_stride apart
+ *   w_cell, b_cell, w_state, b_state   device [>= D] or NULL
+ * All strides are in ELEMENTS.  dtype is F16 or BF16.
+ */
+int arctic_sum_lstm(void *out_state, void *out_cell, const void *states,
+                    const void *z4, const void *prev_cell, const void *w_cell,
+                    const void *b_cell, const void *w_state,
+                    const void *b_state, int64_t rows, int D, int64_t s_stride,
+                    int64_t z_stride, int64_t pc_stride, int64_t out_stride,
+                    float alpha, float eps_cell, float eps_state, int fast_gelu,
+                    int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* ARCTIC_MI355X_H */

@@ -1,0 +1,228 @@
+"""GPU parity of the bulk KV-cache write against the CPU oracle: bit-exact.
+
+Every call goes torch.ops.arctic_inference.reshape_and_cache_flash_bulk ->
+Python shim -> C ABI of libarctic_mi355x.so.
+"""
+import pytest
+import torch
+
+import oracle
+from helpers import (assert_bulk_equal, bulk_args, bulk_case_to, bytes_of, make_bulk_case)
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def run_both(ops, case):
+    dcase = bulk_case_to(case, DEV)
+    ops.reshape_and_cache_flash_bulk(*bulk_args(dcase))
+    torch.cuda.synchronize()
+    oracle.reshape_and_cache_flash_bulk(*bulk_args(case))
+    assert_bulk_equal(dcase["bufs"], case["bufs"])
+    return dcase
+
+
+def test_config1_bf16_passthrough(ops):
+    # BASELINE config 1: 256 tokens, 16 layers, 8 KV heads x 128, block 16, 512 blocks, bf16 cache
+    case = make_bulk_case(T=256, L=16, H=8, D=128, bs=16, NB=512, seed=0)
+    run_both(ops, case)
+
+
+@pytest.mark.parametrize("src_dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("kv", ["auto", "fp8", "fp8_e4m3", "fp8_e5m2"])
+@pytest.mark.parametrize("shape", [
+    dict(T=33, L=4, H=8, D=128, bs=16, NB=8),     # production row width
+    dict(T=2, L=4, H=2, D=16, bs=16, NB=2),        # the reference unit test's sizes
+    dict(T=17, L=3, H=1, D=128, bs=16, NB=4),      # TP-sharded single head
+    dict(T=9, L=5, H=3, D=80, bs=8, NB=6),         # row chunk count not a power of two
+    dict(T=5, L=2, H=1, D=20, bs=4, NB=3),         # not 16-byte divisible: element-wise kernel
+    dict(T=7, L=70, H=2, D=64, bs=16, NB=2),       # more layers than one launch carries
+])
+def test_small_shapes(ops, src_dtype, kv, shape):
+    case = make_bulk_case(src_dtype=src_dtype, kv_cache_dtype=kv, seed=11, std=1.5, pad_fraction=0.2, **shape)
+    run_both(ops, case)
+
+
+@pytest.mark.parametrize("kv", ["auto", "fp8"])
+def test_flashinfer_layout_and_row_pitch(ops, kv):
+    # K = cache[:, 0], V = cache[:, 1] (block stride 2*bs*n) and keys with a padded row pitch
+    case = make_bulk_case(T=40, L=4, H=4, D=64, bs=16, NB=8, kv_cache_dtype=kv, seed=5, layout="flashinfer",
+                          key_pad=24, pad_fraction=0.1)
+    assert case["keys"].stride(0) != case["keys"].size(1)
+    run_both(ops, case)
+
+
+def test_all_padding_leaves_cache_untouched(ops):
+    case = make_bulk_case(T=16, L=3, H=2, D=64, bs=16, NB=4, kv_cache_dtype="fp8", seed=7)
+    case["slot_mapping"].fill_(-1)
+    before = [b.clone() for b in case["bufs"]]
+    dcase = bulk_case_to(case, DEV)
+    ops.reshape_and_cache_flash_bulk(*bulk_args(dcase))
+    torch.cuda.synchronize()
+    assert_bulk_equal(dcase["bufs"], before)
+
+
+def test_empty_inputs(ops):
+    case = make_bulk_case(T=4, L=2, H=2, D=64, bs=16, NB=2, seed=1)
+    dcase = bulk_case_to(case, DEV)
+    # no layers: no-op (reference returns early)
+    ops.reshape_and_cache_flash_bulk(dcase["keys"], dcase["values"], [], [], dcase["slot_mapping"], "auto", [], [],
+                                     2, 64)
+    # no tokens
+    ops.reshape_and_cache_flash_bulk(dcase["keys"][:0], dcase["values"][:0], dcase["key_caches"],
+                                     dcase["value_caches"], dcase["slot_mapping"][:0], "auto", dcase["k_scales"],
+                                     dcase["v_scales"], 2, 64)
+    torch.cuda.synchronize()
+    assert_bulk_equal(dcase["bufs"], case["bufs"])
+
+
+def _exhaustive_case(src_dtype, kv, scales):
+    """Every 16-bit pattern appears once per layer: 64 tokens x 1024 elements."""
+    L = len(scales)
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(src_dtype).view(64, 1024)
+    case = make_bulk_case(T=64, L=L, H=8, D=128, bs=16, NB=4, src_dtype=src_dtype, kv_cache_dtype=kv, seed=3)
+    case["keys"] = bits.repeat(1, L).contiguous()
+    case["values"] = bits.flip(0).repeat(1, L).contiguous()
+    case["k_scales"] = [torch.tensor(s, dtype=torch.float32) for s in scales]
+    case["v_scales"] = [torch.tensor(s, dtype=torch.float32) for s in reversed(scales)]
+    return case
+
+
+SCALES = [1.0, 0.013392857, 0.1, 2.0 ** -7, 3.7, 1e-3, 447.9, 0.33333334, 5.9e-8 * 1e-31, 3.0e38]
+
+
+@pytest.mark.parametrize("src_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("kv", ["fp8", "fp8_e5m2"])
+def test_fp8_codes_exhaustive_16bit(ops, src_dtype, kv):
+    """All 65 536 source bit patterns (incl. +-0, subnormals, +-inf, NaN) x 10 scales,
+    among them a subnormal and a near-overflow scale."""
+    case = _exhaustive_case(src_dtype, kv, SCALES)
+    run_both(ops, case)
+
+
+@pytest.mark.parametrize("scale", [0.0, float("inf"), -0.5, float("nan")])
+def test_fp8_degenerate_scales(ops, scale):
+    """x/0, x/inf, negative and NaN scales follow IEEE division. NaN codes are compared
+    without their sign bit: the sign of a NaN produced by 0/0 is not defined by IEEE
+    (x86 gives -NaN, the GPU +NaN), and the reference does not pin it either."""
+    case = _exhaustive_case(torch.bfloat16, "fp8", [scale])
+    dcase = bulk_case_to(case, DEV)
+    ops.reshape_and_cache_flash_bulk(*bulk_args(dcase))
+    torch.cuda.synchronize()
+    oracle.reshape_and_cache_flash_bulk(*bulk_args(case))
+    for g, w in zip(dcase["bufs"], case["bufs"]):
+        gb, wb = bytes_of(g.cpu()), bytes_of(w)
+        nan = (wb & 0x7F) == 0x7F
+        assert torch.equal(gb[~nan], wb[~nan])
+        assert torch.equal(gb[nan] & 0x7F, wb[nan] & 0x7F)
+
+
+def test_fp8_from_fp32_rounding_boundaries(ops):
+    """fp32 sources placed on and next to every e4m3 rounding boundary, scale 1 and a
+    non-trivial scale chosen so that quotients land near boundaries too."""
+    codes = torch.arange(0, 0x7F, dtype=torch.int64)
+    vals = oracle.e4m3fn_decode(codes)                       # all finite non-negative values
+    mids = (vals[:-1] + vals[1:]) / 2                        # exact in fp32
+    pts = torch.cat([vals, mids, torch.tensor([448.0, 464.0, 480.0, 2.0 ** -10, 2.0 ** -11])])
+    ulp = torch.tensor([-2, -1, 0, 1, 2], dtype=torch.int32)
+    grid = (pts.view(torch.int32)[:, None] + ulp[None, :]).view(torch.float32).reshape(-1)
+    grid = torch.cat([grid, -grid])
+    n = 1024
+    T = (grid.numel() + n - 1) // n
+    flat = torch.zeros(T * n)
+    flat[: grid.numel()] = grid
+    scales = [1.0, 3.0, 0.7]
+    case = make_bulk_case(T=T, L=len(scales), H=8, D=128, bs=16, NB=2, src_dtype=torch.float32,
+                          kv_cache_dtype="fp8", seed=9)
+    keys = torch.cat([flat.view(T, n) * s for s in scales], dim=1).contiguous()   # quotient ~ boundary
+    case["keys"] = keys
+    case["values"] = keys.flip(0).contiguous()
+    case["k_scales"] = [torch.tensor(s, dtype=torch.float32) for s in scales]
+    case["v_scales"] = [torch.tensor(s, dtype=torch.float32) for s in scales]
+    run_both(ops, case)
+
+
+def test_config2_fp8_prefill_chunk(ops):
+    # BASELINE config 2: 8192 tokens, 16 layers, fp8 cache with amax/448 scales
+    case = make_bulk_case(T=8192, L=16, H=8, D=128, bs=16, NB=8192, kv_cache_dtype="fp8", seed=1, std=1.5)
+    run_both(ops, case)
+
+
+def test_config3_shape_properties(ops):
+    """BASELINE config 3 at full size (16384 tokens, 40 layers, 10 % padding): too large
+    for the CPU oracle in seconds, so it is checked through size-independent properties:
+    rows of padded tokens and unaddressed slots keep their sentinel, a random sample of
+    tokens matches the oracle bit for bit, and the write is idempotent."""
+    T, L, H, D, bs, NB = 16384, 40, 8, 128, 16, 8192
+    n = H * D
+    dev = torch.device(DEV)
+    g = torch.Generator().manual_seed(2)
+    gd = torch.Generator(device=dev).manual_seed(2)
+    # generated on the GPU (1.3 GB per tensor); the sampled rows are copied back for the oracle
+    dkeys = torch.empty(T, L * n, dtype=torch.bfloat16, device=dev)
+    dvalues = torch.empty(T, L * n, dtype=torch.bfloat16, device=dev)
+    for t0 in range(0, T, 2048):
+        dkeys[t0:t0 + 2048] = (torch.randn(2048, L * n, generator=gd, device=dev) * 1.5).to(torch.bfloat16)
+        dvalues[t0:t0 + 2048] = (torch.randn(2048, L * n, generator=gd, device=dev) * 1.5).to(torch.bfloat16)
+    from helpers import make_slots
+    slots = make_slots(T, NB * bs, g, pad_fraction=0.1)
+    assert int((slots < 0).sum()) == 1638
+    dks = [(dkeys[:, l * n:(l + 1) * n].float().abs().max() / 448.0) for l in range(L)]
+    dvs = [(dvalues[:, l * n:(l + 1) * n].float().abs().max() / 448.0) for l in range(L)]
+    k_scales, v_scales = [s.cpu() for s in dks], [s.cpu() for s in dvs]
+    dslots = slots.to(dev)
+    sentinel = 0xA5
+    bufs = [torch.full((2, NB, bs, H, D), sentinel, dtype=torch.uint8, device=dev) for _ in range(L)]
+    kc, vc = [b[0] for b in bufs], [b[1] for b in bufs]
+    ops.reshape_and_cache_flash_bulk(dkeys, dvalues, kc, vc, dslots, "fp8", dks, dvs, H, D)
+    torch.cuda.synchronize()
+
+    valid = slots >= 0
+    written = torch.zeros(NB * bs, dtype=torch.bool)
+    written[slots[valid]] = True
+    # (1) untouched rows: every row not addressed by a valid slot is still all-sentinel
+    for l in (0, 17, 39):
+        for c in (kc[l], vc[l]):
+            rows = c.view(NB * bs, n)
+            untouched = rows[(~written).to(dev)]
+            assert bool((untouched == sentinel).all())
+    # (2) sampled tokens against the oracle
+    sample = torch.randperm(T, generator=g)[:96]
+    sub_slots = slots[sample]
+    remap = torch.full_like(sub_slots, -1)
+    nvalid = int((sub_slots >= 0).sum())
+    remap[sub_slots >= 0] = torch.arange(nvalid)
+    obufs = [torch.zeros(2, (nvalid + bs - 1) // bs, bs, H, D, dtype=torch.uint8) for _ in range(L)]
+    dsample = sample.to(dev)
+    oracle.reshape_and_cache_flash_bulk(dkeys[dsample].cpu().contiguous(), dvalues[dsample].cpu().contiguous(),
+                                        [b[0] for b in obufs], [b[1] for b in obufs], remap, "fp8",
+                                        k_scales, v_scales, H, D)
+    src_rows = sub_slots[sub_slots >= 0].to(dev)
+    for l in range(L):
+        for which in (0, 1):
+            got = bufs[l][which].view(NB * bs, n)[src_rows].cpu()
+            want = obufs[l][which].view(-1, n)[:nvalid]
+            assert torch.equal(got, want), f"layer {l} {'KV'[which]} sample mismatch"
+    # (3) idempotence: a second identical write changes nothing
+    sums = [int(b.view(-1).to(torch.int64).sum()) for b in bufs[:4]]
+    ops.reshape_and_cache_flash_bulk(dkeys, dvalues, kc, vc, dslots, "fp8", dks, dvs, H, D)
+    torch.cuda.synchronize()
+    assert sums == [int(b.view(-1).to(torch.int64).sum()) for b in bufs[:4]]
+
+
+def test_errors(ops):
+    case = make_bulk_case(T=4, L=2, H=2, D=64, bs=16, NB=2, seed=1)
+    d = bulk_case_to(case, DEV)
+    a = list(bulk_args(d))
+    with pytest.raises(RuntimeError, match="Unsupported data type of kv cache"):
+        ops.reshape_and_cache_flash_bulk(*a[:5], "int4", *a[6:])
+    with pytest.raises(RuntimeError, match="Unsupported input type of kv cache"):
+        ops.reshape_and_cache_flash_bulk(a[0].to(torch.float64), a[1].to(torch.float64), *a[2:])
+    with pytest.raises(RuntimeError):
+        ops.reshape_and_cache_flash_bulk(*a[:3], a[3][:1], *a[4:])          # list length mismatch
+    with pytest.raises(RuntimeError, match="Long"):
+        ops.reshape_and_cache_flash_bulk(*a[:4], a[4].to(torch.int32), *a[5:])
+    with pytest.raises(RuntimeError, match="element size"):
+        ops.reshape_and_cache_flash_bulk(*a[:5], "fp8", *a[6:])            # bf16 cache passed as fp8
+    torch.cuda.synchronize()
+    assert_bulk_equal(d["bufs"], case["bufs"])                              # nothing was written

@@ -1,0 +1,106 @@
+"""GPU parity of sum_lstm against the CPU oracle (1e-2 rel / 2e-2 abs)."""
+import pytest
+import torch
+
+import oracle
+from helpers import assert_close, make_lstm_case, speculator_alpha, to_device_pitched
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+RTOL, ATOL = 1e-2, 2e-2
+
+
+def dev(t):
+    return None if t is None else to_device_pitched(t, DEV)
+
+
+def run(ops, c, alpha, eps_cell=1e-6, eps_state=1e-6, fast=False):
+    got_s, got_c = ops.sum_lstm(dev(c["states"]), dev(c["z4"]), dev(c["prev_cell"]), dev(c["w_cell"]),
+                                dev(c["b_cell"]), dev(c["w_state"]), dev(c["b_state"]), alpha, eps_cell,
+                                eps_state, fast)
+    torch.cuda.synchronize()
+    want_s, want_c = oracle.sum_lstm(c["states"], c["z4"], c["prev_cell"], c["w_cell"], c["b_cell"],
+                                     c["w_state"], c["b_state"], alpha, eps_cell, eps_state, fast)
+    pc = c["prev_cell"]
+    for got in (got_s, got_c):
+        assert got.shape == pc.shape and got.dtype == pc.dtype
+        assert got.stride() == pc.stride()          # outputs inherit prev_cell's row pitch
+    assert_close(got_c, want_c, RTOL, ATOL, "cell")
+    assert_close(got_s, want_s, RTOL, ATOL, "state")
+    return got_s, got_c, want_s, want_c
+
+
+# the reference's cases (tests/unit_tests/test_sum_lstm.py:174-179): pad4=7/padD=3 forces the element-wise kernel
+@pytest.mark.parametrize("cfg", [
+    dict(rows=1, D=64, pad4=0, padD=0),
+    dict(rows=4, D=128, pad4=7, padD=3),
+    dict(rows=32, D=256, pad4=0, padD=0),
+    dict(rows=64, D=512, pad4=16, padD=8),
+    dict(rows=3, D=12, pad4=0, padD=0),
+    dict(rows=2, D=8200, pad4=0, padD=0),
+    dict(rows=2, D=16392, pad4=0, padD=0),
+])
+@pytest.mark.parametrize("wb_cell", [True, False])
+@pytest.mark.parametrize("wb_state", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_reference_cases(ops, cfg, wb_cell, wb_state, dtype):
+    c = make_lstm_case(dtype=dtype, seed=1234, wb_cell=wb_cell, wb_state=wb_state, repeat_z=True, **cfg)
+    run(ops, c, alpha=0.35)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fast_gelu(ops, dtype):
+    c = make_lstm_case(rows=16, D=512, dtype=dtype, seed=5)
+    run(ops, c, alpha=0.35, fast=True)
+
+
+@pytest.mark.parametrize("alpha", [speculator_alpha(3, 4096), 1.0])
+def test_config4_three_steps(ops, alpha):
+    """BASELINE config 4: T=512, H=4096, bf16, 3 chained steps (cell_{k+1} = out_cell_k,
+    fresh pre-activations per step)."""
+    cell_gpu = cell_cpu = None
+    for step in range(3):
+        c = make_lstm_case(rows=512, D=4096, seed=3 + 10 * step)
+        if step:
+            # both sides continue from the oracle's cell so that one step's rounding
+            # differences are not fed through the next
+            c["prev_cell"] = cell_cpu
+        got_s, got_c, want_s, want_c = run(ops, c, alpha=alpha)
+        cell_cpu = want_c
+        same = (got_c.cpu().view(torch.int16) == want_c.view(torch.int16)).float().mean().item()
+        assert same > 0.97, f"step {step}: only {same:.4f} of the cells are bit-identical to the oracle"
+
+
+def test_rank3_inputs(ops):
+    c = make_lstm_case(rows=6, D=256, seed=8)
+    for k in ("states", "z4", "prev_cell"):
+        c[k] = c[k].contiguous().view(2, 3, -1)
+    got_s, got_c, _, _ = run(ops, c, alpha=0.5)
+    assert got_s.shape == (2, 3, 256)
+
+
+def test_empty(ops):
+    z = torch.empty(0, 256, dtype=torch.bfloat16, device=DEV)
+    s, c = ops.sum_lstm(z, z, torch.empty(0, 64, dtype=torch.bfloat16, device=DEV), None, None, None, None,
+                        1.0, 1e-6, 1e-6, False)
+    assert s.shape == (0, 64) and c.shape == (0, 64)
+
+
+def test_errors(ops):
+    bf = dict(dtype=torch.bfloat16, device=DEV)
+    s, z, pc = torch.randn(4, 256, **bf), torch.randn(4, 256, **bf), torch.randn(4, 64, **bf)
+    args = (None, None, None, None, 1.0, 1e-6, 1e-6, False)
+    with pytest.raises(RuntimeError, match="sum_lstm: only fp16 and bf16"):
+        ops.sum_lstm(s.float(), z.float(), pc.float(), *args)
+    with pytest.raises(RuntimeError, match="all input dtypes must match"):
+        ops.sum_lstm(s, z.half(), pc, *args)
+    with pytest.raises(RuntimeError, match="last dim of states must be 4\\*D_gate"):
+        ops.sum_lstm(s[:, :254], z[:, :254], pc, *args)
+    with pytest.raises(RuntimeError, match="z4 must have last dim"):
+        ops.sum_lstm(s, z[:, :128], pc, *args)
+    with pytest.raises(RuntimeError, match="prev_cell last dim must equal D_gate"):
+        ops.sum_lstm(s, z, pc[:, :32], *args)
+    with pytest.raises(RuntimeError, match="w_cell must have length >= D_eff"):
+        ops.sum_lstm(s, z, pc, torch.ones(8, **bf), None, None, None, 1.0, 1e-6, 1e-6, False)
+    with pytest.raises(RuntimeError, match="b_state dtype mismatch"):
+        ops.sum_lstm(s, z, pc, None, None, None, torch.ones(64, device=DEV), 1.0, 1e-6, 1e-6, False)

@@ -95,20 +95,42 @@ __device__ __forceinline__ uint4 load16(const void *p) {
   return make_uint4(v.x, v.y, v.z, v.w);
 }
 // streaming variants: every byte on these paths is touched exactly once
+#ifndef ARCTIC_NT_LOAD
+#define ARCTIC_NT_LOAD 1
+#endif
+#ifndef ARCTIC_NT_STORE
+#define ARCTIC_NT_STORE 1
+#endif
 __device__ __forceinline__ uint4 load16_stream(const void *p) {
+#if ARCTIC_NT_LOAD
   const u32x4 v = __builtin_nontemporal_load((const ARCTIC_GLOBAL u32x4 *)p);
+#else
+  const u32x4 v = *(const ARCTIC_GLOBAL u32x4 *)p;
+#endif
   return make_uint4(v.x, v.y, v.z, v.w);
 }
 __device__ __forceinline__ void store16_stream(void *p, const uint4 &v) {
   const u32x4 t = {v.x, v.y, v.z, v.w};
+#if ARCTIC_NT_STORE
   __builtin_nontemporal_store(t, (ARCTIC_GLOBAL u32x4 *)p);
+#else
+  *(ARCTIC_GLOBAL u32x4 *)p = t;
+#endif
 }
 __device__ __forceinline__ void store8_stream(void *p, const uint2 &v) {
   const u32x2 t = {v.x, v.y};
+#if ARCTIC_NT_STORE
   __builtin_nontemporal_store(t, (ARCTIC_GLOBAL u32x2 *)p);
+#else
+  *(ARCTIC_GLOBAL u32x2 *)p = t;
+#endif
 }
 __device__ __forceinline__ void store4_stream(void *p, uint32_t v) {
+#if ARCTIC_NT_STORE
   __builtin_nontemporal_store(v, (ARCTIC_GLOBAL uint32_t *)p);
+#else
+  *(ARCTIC_GLOBAL uint32_t *)p = v;
+#endif
 }
 
 // ---- wave64 / workgroup reductions ------------------------------------------

@@ -23,6 +23,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdlib>
 #include <type_traits>
 
 #include "common.hpp"
@@ -30,7 +31,7 @@
 
 namespace arctic {
 
-constexpr int kBulkThreads = 256;
+constexpr int kScalarThreads = 256;
 constexpr int kLayersPerLaunch = 64;  // 4 tables x 64 pointers = 2 KiB of kernel arguments
 
 struct LayerTables {
@@ -107,49 +108,20 @@ __device__ __forceinline__ void emit_chunk(const uint4 &v, const RowDesc &d, int
   }
 }
 
-template <typename Src, typename Dst, bool kPow2>
+// kBulkThreads x kUnroll 16-byte chunks form one batch of a workgroup.  Two shapes
+// are built: 512 x 2 (long prefill launches) and 256 x 4 (few tokens).
+template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll>
 __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
     const BulkParams p, const LayerTables tab) {
   constexpr bool kCopy = std::is_same<Dst, Copy>::value;
   constexpr int kDstElemBytes = kCopy ? Src::kBytes : 1;
-  constexpr int kUnroll = 4;
 
   __shared__ RowDesc rows[2 * kLayersPerLaunch];
 
-  const int64_t token = blockIdx.x / p.groups_per_token;
-  const int group = blockIdx.x - (int)(token * p.groups_per_token);
+  const int64_t token = blockIdx.x / (unsigned)p.groups_per_token;
+  const int group = blockIdx.x - (unsigned)token * (unsigned)p.groups_per_token;
   const int layer0 = group * p.layers_per_group;
   const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
-
-  const int64_t slot = p.slot_mapping[token];
-  if (slot < 0) return;  // padding token: uniform exit, before any barrier
-
-  int64_t blk, off;
-  if (slot < 0x7fffffffLL) {
-    const uint32_t s32 = (uint32_t)slot, bs = (uint32_t)p.block_size;
-    blk = s32 / bs;
-    off = s32 - (uint32_t)blk * bs;
-  } else {
-    blk = slot / p.block_size;
-    off = slot - blk * p.block_size;
-  }
-  const int64_t row_elem = blk * p.block_stride + off * (int64_t)p.n;
-
-  // prologue: one lane per (layer, K|V) row of this token
-  for (int r = threadIdx.x; r < 2 * nlayers; r += kBulkThreads) {
-    const int layer = layer0 + (r >> 1);
-    const bool is_v = r & 1;
-    const void *base = is_v ? tab.value_cache[layer] : tab.key_cache[layer];
-    RowDesc d;
-    d.dst = (char *)base + row_elem * kDstElemBytes;
-    d.inv = 0.0;
-    if constexpr (!kCopy) {
-      const float *sp = is_v ? tab.v_scale[layer] : tab.k_scale[layer];
-      d.inv = 1.0 / (double)(*sp);
-    }
-    rows[r] = d;
-  }
-  __syncthreads();
 
   const char *ksrc = p.keys + token * p.key_stride_bytes + (int64_t)layer0 * p.n * Src::kBytes;
   const char *vsrc = p.values + token * p.value_stride_bytes + (int64_t)layer0 * p.n * Src::kBytes;
@@ -165,40 +137,86 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
       col = c - r * cpr;
     }
   };
-  auto src_of = [&](int r, int col) -> const char * {
-    const char *base = (r & 1) ? vsrc : ksrc;
-    return base + ((int64_t)(r >> 1) * cpr + col) * 16;
-  };
-
-  int c = threadIdx.x;
-  // main loop: kUnroll independent 16-byte loads in flight per lane
-  for (; c + (kUnroll - 1) * kBulkThreads < total; c += kUnroll * kBulkThreads) {
-    uint4 v[kUnroll];
-    int r[kUnroll], col[kUnroll];
+  // kUnroll independent 16-byte loads per lane; lanes past the end load nothing
+  auto load_batch = [&](int c, uint4 (&v)[kUnroll]) {
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-      locate(c + u * kBulkThreads, r[u], col[u]);
-      v[u] = load16_stream(src_of(r[u], col[u]));
+      const int cu = c + u * kBulkThreads;
+      if (cu < total) {
+        int r, col;
+        locate(cu, r, col);
+        const char *base = (r & 1) ? vsrc : ksrc;
+        v[u] = load16_stream(base + ((int64_t)(r >> 1) * cpr + col) * 16);
+      }
+    }
+  };
+
+  // The slot lookup and the first batch of source loads are issued together:
+  // source addresses do not depend on the slot, so HBM is already streaming
+  // while the row descriptors below are being built.  (A padding token throws
+  // its first batch away.)
+  const int64_t slot = p.slot_mapping[token];
+  int c = threadIdx.x;
+  uint4 cur[kUnroll];
+  load_batch(c, cur);
+  if (slot < 0) return;  // padding token: uniform exit, before any barrier
+
+  int64_t blk, off;
+  if (slot < 0x7fffffffLL) {
+    const uint32_t s32 = (uint32_t)slot, bs = (uint32_t)p.block_size;
+    blk = s32 / bs;
+    off = s32 - (uint32_t)blk * bs;
+  } else {
+    blk = slot / p.block_size;
+    off = slot - blk * p.block_size;
+  }
+  const int64_t row_elem = blk * p.block_stride + off * (int64_t)p.n;
+
+  // one lane per (layer, K|V) row of this token
+  for (int r = threadIdx.x; r < 2 * nlayers; r += kBulkThreads) {
+    const int layer = layer0 + (r >> 1);
+    const bool is_v = r & 1;
+    const void *base = is_v ? tab.value_cache[layer] : tab.key_cache[layer];
+    RowDesc d;
+    d.dst = (char *)base + row_elem * kDstElemBytes;
+    d.inv = 0.0;
+    if constexpr (!kCopy) {
+      const float *sp = is_v ? tab.v_scale[layer] : tab.k_scale[layer];
+      d.inv = 1.0 / (double)(*sp);
+    }
+    rows[r] = d;
+  }
+  __syncthreads();
+
+  // software-pipelined main loop: the next batch is in flight while this one
+  // is converted and stored
+  while (c < total) {
+    const int cn = c + kUnroll * kBulkThreads;
+    uint4 nxt[kUnroll];
+    load_batch(cn, nxt);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int cu = c + u * kBulkThreads;
+      if (cu < total) {
+        int r, col;
+        locate(cu, r, col);
+        emit_chunk<Src, Dst>(cur[u], rows[r], col);
+      }
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) emit_chunk<Src, Dst>(v[u], rows[r[u]], col[u]);
-  }
-  for (; c < total; c += kBulkThreads) {
-    int r, col;
-    locate(c, r, col);
-    const uint4 v = load16_stream(src_of(r, col));
-    emit_chunk<Src, Dst>(v, rows[r], col);
+    for (int u = 0; u < kUnroll; ++u) cur[u] = nxt[u];
+    c = cn;
   }
 }
 
 // Fallback for shapes or addresses that do not allow 16-byte accesses: one
 // element per lane per step, any alignment.  Same arithmetic, no vector access.
 template <typename SrcElem, typename Dst>
-__global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_scalar_kernel(
+__global__ __launch_bounds__(kScalarThreads) void kv_write_bulk_scalar_kernel(
     const BulkParams p, const LayerTables tab, const int src_dtype) {
   constexpr bool kCopy = std::is_same<Dst, Copy>::value;
-  const int64_t token = blockIdx.x / p.groups_per_token;
-  const int group = blockIdx.x - (int)(token * p.groups_per_token);
+  const int64_t token = blockIdx.x / (unsigned)p.groups_per_token;
+  const int group = blockIdx.x - (unsigned)token * (unsigned)p.groups_per_token;
   const int layer0 = group * p.layers_per_group;
   const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
   const int64_t slot = p.slot_mapping[token];
@@ -215,7 +233,7 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_scalar_kernel(
       kinv = 1.0 / (double)(*tab.k_scale[l]);
       vinv = 1.0 / (double)(*tab.v_scale[l]);
     }
-    for (int i = threadIdx.x; i < p.n; i += kBulkThreads) {
+    for (int i = threadIdx.x; i < p.n; i += kScalarThreads) {
       const SrcElem k = ks[(int64_t)l * p.n + i];
       const SrcElem v = vs[(int64_t)l * p.n + i];
       if constexpr (kCopy) {
@@ -243,27 +261,32 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_scalar_kernel(
 }
 
 template <typename Src, typename Dst>
-static void launch_vec(const BulkParams &p, const LayerTables &tab, int64_t grid, hipStream_t s) {
-  if (p.chunk_shift >= 0)
-    hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true>), dim3((unsigned)grid), dim3(kBulkThreads), 0, s, p, tab);
-  else
-    hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, false>), dim3((unsigned)grid), dim3(kBulkThreads), 0, s, p, tab);
+static void launch_vec(const BulkParams &p, const LayerTables &tab, int64_t grid, bool wide, hipStream_t s) {
+  const dim3 g((unsigned)grid);
+  if (p.chunk_shift >= 0) {
+    if (wide)
+      hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 512, 2>), g, dim3(512), 0, s, p, tab);
+    else
+      hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 256, 4>), g, dim3(256), 0, s, p, tab);
+  } else {
+    hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, false, 256, 4>), g, dim3(256), 0, s, p, tab);
+  }
 }
 template <typename SrcElem, typename Dst>
 static void launch_scalar(const BulkParams &p, const LayerTables &tab, int64_t grid, int src_dtype,
                           hipStream_t s) {
   hipLaunchKernelGGL((kv_write_bulk_scalar_kernel<SrcElem, Dst>), dim3((unsigned)grid),
-                     dim3(kBulkThreads), 0, s, p, tab, src_dtype);
+                     dim3(kScalarThreads), 0, s, p, tab, src_dtype);
 }
 
 template <typename Dst>
-static void dispatch_src(bool vec, int src_dtype, const BulkParams &p, const LayerTables &tab,
+static void dispatch_src(bool vec, bool wide, int src_dtype, const BulkParams &p, const LayerTables &tab,
                          int64_t grid, hipStream_t s) {
   if (vec) {
     switch (src_dtype) {
-      case ARCTIC_DTYPE_BF16: launch_vec<SrcBF16, Dst>(p, tab, grid, s); break;
-      case ARCTIC_DTYPE_F16: launch_vec<SrcF16, Dst>(p, tab, grid, s); break;
-      default: launch_vec<SrcF32, Dst>(p, tab, grid, s); break;
+      case ARCTIC_DTYPE_BF16: launch_vec<SrcBF16, Dst>(p, tab, grid, wide, s); break;
+      case ARCTIC_DTYPE_F16: launch_vec<SrcF16, Dst>(p, tab, grid, wide, s); break;
+      default: launch_vec<SrcF32, Dst>(p, tab, grid, wide, s); break;
     }
   } else {
     if (src_dtype == ARCTIC_DTYPE_F32)
@@ -291,7 +314,8 @@ extern "C" int arctic_reshape_and_cache_flash_bulk(
   if (num_layers < 0 || num_layers > ARCTIC_MAX_LAYERS)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: num_layers=%d outside [0, %d]", fn, num_layers,
                 ARCTIC_MAX_LAYERS);
-  if (num_tokens < 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: num_tokens=%lld < 0", fn, (long long)num_tokens);
+  if (num_tokens < 0 || num_tokens > 0x7fffffffLL)
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: num_tokens=%lld outside [0, 2^31)", fn, (long long)num_tokens);
   if (num_heads <= 0 || head_size <= 0 || block_size <= 0)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: num_heads, head_size and block_size must be positive", fn);
   if (src_dtype != ARCTIC_DTYPE_F32 && src_dtype != ARCTIC_DTYPE_F16 && src_dtype != ARCTIC_DTYPE_BF16)
@@ -350,16 +374,25 @@ extern "C" int arctic_reshape_and_cache_flash_bulk(
     p.chunk_shift = -1;
     if (vec && (p.chunks_per_row & (p.chunks_per_row - 1)) == 0) p.chunk_shift = __builtin_ctz(p.chunks_per_row);
 
-    // Split a token's layers over several workgroups when there are too few
-    // tokens to fill the 256 CUs, but keep every workgroup at >= 4 steps of work.
-    const int64_t want_groups = 8192;
-    int groups = (int)std::min<int64_t>(count, (want_groups + num_tokens - 1) / num_tokens);
+    // One workgroup per token is best when there are thousands of tokens.  With
+    // few tokens (decode) a token's layers are split over several workgroups so
+    // that about eight workgroups per CU exist, each still moving at least one
+    // full batch of 1024 chunks.
+    int groups = 1;
+    bool wide = false;
     if (vec) {
       const int64_t chunks_per_layer = 2LL * p.chunks_per_row;
-      const int min_layers = (int)std::max<int64_t>(1, (4LL * kBulkThreads + chunks_per_layer - 1) / chunks_per_layer);
-      groups = std::min(groups, std::max(1, count / min_layers));
+      const int min_layers = (int)std::max<int64_t>(1, (1024 + chunks_per_layer - 1) / chunks_per_layer);
+      const int64_t want = (2048 + num_tokens - 1) / num_tokens;
+      groups = (int)std::max<int64_t>(1, std::min<int64_t>(want, count / min_layers));
+      wide = num_tokens >= 4096 && chunks_per_layer * count >= 8 * 1024;
+    } else {
+      groups = (int)std::max<int64_t>(1, std::min<int64_t>(count, (2048 + num_tokens - 1) / num_tokens));
     }
-    groups = std::max(groups, 1);
+#ifdef ARCTIC_TUNING
+    if (const char *e = getenv("ARCTIC_BULK_GROUPS")) groups = std::max(1, std::min(count, atoi(e)));
+    if (const char *e = getenv("ARCTIC_BULK_WIDE")) wide = atoi(e) != 0;
+#endif
     p.layers_per_group = (count + groups - 1) / groups;
     p.groups_per_token = (count + p.layers_per_group - 1) / p.layers_per_group;
     const int64_t grid = num_tokens * p.groups_per_token;
@@ -367,9 +400,9 @@ extern "C" int arctic_reshape_and_cache_flash_bulk(
       return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: too many tokens (%lld)", fn, (long long)num_tokens);
 
     switch (kv_cache_dtype) {
-      case ARCTIC_KV_AUTO: dispatch_src<Copy>(vec, src_dtype, p, tab, grid, s); break;
-      case ARCTIC_KV_FP8_E4M3: dispatch_src<E4M3>(vec, src_dtype, p, tab, grid, s); break;
-      default: dispatch_src<E5M2>(vec, src_dtype, p, tab, grid, s); break;
+      case ARCTIC_KV_AUTO: dispatch_src<Copy>(vec, wide, src_dtype, p, tab, grid, s); break;
+      case ARCTIC_KV_FP8_E4M3: dispatch_src<E4M3>(vec, wide, src_dtype, p, tab, grid, s); break;
+      default: dispatch_src<E5M2>(vec, wide, src_dtype, p, tab, grid, s); break;
     }
     const int rc = check_launch(fn);
     if (rc) return rc;

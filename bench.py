@@ -1,0 +1,315 @@
+#!/usr/bin/env python3
+"""Benchmark of the csrc/custom_ops hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one bulk KV-cache write (one launch of the hot path) over the 70B
+SwiftKV shape of BASELINE.json (configs[2]): 16384 tokens, 40 layers, 8 KV heads
+x 128, block 16, fp8-e4m3 cache with per-tensor amax/448 scales, 10 % of the
+slots are padding.  Inputs are resident in HBM before the timed region.  The
+last stdout line is ONE JSON object:
+
+  value / ms_per_step   wall clock around exactly K steps (sync on both sides)
+  roofline              the kernel's own duration from HIP events recorded on the
+                        stream it is launched on, against the 8 TB/s HBM peak
+  cpu_baseline          the CPU oracle (a C port of the reference kernel, OpenMP)
+                        timed on this machine's host cores on a bounded sample
+  extras                the other BASELINE configs (speculator ops, decode mix)
+
+Only one GPU is used; --gpus N with N > 1 is refused.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+HBM_PEAK_GBS = 8000.0
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_slots(num_tokens, num_slots, gen, pad_fraction):
+    n_pad = int(pad_fraction * num_tokens)
+    slots = torch.full((num_tokens,), -1, dtype=torch.int64)
+    order = torch.randperm(num_tokens, generator=gen)
+    valid = order[n_pad:]
+    slots[valid] = torch.randperm(num_slots, generator=gen)[: valid.numel()]
+    return slots
+
+
+class BulkWorkload:
+    """One bulk KV-write configuration, resident on the GPU."""
+
+    def __init__(self, name, T, L, H, D, bs, NB, kv, pad_fraction, seed, std, dev):
+        self.name, self.T, self.L, self.H, self.D, self.bs, self.NB, self.kv = name, T, L, H, D, bs, NB, kv
+        n = H * D
+        self.n = n
+        g = torch.Generator().manual_seed(seed)
+        gd = torch.Generator(device=dev).manual_seed(seed)
+        self.keys = torch.empty(T, L * n, dtype=torch.bfloat16, device=dev)
+        self.values = torch.empty(T, L * n, dtype=torch.bfloat16, device=dev)
+        step = max(1, min(T, (1 << 24) // (L * n)))
+        for t0 in range(0, T, step):
+            t1 = min(T, t0 + step)
+            self.keys[t0:t1] = (torch.randn(t1 - t0, L * n, generator=gd, device=dev) * std).to(torch.bfloat16)
+            self.values[t0:t1] = (torch.randn(t1 - t0, L * n, generator=gd, device=dev) * std).to(torch.bfloat16)
+        self.slots_cpu = make_slots(T, NB * bs, g, pad_fraction)
+        self.slots = self.slots_cpu.to(dev)
+        self.valid = int((self.slots_cpu >= 0).sum())
+        quant = kv != "auto"
+        cdt = torch.uint8 if quant else torch.bfloat16
+        self.bufs = [torch.zeros(2, NB, bs, H, D, dtype=cdt, device=dev) for _ in range(L)]
+        self.key_caches = [b[0] for b in self.bufs]
+        self.value_caches = [b[1] for b in self.bufs]
+        if quant:
+            self.k_scales = [(self.keys[:, l * n:(l + 1) * n].float().abs().max() / 448.0) for l in range(L)]
+            self.v_scales = [(self.values[:, l * n:(l + 1) * n].float().abs().max() / 448.0) for l in range(L)]
+        else:
+            self.k_scales = [torch.ones((), device=dev) for _ in range(L)]
+            self.v_scales = [torch.ones((), device=dev) for _ in range(L)]
+        # algorithmic bytes: read K+V once (2 B each), write the cache once (1 or 2 B each)
+        self.bytes_per_unit = n * (4 + (2 if quant else 4))
+        self.bytes = self.valid * L * self.bytes_per_unit
+
+    def args(self):
+        return (self.keys, self.values, self.key_caches, self.value_caches, self.slots, self.kv,
+                self.k_scales, self.v_scales, self.H, self.D)
+
+
+def event_times_us(fn, iters):
+    """Duration of each call of fn() from HIP events on the current stream."""
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+    for i in range(iters):
+        starts[i].record()
+        fn()
+        ends[i].record()
+    torch.cuda.synchronize()
+    return [s.elapsed_time(e) * 1e3 for s, e in zip(starts, ends)]
+
+
+def cpu_baseline_bulk(w: BulkWorkload, target_seconds=6.0):
+    """Time the CPU oracle on a sample of the workload's tokens (all layers)."""
+    import oracle
+    threads = oracle.num_threads()
+    n, L = w.n, w.L
+
+    def run(sample_tokens):
+        g = torch.Generator().manual_seed(99)
+        sample = torch.randperm(w.T, generator=g)[:sample_tokens]
+        sub = w.slots_cpu[sample]
+        nvalid = int((sub >= 0).sum())
+        remap = torch.full_like(sub, -1)
+        remap[sub >= 0] = torch.arange(nvalid)
+        keys = w.keys[sample.to(w.keys.device)].cpu().contiguous()
+        values = w.values[sample.to(w.keys.device)].cpu().contiguous()
+        nb = (nvalid + w.bs - 1) // w.bs
+        bufs = [torch.zeros(2, nb, w.bs, w.H, w.D, dtype=w.bufs[0].dtype) for _ in range(L)]
+        ks = [s.cpu() for s in w.k_scales]
+        vs = [s.cpu() for s in w.v_scales]
+        t0 = time.perf_counter()
+        oracle.reshape_and_cache_flash_bulk(keys, values, [b[0] for b in bufs], [b[1] for b in bufs], remap,
+                                            w.kv, ks, vs, w.H, w.D)
+        dt = time.perf_counter() - t0
+        return dt, nvalid * L * w.bytes_per_unit
+
+    dt, nbytes = run(min(w.T, 128))             # calibration pass (also warms the library)
+    rate = nbytes / dt
+    tokens = int(min(w.T, max(128, target_seconds * rate / (L * w.bytes_per_unit))))
+    dt, nbytes = run(tokens)
+    return {
+        "value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": f"{tokens} of {w.T} tokens x {L} layers of the same workload "
+                  f"({nbytes / 1e6:.0f} MB algorithmic) in {dt:.2f} s, C oracle with OpenMP",
+    }
+
+
+def bench_speculator(ops, dev, steps, warmup):
+    """BASELINE config 4: sum_lstm (3 chained steps) and the standalone LayerNorm at
+    T=512, H=4096, bf16.  Eight buffer sets (> 256 MB in total) are rotated so that
+    the inputs do not stay resident in the last-level cache between launches."""
+    T, Hd, sets = 512, 4096, 8
+    g = torch.Generator(device=dev).manual_seed(3)
+    rn = lambda *s: torch.randn(*s, generator=g, device=dev).to(torch.bfloat16)
+    S = [[rn(T, 4 * Hd) for _ in range(3)] for _ in range(sets)]
+    Z = [[rn(T, 4 * Hd) for _ in range(3)] for _ in range(sets)]
+    C0 = [rn(T, Hd) for _ in range(sets)]
+    X = [rn(T, Hd) for _ in range(sets)]
+    vec = lambda m: (m + 0.02 * torch.randn(Hd, generator=g, device=dev)).to(torch.bfloat16)
+    w_cell, b_cell, w_state, b_state = vec(1.0), vec(0.0), vec(1.0), vec(0.0)
+    sw = 0.5 ** (0.5 / 3)
+    alpha = ((1 - sw * sw) * (Hd / 2)) ** 0.5 / sw
+
+    def lstm3(i):
+        cell = C0[i % sets]
+        for k in range(3):
+            _, cell = ops.sum_lstm(S[i % sets][k], Z[i % sets][k], cell, w_cell, b_cell, w_state, b_state,
+                                   alpha, 1e-6, 1e-6, False)
+
+    def ln(i):
+        ops.speculator_ln(X[i % sets], w_cell, b_cell, 1e-6)
+
+    out = {}
+    for name, fn, per_call, calls in (("sum_lstm", lstm3, 22 * Hd * T, 3), ("speculator_ln", ln, 4 * Hd * T, 1)):
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        counter = iter(range(10 ** 9))
+        us = event_times_us(lambda: fn(next(counter)), steps)
+        med = statistics.median(us) / calls
+        out[name] = {"us_per_call_eager": round(med, 2), "bytes_per_call": per_call}
+        # the same loop inside one HIP graph: kernel time without host launch gaps
+        graph = torch.cuda.CUDAGraph()
+        reps = sets
+        with torch.cuda.graph(graph):
+            for i in range(reps):
+                fn(i)
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        us = event_times_us(graph.replay, max(10, steps // 2))
+        med = statistics.median(us) / (reps * calls)
+        out[name].update({"us_per_call_graph": round(med, 2),
+                          "GBps_graph": round(per_call / med / 1e3, 1),
+                          "hbm_frac_graph": round(per_call / med / 1e3 / HBM_PEAK_GBS, 4)})
+    return out
+
+
+def bench_decode_mix(ops, dev, steps):
+    """BASELINE config 5: 512 decode tokens; bulk fp8 KV write over 16 layers into
+    32768-block caches, ln0, three sum_lstm steps; one HIP graph per step."""
+    w = BulkWorkload("decode", 512, 16, 8, 128, 16, 32768, "fp8", 0.0, 4, 1.5, dev)
+    T, Hd = 512, 4096
+    g = torch.Generator(device=dev).manual_seed(4)
+    rn = lambda *s: torch.randn(*s, generator=g, device=dev).to(torch.bfloat16)
+    sets = 4
+    S = [[rn(T, 4 * Hd) for _ in range(3)] for _ in range(sets)]
+    Z = [[rn(T, 4 * Hd) for _ in range(3)] for _ in range(sets)]
+    X = [rn(T, Hd) for _ in range(sets)]
+    vec = lambda m: (m + 0.02 * torch.randn(Hd, generator=g, device=dev)).to(torch.bfloat16)
+    w_cell, b_cell, w_state, b_state = vec(1.0), vec(0.0), vec(1.0), vec(0.0)
+    sw = 0.5 ** (0.5 / 3)
+    alpha = ((1 - sw * sw) * (Hd / 2)) ** 0.5 / sw
+
+    def step(i):
+        ops.reshape_and_cache_flash_bulk(*w.args())
+        ops.speculator_ln(X[i], None, None, 1e-6)
+        cell = torch.zeros(T, Hd, dtype=torch.bfloat16, device=dev)
+        for k in range(3):
+            _, cell = ops.sum_lstm(S[i][k], Z[i][k], cell, w_cell, b_cell, w_state, b_state, alpha, 1e-6, 1e-6,
+                                   False)
+
+    step(0)
+    torch.cuda.synchronize()
+    graphs = []
+    for i in range(sets):
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            step(i)
+        graphs.append(gr)
+    for gr in graphs:
+        gr.replay()
+    torch.cuda.synchronize()
+    counter = iter(range(10 ** 9))
+    us = event_times_us(lambda: graphs[next(counter) % sets].replay(), max(40, steps))
+    med = statistics.median(us)
+    nbytes = w.bytes + 4 * Hd * T + 3 * 22 * Hd * T
+    return {"us_per_step_graph": round(med, 2), "bytes_per_step": nbytes,
+            "GBps": round(nbytes / med / 1e3, 1), "hbm_frac": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-extras", action="store_true", help="skip the speculator / decode-mix measurements")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path is built and measured on ONE GPU (every token, layer and row is "
+                 "independent, so more GPUs only run the same kernel on their own share); use --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+
+    from arcticinference_amd import py_custom_ops as ops
+    if not ops.try_load_torch_library():
+        sys.exit("bench.py: libarctic_mi355x.so is not built; run `python -c 'import __graft_entry__ as g; g.build()'`")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    log(f"device: {torch.cuda.get_device_name(0)}; host cores: {os.cpu_count()}")
+
+    w = BulkWorkload("70B-SwiftKV", 16384, 40, 8, 128, 16, 8192, "fp8", 0.10, 2, 1.5, dev)
+    fn = lambda: ops.reshape_and_cache_flash_bulk(*w.args())
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        fn()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    value = w.bytes / (wall / args.steps) / 1e9
+
+    us = event_times_us(fn, args.steps)
+    kernel_us = statistics.mean(us)
+    achieved = w.bytes / kernel_us / 1e3
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get("kv_write_bulk_fp8_70b", {}).get("hbm_bytes_per_launch")
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "kernel": "kv_write_bulk_kernel<bf16, e4m3>", "kernel_us_mean": round(kernel_us, 2),
+                "kernel_us_median": round(statistics.median(us), 2), "algorithmic_bytes": w.bytes}
+    log(f"bulk fp8 70B shape: {ms_per_step:.3f} ms/step wall, kernel {kernel_us:.1f} us, {achieved:.0f} GB/s")
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline_bulk(w)
+        log(f"cpu baseline: {cpu}")
+
+    extras = {}
+    if not args.no_extras:
+        w2 = BulkWorkload("8B-prefill", 8192, 16, 8, 128, 16, 8192, "fp8", 0.0, 1, 1.5, dev)
+        f2 = lambda: ops.reshape_and_cache_flash_bulk(*w2.args())
+        for _ in range(5):
+            f2()
+        m = statistics.median(event_times_us(f2, args.steps))
+        extras["bulk_fp8_8b_prefill"] = {"kernel_us": round(m, 2), "GBps": round(w2.bytes / m / 1e3, 1),
+                                         "hbm_frac": round(w2.bytes / m / 1e3 / HBM_PEAK_GBS, 4)}
+        del w2, f2
+        torch.cuda.empty_cache()
+        extras["speculator"] = bench_speculator(ops, dev, args.steps, args.warmup)
+        extras["decode_mix"] = bench_decode_mix(ops, dev, args.steps)
+        log(f"extras: {extras}")
+
+    result = {
+        "metric": "bulk KV-write HBM GB/s (fp8-e4m3, 70B SwiftKV shape)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "fp8_e4m3",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE configs[2]: bulk KV write, 16384 tokens x 40 layers x 8 KV heads x 128, "
+                               "block 16, 8192 blocks, fp8-e4m3 cache, amax/448 scales, 10% slots = -1",
+                   "tokens": w.T, "valid_tokens": w.valid, "layers": w.L, "kv_heads": w.H, "head_size": w.D,
+                   "block_size": w.bs, "num_blocks": w.NB, "parallelism": "single GPU"},
+        "roofline": roofline, "cpu_baseline": cpu, "extras": extras,
+    }
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

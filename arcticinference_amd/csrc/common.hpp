@@ -26,17 +26,17 @@ struct BF16 {
   __device__ static __forceinline__ float hi(uint32_t w) {
     return __uint_as_float(w & 0xffff0000u);
   }
-  __device__ static __forceinline__ uint32_t round_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-    return (f != f) ? 0x7fffu : r;
-  }
+  // gfx950 rounds fp32 pairs to bf16 in hardware (v_cvt_pk_bf16_f32, RNE)
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
   __device__ static __forceinline__ uint32_t pack(float a, float b) {
-    return round_bits(a) | (round_bits(b) << 16);
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
   }
+  __device__ static __forceinline__ uint32_t round_bits(float f) { return pack(f, 0.f) & 0xffffu; }
   // value of the rounded 16-bit number, as fp32
   __device__ static __forceinline__ float requant(float f) {
-    return __uint_as_float(round_bits(f) << 16);
+    return __uint_as_float(pack(f, 0.f) << 16);
   }
 };
 
@@ -155,19 +155,25 @@ __device__ __forceinline__ float wave_sum(float v) {
   return (r0 + r1) + (r2 + r3);
 }
 
-// Sum over the whole workgroup (blockDim.x a multiple of 64, at most 1024).
-// `slots` is LDS for 16 floats, private to this call site; all threads get the
-// same value because all of them add the partials in the same order.
+// Sum over the whole workgroup (blockDim.x a multiple of 64, at most 1024 = 16
+// waves).  `slots` is LDS for 16 floats, private to this call site.  Each wave
+// leaves its total in slots[wave]; after the barrier every row of 16 lanes reads
+// the 16 slots (zero beyond the last wave) and folds them with the same DPP
+// butterfly, so all lanes of all waves end with the identical total and no loop
+// or branch depends on the number of waves.
 __device__ __forceinline__ float block_sum(float v, float *slots) {
   v = wave_sum(v);
   const int nwaves = blockDim.x >> 6;
   if (nwaves == 1) return v;
-  const int wave = threadIdx.x >> 6;
-  if ((threadIdx.x & 63) == 0) slots[wave] = v;
+  const int lane = threadIdx.x & 63;
+  if (lane == 0) slots[threadIdx.x >> 6] = v;
   __syncthreads();
-  float total = 0.f;
-  for (int w = 0; w < nwaves; ++w) total += slots[w];
-  return total;
+  float t = ((lane & 15) < nwaves) ? slots[lane & 15] : 0.f;
+  t = dpp_add<0xB1>(t);   // quad_perm [1,0,3,2]
+  t = dpp_add<0x4E>(t);   // quad_perm [2,3,0,1]
+  t = dpp_add<0x141>(t);  // row_half_mirror
+  t = dpp_add<0x140>(t);  // row_mirror
+  return t;
 }
 
 }  // namespace arctic

@@ -19,14 +19,22 @@ namespace arctic {
 template <typename T, int kChunksPerThread>
 __global__ __launch_bounds__(1024) void spec_ln_vec_kernel(
     char *__restrict__ out, const char *__restrict__ in, const char *__restrict__ weight,
-    const char *__restrict__ bias, int64_t in_row_stride_bytes, int hidden, float eps) {
+    const char *__restrict__ bias, int64_t in_row_stride_bytes, int hidden, float inv_hidden, float eps) {
   __shared__ float slots[16];
   const int chunks = hidden >> 3;
   const char *row_in = in + (int64_t)blockIdx.x * in_row_stride_bytes;
   char *row_out = out + (int64_t)blockIdx.x * hidden * 2;
 
-  uint4 raw[kChunksPerThread];
+  uint4 raw[kChunksPerThread], wv[kChunksPerThread], bv[kChunksPerThread];
   float ss = 0.f;
+  // scale / shift first: they are cache resident and memory returns loads in issue
+  // order, so asking for them after the row sum would add a full round trip
+#pragma unroll
+  for (int k = 0; k < kChunksPerThread; ++k) {
+    const int c = threadIdx.x + k * blockDim.x;
+    if (weight && c < chunks) wv[k] = load16(weight + (int64_t)c * 16);
+    if (bias && c < chunks) bv[k] = load16(bias + (int64_t)c * 16);
+  }
 #pragma unroll
   for (int k = 0; k < kChunksPerThread; ++k) {
     const int c = threadIdx.x + k * blockDim.x;
@@ -41,7 +49,7 @@ __global__ __launch_bounds__(1024) void spec_ln_vec_kernel(
     for (int j = 0; j < 8; ++j) ss += x[j] * x[j];
   }
   const float total = block_sum(ss, slots);
-  const float inv = rsqrtf(total / (float)hidden + eps);
+  const float inv = rsqrtf(total * inv_hidden + eps);
 
 #pragma unroll
   for (int k = 0; k < kChunksPerThread; ++k) {
@@ -53,13 +61,13 @@ __global__ __launch_bounds__(1024) void spec_ln_vec_kernel(
     for (int j = 0; j < 8; ++j) x[j] *= inv;
     if (weight) {
       float w[8];
-      unpack8<T>(load16(weight + (int64_t)c * 16), w);
+      unpack8<T>(wv[k], w);
 #pragma unroll
       for (int j = 0; j < 8; ++j) x[j] *= w[j];
     }
     if (bias) {
       float b[8];
-      unpack8<T>(load16(bias + (int64_t)c * 16), b);
+      unpack8<T>(bv[k], b);
 #pragma unroll
       for (int j = 0; j < 8; ++j) x[j] += b[j];
     }
@@ -71,7 +79,7 @@ __global__ __launch_bounds__(1024) void spec_ln_vec_kernel(
 template <typename T>
 __global__ __launch_bounds__(256) void spec_ln_scalar_kernel(
     uint16_t *__restrict__ out, const uint16_t *__restrict__ in, const uint16_t *__restrict__ weight,
-    const uint16_t *__restrict__ bias, int64_t in_row_stride, int hidden, float eps) {
+    const uint16_t *__restrict__ bias, int64_t in_row_stride, int hidden, float inv_hidden, float eps) {
   __shared__ float slots[16];
   const uint16_t *row_in = in + (int64_t)blockIdx.x * in_row_stride;
   uint16_t *row_out = out + (int64_t)blockIdx.x * hidden;
@@ -81,7 +89,7 @@ __global__ __launch_bounds__(256) void spec_ln_scalar_kernel(
     ss += x * x;
   }
   const float total = block_sum(ss, slots);
-  const float inv = rsqrtf(total / (float)hidden + eps);
+  const float inv = rsqrtf(total * inv_hidden + eps);
   for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
     float y = T::lo(row_in[j]) * inv;
     if (weight) y *= T::lo(weight[j]);
@@ -96,6 +104,7 @@ template <typename T>
 static void launch_ln(void *out, const void *in, const void *w, const void *b, int64_t rows, int hidden,
                       int64_t in_row_stride, float eps, hipStream_t s) {
   const int chunks = hidden / 8;
+  const float inv_hidden = 1.0f / (float)hidden;
   const bool vec = (hidden % 8 == 0) && (in_row_stride % 8 == 0 || rows == 1) && aligned16(in) &&
                    aligned16(out) && (!w || aligned16(w)) && (!b || aligned16(b)) && chunks <= 8 * 1024;
   const dim3 grid((unsigned)rows);
@@ -107,7 +116,7 @@ static void launch_ln(void *out, const void *in, const void *w, const void *b, i
     const int64_t stride_bytes = in_row_stride * 2;
 #define ARCTIC_LN_LAUNCH(CPT)                                                                         \
   hipLaunchKernelGGL((spec_ln_vec_kernel<T, CPT>), grid, dim3(threads), 0, s, (char *)out,             \
-                     (const char *)in, (const char *)w, (const char *)b, stride_bytes, hidden, eps)
+                     (const char *)in, (const char *)w, (const char *)b, stride_bytes, hidden, inv_hidden, eps)
     switch (cpt) {
       case 1: ARCTIC_LN_LAUNCH(1); break;
       case 2: ARCTIC_LN_LAUNCH(2); break;
@@ -118,7 +127,7 @@ static void launch_ln(void *out, const void *in, const void *w, const void *b, i
   } else {
     hipLaunchKernelGGL((spec_ln_scalar_kernel<T>), grid, dim3(256), 0, s, (uint16_t *)out,
                        (const uint16_t *)in, (const uint16_t *)w, (const uint16_t *)b, in_row_stride, hidden,
-                       eps);
+                       inv_hidden, eps);
   }
 }
 

@@ -13,18 +13,43 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdlib>
 
 #include "common.hpp"
 
 namespace arctic {
 
-// sigmoid_f / gelu_erf / gelu_tanh of the reference (sum_lstm.cu:14-26).
-__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+// sigmoid_f / gelu_erf / gelu_tanh of the reference (sum_lstm.cu:14-26), built on
+// the hardware exp2 and reciprocal instructions (1 ulp each) instead of library
+// calls: per output element the operator needs three sigmoids and two GELUs, and
+// with library expf / erff / IEEE division the arithmetic alone would take longer
+// than moving the row through HBM.
+__device__ __forceinline__ float fast_exp(float x) {            // e^x
+  return __builtin_amdgcn_exp2f(x * 1.4426950408889634f);
+}
+__device__ __forceinline__ float sigmoid_f(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + fast_exp(-x));
+}
+// gelu(x) = x * Phi(x) with Phi from Abramowitz & Stegun 7.1.26
+//   erfc(z) = (a1 t + ... + a5 t^5) exp(-z^2),  t = 1 / (1 + 0.3275911 z),  z >= 0
+// (|error| <= 1.5e-7, the level of fp32 rounding).  With z = |x| / sqrt(2) and
+// q = erfc(z) / 2:   gelu(x) = x - x q  for x >= 0  and  x q  for x < 0,
+// i.e. max(x, 0) - |x| q.  One reciprocal and one exp2 per value.
 __device__ __forceinline__ float gelu_erf(float x) {
-  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+  const float ax = fabsf(x);
+  const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f * 0.70710678118654752440f, ax, 1.0f));
+  float poly = fmaf(0.5f * 1.061405429f, t, 0.5f * -1.453152027f);
+  poly = fmaf(poly, t, 0.5f * 1.421413741f);
+  poly = fmaf(poly, t, 0.5f * -0.284496736f);
+  poly = fmaf(poly, t, 0.5f * 0.254829592f);
+  poly *= t;
+  const float q = poly * __builtin_amdgcn_exp2f((x * (-0.5f * 1.4426950408889634f)) * x);
+  return fmaf(-ax, q, fmaxf(x, 0.0f));
 }
 __device__ __forceinline__ float gelu_tanh(float x) {
-  return 0.5f * x * (1.0f + tanhf(0.79788456080286535588f * (x + 0.044715f * x * x * x)));
+  // 0.5 x (1 + tanh(u)) = x * sigmoid(2u),  u = sqrt(2/pi) (x + 0.044715 x^3)
+  const float u = 0.79788456080286535588f * fmaf(0.044715f * x * x, x, x);
+  return x * sigmoid_f(2.0f * u);
 }
 template <bool kFastGelu>
 __device__ __forceinline__ float gelu(float x) {
@@ -46,15 +71,22 @@ struct LstmParams {
   int64_t pc_stride;
   int64_t out_stride;
   int D;
+  float inv_D;        // 1 / D
   float alpha;
   float eps_cell;
   float eps_state;
 };
 
-template <typename T, int kChunksPerThread, bool kFastGelu>
-__global__ __launch_bounds__(1024) void sum_lstm_vec_kernel(const LstmParams p) {
+// Loads are issued in the order in which the arithmetic needs them - cell gate,
+// forget gate, previous cell, input gate, output gate - and memory returns them
+// in that order, so the first row sum, the candidate GELU and the early sigmoids
+// run while the later gates are still on their way, and only one sigmoid, one
+// multiply and the store remain after the last load has landed.
+template <typename T, int kChunksPerThread, bool kFastGelu, int kMaxThreads>
+__global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmParams p) {
   __shared__ float slots_cpre[16];
   __shared__ float slots_cnew[16];
+  constexpr int K = kChunksPerThread;
   const int D = p.D;
   const int chunks = D >> 3;
   const int64_t row = blockIdx.x;
@@ -65,96 +97,129 @@ __global__ __launch_bounds__(1024) void sum_lstm_vec_kernel(const LstmParams p) 
   char *oc_row = p.out_cell + row * p.out_stride * 2;
   char *os_row = p.out_state + row * p.out_stride * 2;
 
-  uint4 s[kChunksPerThread][4], z[kChunksPerThread][4], pc[kChunksPerThread];
+  bool live[K];
+  int64_t off[K];
+  uint4 sc[K], zc[K], sf[K], zf[K], si[K], zi[K], pc[K], so[K], zo[K];
+  uint4 wc[K], bc[K], ws[K], bs[K];
 #pragma unroll
-  for (int k = 0; k < kChunksPerThread; ++k) {
+  for (int k = 0; k < K; ++k) {
     const int c = threadIdx.x + k * blockDim.x;
-    const int64_t off = (int64_t)c * 16;
+    live[k] = c < chunks;
+    off[k] = (int64_t)(live[k] ? c : 0) * 16;  // idle lanes re-read chunk 0 and discard it
+  }
+  // The scale / shift vectors are the same for every row (cache resident).  They
+  // are requested first: memory returns loads in issue order, so asking for them
+  // later would park the arithmetic behind the whole row.
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      s[k][g] = make_uint4(0, 0, 0, 0);
-      z[k][g] = make_uint4(0, 0, 0, 0);
-    }
-    pc[k] = make_uint4(0, 0, 0, 0);
-    if (c < chunks) {
-      // cell gate first: the first reduction only needs it
-      s[k][3] = load16_stream(s_row + 3 * gate_bytes + off);
-      z[k][3] = load16_stream(z_row + 3 * gate_bytes + off);
+  for (int k = 0; k < K; ++k) {
+    if (p.w_cell) wc[k] = load16(p.w_cell + off[k]);
+    if (p.b_cell) bc[k] = load16(p.b_cell + off[k]);
+    if (p.w_state) ws[k] = load16(p.w_state + off[k]);
+    if (p.b_state) bs[k] = load16(p.b_state + off[k]);
+  }
 #pragma unroll
-      for (int g = 0; g < 3; ++g) {
-        s[k][g] = load16_stream(s_row + g * gate_bytes + off);
-        z[k][g] = load16_stream(z_row + g * gate_bytes + off);
-      }
-      pc[k] = load16_stream(pc_row + off);
-    }
+  for (int k = 0; k < K; ++k) {
+    sc[k] = load16_stream(s_row + 3 * gate_bytes + off[k]);
+    zc[k] = load16_stream(z_row + 3 * gate_bytes + off[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    sf[k] = load16_stream(s_row + off[k]);
+    zf[k] = load16_stream(z_row + off[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < K; ++k) pc[k] = load16_stream(pc_row + off[k]);
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    si[k] = load16_stream(s_row + gate_bytes + off[k]);
+    zi[k] = load16_stream(z_row + gate_bytes + off[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    so[k] = load16_stream(s_row + 2 * gate_bytes + off[k]);
+    zo[k] = load16_stream(z_row + 2 * gate_bytes + off[k]);
   }
 
-  // phase 1: pre_c and its sum of squares (reference :65-82)
-  float cpre[kChunksPerThread][8];
+  // Lanes beyond the row take part in the sums with zeros.  (Each value is
+  // cleared where it is first used, not here: touching pc now would wait for it.)
+  // phase 1: pre_c and its sum of squares (reference :65-82); needs the cell gate only
+  float cact[K][8];
   float ss = 0.f;
 #pragma unroll
-  for (int k = 0; k < kChunksPerThread; ++k) {
+  for (int k = 0; k < K; ++k) {
     float a[8], b[8];
-    unpack8<T>(s[k][3], a);
-    unpack8<T>(z[k][3], b);
+    if (!live[k]) sc[k] = zc[k] = make_uint4(0, 0, 0, 0);
+    unpack8<T>(sc[k], a);
+    unpack8<T>(zc[k], b);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      cpre[k][j] = a[j] + p.alpha * b[j];
-      ss += cpre[k][j] * cpre[k][j];
+      cact[k][j] = fmaf(p.alpha, b[j], a[j]);
+      ss = fmaf(cact[k][j], cact[k][j], ss);
     }
   }
-  const float inv_cpre = rsqrtf(block_sum(ss, slots_cpre) / (float)D + p.eps_cell);
-
-  // phase 2: gates f, i; cell update; write out_cell (reference :104-140)
-  float cell[kChunksPerThread][8];  // the ROUNDED new cell, as the state phase must see it
-  ss = 0.f;
+  const float inv_cpre = rsqrtf(block_sum(ss, slots_cpre) * p.inv_D + p.eps_cell);
+  // candidate = gelu(rmsnorm(pre_c)): runs while the other gates are still arriving
 #pragma unroll
-  for (int k = 0; k < kChunksPerThread; ++k) {
-    const int c = threadIdx.x + k * blockDim.x;
-    const bool live = c < chunks;
-    float sf[8], zf[8], si[8], zi[8], pcv[8], w[8], b[8];
-    unpack8<T>(s[k][0], sf);
-    unpack8<T>(z[k][0], zf);
-    unpack8<T>(s[k][1], si);
-    unpack8<T>(z[k][1], zi);
-    unpack8<T>(pc[k], pcv);
-    if (p.w_cell && live) unpack8<T>(load16(p.w_cell + (int64_t)c * 16), w);
-    if (p.b_cell && live) unpack8<T>(load16(p.b_cell + (int64_t)c * 16), b);
+  for (int k = 0; k < K; ++k) {
+    float w[8], b[8];
+    if (p.w_cell) unpack8<T>(wc[k], w);
+    if (p.b_cell) unpack8<T>(bc[k], b);
+    const float mask = live[k] ? 1.f : 0.f;  // idle lanes must add nothing to the second sum
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const float fgate = sigmoid_f(sf[j] + p.alpha * zf[j]);
-      const float igate = sigmoid_f(si[j] + p.alpha * zi[j]);
-      float cn = cpre[k][j] * inv_cpre;
+      float cn = cact[k][j] * inv_cpre;
       if (p.w_cell) cn *= w[j];
       if (p.b_cell) cn += b[j];
-      const float cnew = live ? pcv[j] * fgate + gelu<kFastGelu>(cn) * igate : 0.f;
-      ss += cnew * cnew;  // unrounded, as in the reference (:136)
+      cact[k][j] = gelu<kFastGelu>(cn) * mask;
+    }
+  }
+
+  // phase 2: cell update; write out_cell (reference :104-140)
+  float cell[K][8];  // ends up as the ROUNDED new cell, as the state phase must see it
+  ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    float a[8], b[8], c[8];
+    unpack8<T>(sf[k], a);
+    unpack8<T>(zf[k], b);
+    if (!live[k]) pc[k] = make_uint4(0, 0, 0, 0);
+    unpack8<T>(pc[k], c);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) cell[k][j] = sigmoid_f(fmaf(p.alpha, b[j], a[j])) * c[j];
+    unpack8<T>(si[k], a);
+    unpack8<T>(zi[k], b);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float cnew = fmaf(cact[k][j], sigmoid_f(fmaf(p.alpha, b[j], a[j])), cell[k][j]);
+      ss = fmaf(cnew, cnew, ss);  // unrounded, as in the reference (:136)
       cell[k][j] = cnew;
     }
     const uint4 packed = pack8<T>(cell[k]);
-    if (live) store16_stream(oc_row + (int64_t)c * 16, packed);
+    if (live[k]) store16_stream(oc_row + off[k], packed);
     unpack8<T>(packed, cell[k]);
   }
-  const float inv_cnew = rsqrtf(block_sum(ss, slots_cnew) / (float)D + p.eps_state);
+  const float inv_cnew = rsqrtf(block_sum(ss, slots_cnew) * p.inv_D + p.eps_state);
 
-  // phase 3: state = gelu(rmsnorm(rounded cell)) * sigmoid(pre_o) (reference :160-190)
+  // phase 3: state = gelu(rmsnorm(rounded cell)) * sigmoid(pre_o) (reference :160-190);
+  // the output gate is the last load to arrive and is consumed last
 #pragma unroll
-  for (int k = 0; k < kChunksPerThread; ++k) {
-    const int c = threadIdx.x + k * blockDim.x;
-    if (c >= chunks) continue;
-    float so[8], zo[8], w[8], b[8], st[8];
-    unpack8<T>(s[k][2], so);
-    unpack8<T>(z[k][2], zo);
-    if (p.w_state) unpack8<T>(load16(p.w_state + (int64_t)c * 16), w);
-    if (p.b_state) unpack8<T>(load16(p.b_state + (int64_t)c * 16), b);
+  for (int k = 0; k < K; ++k) {
+    float w[8], b[8], st[8];
+    if (p.w_state) unpack8<T>(ws[k], w);
+    if (p.b_state) unpack8<T>(bs[k], b);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       float cn = cell[k][j] * inv_cnew;
       if (p.w_state) cn *= w[j];
       if (p.b_state) cn += b[j];
-      st[j] = gelu<kFastGelu>(cn) * sigmoid_f(so[j] + p.alpha * zo[j]);
+      st[j] = gelu<kFastGelu>(cn);
     }
-    store16_stream(os_row + (int64_t)c * 16, pack8<T>(st));
+    float a[8], g[8];
+    unpack8<T>(so[k], a);
+    unpack8<T>(zo[k], g);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) st[j] *= sigmoid_f(fmaf(p.alpha, g[j], a[j]));
+    if (live[k]) store16_stream(os_row + off[k], pack8<T>(st));
   }
 }
 
@@ -179,7 +244,7 @@ __global__ __launch_bounds__(256) void sum_lstm_scalar_kernel(const LstmParams p
     const float c = T::lo(s[3 * (int64_t)D + j]) + p.alpha * T::lo(z[3 * (int64_t)D + j]);
     ss += c * c;
   }
-  const float inv_cpre = rsqrtf(block_sum(ss, slots_cpre) / (float)D + p.eps_cell);
+  const float inv_cpre = rsqrtf(block_sum(ss, slots_cpre) * p.inv_D + p.eps_cell);
 
   ss = 0.f;
   for (int j = threadIdx.x; j < D; j += blockDim.x) {
@@ -193,7 +258,7 @@ __global__ __launch_bounds__(256) void sum_lstm_scalar_kernel(const LstmParams p
     ss += cnew * cnew;
     oc[j] = (uint16_t)T::round_bits(cnew);
   }
-  const float inv_cnew = rsqrtf(block_sum(ss, slots_cnew) / (float)D + p.eps_state);
+  const float inv_cnew = rsqrtf(block_sum(ss, slots_cnew) * p.inv_D + p.eps_state);
 
   // each thread re-reads only the out_cell elements it wrote itself
   for (int j = threadIdx.x; j < D; j += blockDim.x) {
@@ -219,13 +284,22 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
                    aligned16(p.b_cell) && aligned16(p.w_state) && aligned16(p.b_state);
   const dim3 grid((unsigned)rows);
   if (vec) {
-    const int cpt = chunks > 1024 ? 2 : 1;
+    // one 16-byte chunk per lane up to 512 lanes (D <= 4096), two beyond that
+    int cpt = chunks > 512 ? 2 : 1;
+#ifdef ARCTIC_TUNING
+    if (const char *e = getenv("ARCTIC_LSTM_CPT")) cpt = atoi(e) == 2 ? 2 : 1;
+#endif
+    if (cpt == 1 && chunks > 1024) cpt = 2;
     int threads = (chunks + cpt - 1) / cpt;
     threads = std::max(64, (threads + 63) & ~63);
-    if (cpt == 1)
-      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 1, kFastGelu>), grid, dim3(threads), 0, s, p);
+    if (cpt == 1 && threads <= 512)
+      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 1, kFastGelu, 512>), grid, dim3(threads), 0, s, p);
+    else if (cpt == 1)
+      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 1, kFastGelu, 1024>), grid, dim3(threads), 0, s, p);
+    else if (threads <= 256)
+      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 2, kFastGelu, 256>), grid, dim3(threads), 0, s, p);
     else
-      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 2, kFastGelu>), grid, dim3(threads), 0, s, p);
+      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 2, kFastGelu, 1024>), grid, dim3(threads), 0, s, p);
   } else {
     hipLaunchKernelGGL((sum_lstm_scalar_kernel<T, kFastGelu>), grid, dim3(256), 0, s, p);
   }
@@ -264,6 +338,7 @@ extern "C" int arctic_sum_lstm(void *out_state, void *out_cell, const void *stat
   p.pc_stride = pc_stride;
   p.out_stride = out_stride;
   p.D = D;
+  p.inv_D = 1.0f / (float)D;
   p.alpha = alpha;
   p.eps_cell = eps_cell;
   p.eps_state = eps_state;

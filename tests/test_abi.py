@@ -1,0 +1,90 @@
+"""The C-ABI library: loads without a GPU, exports exactly what include/arctic_mi355x.h
+declares, depends on no torch library, and rejects bad arguments before any launch."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+from arcticinference_amd import _native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "arctic_mi355x.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)          # drop comments
+    return sorted(set(re.findall(r"\b(arctic_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    path = _native.library_path()
+    assert path is not None, "libarctic_mi355x.so is not built (python -c 'import __graft_entry__ as g; g.build()')"
+    return _native.load()
+
+
+def test_header_and_binding_list_agree():
+    assert declared_functions() == sorted(_native.EXPORTED_SYMBOLS)
+
+
+def test_every_declared_symbol_is_exported(lib):
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported"
+    out = subprocess.run(["nm", "-D", "--defined-only", _native.library_path()], capture_output=True, text=True).stdout
+    exported_c = {l.split()[-1] for l in out.splitlines() if " T " in l and not l.split()[-1].startswith("_Z")}
+    assert set(declared_functions()) <= exported_c
+
+
+def test_abi_version_matches_header(lib):
+    m = re.search(r"#define\s+ARCTIC_ABI_VERSION\s+(\d+)", open(HEADER).read())
+    assert lib.arctic_abi_version() == int(m.group(1)) == _native.ABI_VERSION
+
+
+def test_no_torch_dependency():
+    out = subprocess.run(["ldd", _native.library_path()], capture_output=True, text=True).stdout
+    assert "torch" not in out and "c10" not in out and "python" not in out.lower()
+    assert "amdhip64" in out
+
+
+def test_header_compiles_as_plain_c(tmp_path):
+    src = tmp_path / "t.c"
+    src.write_text('#include "arctic_mi355x.h"\nint main(void) { return ARCTIC_ABI_VERSION == 1 ? 0 : 1; }\n')
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), "-c", str(src), "-o",
+                    str(tmp_path / "t.o")], check=True)
+
+
+def test_argument_errors_return_codes_without_launching(lib):
+    # every call below fails validation, so nothing is enqueued and no GPU is needed
+    rc = lib.arctic_speculator_ln(None, None, None, None, 4, 128, 128, 1e-6, _native.DTYPE_F32, None)
+    assert rc == 2 and b"only fp16 and bf16" in lib.arctic_last_error()
+    rc = lib.arctic_speculator_ln(None, None, None, None, 4, 0, 0, 1e-6, _native.DTYPE_BF16, None)
+    assert rc == 1 and b"hidden size must be > 0" in lib.arctic_last_error()
+    rc = lib.arctic_speculator_ln(None, None, None, None, 4, 128, 128, 1e-6, _native.DTYPE_BF16, None)
+    assert rc == 1 and b"null" in lib.arctic_last_error()
+    rc = lib.arctic_sum_lstm(*([None] * 9), 4, 64, 256, 256, 64, 64, 1.0, 1e-6, 1e-6, 0, _native.DTYPE_F32, None)
+    assert rc == 2 and b"sum_lstm: only fp16 and bf16" in lib.arctic_last_error()
+    rc = lib.arctic_reshape_and_cache_flash_bulk(None, None, 0, 0, None, None, None, None, None, 4, 2, 2, 64, 16, 0,
+                                                 _native.DTYPE_BF16, 7, None)
+    assert rc == 2 and b"Unsupported data type of kv cache" in lib.arctic_last_error()
+    rc = lib.arctic_reshape_and_cache_flash_bulk(None, None, 0, 0, None, None, None, None, None, 4, 2, 2, 64, 16, 0,
+                                                 9, _native.KV_AUTO, None)
+    assert rc == 2 and b"Unsupported input type of kv cache" in lib.arctic_last_error()
+    rc = lib.arctic_reshape_and_cache_flash_bulk(None, None, 0, 0, None, None, None, None, None, 4, 100000, 2, 64, 16,
+                                                 0, _native.DTYPE_BF16, _native.KV_AUTO, None)
+    assert rc == 1 and b"num_layers" in lib.arctic_last_error()
+    # empty problems are successful no-ops (reference: reshape_and_cache_flash_bulk.cu:87-89)
+    assert lib.arctic_reshape_and_cache_flash_bulk(None, None, 0, 0, None, None, None, None, None, 4, 0, 2, 64, 16, 0,
+                                                   _native.DTYPE_BF16, _native.KV_AUTO, None) == 0
+    assert lib.arctic_speculator_ln(None, None, None, None, 0, 128, 128, 1e-6, _native.DTYPE_BF16, None) == 0
+
+
+def test_product_never_touches_the_oracle():
+    pkg = os.path.join(ROOT, "arcticinference_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".cpp", ".h")) or f == "Makefile":
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower(), f"{f} mentions the oracle"

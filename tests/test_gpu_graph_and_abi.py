@@ -1,0 +1,132 @@
+"""HIP-graph capture of the whole path and direct calls into the C ABI."""
+import ctypes
+
+import pytest
+import torch
+
+import oracle
+from arcticinference_amd import _native
+from helpers import (assert_bulk_equal, assert_close, bulk_args, bulk_case_to, make_bulk_case, make_lstm_case,
+                     speculator_alpha)
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def test_decode_step_in_one_graph(ops):
+    """BASELINE config 5 in miniature: bulk fp8 KV write, ln0 (no affine) and three chained
+    sum_lstm steps captured as one graph.  The graph is replayed several times with eager
+    work and synchronisation in between; every replay must equal the eager result and
+    the oracle."""
+    T, D = 64, 1024
+    case = make_bulk_case(T=T, L=4, H=8, D=128, bs=16, NB=16, kv_cache_dtype="fp8", seed=4, std=1.5)
+    dcase = bulk_case_to(case, DEV)
+    steps = [make_lstm_case(rows=T, D=D, seed=40 + k) for k in range(3)]
+    dsteps = [{k: (None if v is None else v.to(DEV)) for k, v in s.items()} for s in steps]
+    g = torch.Generator().manual_seed(44)
+    x = torch.randn(T, D, generator=g).to(torch.bfloat16)
+    dx = x.to(DEV)
+    alpha = speculator_alpha(3, D)
+
+    def step():
+        ops.reshape_and_cache_flash_bulk(*bulk_args(dcase))
+        h = ops.speculator_ln(dx, None, None, 1e-6)
+        cell = torch.zeros(T, D, dtype=torch.bfloat16, device=DEV)
+        states = []
+        for s in dsteps:
+            st, cell = ops.sum_lstm(s["states"], s["z4"], cell, s["w_cell"], s["b_cell"], s["w_state"], s["b_state"],
+                                    alpha, 1e-6, 1e-6, False)
+            states.append(st)
+        return h, states, cell
+
+    # oracle
+    oracle.reshape_and_cache_flash_bulk(*bulk_args(case))
+    want_h = oracle.speculator_ln(x, None, None, 1e-6)
+
+    sentinel = [b.clone() for b in dcase["bufs"]]
+    eager_h, eager_states, eager_cell = step()
+    torch.cuda.synchronize()
+    assert_bulk_equal(dcase["bufs"], case["bufs"])
+    assert_close(eager_h, want_h, what="ln0")
+    cell = torch.zeros(T, D, dtype=torch.bfloat16)
+    for k, s in enumerate(steps):
+        # chain through the GPU's own cell so that only this step's arithmetic is compared
+        prev = cell
+        want_st, want_cell = oracle.sum_lstm(s["states"], s["z4"], prev, s["w_cell"], s["b_cell"], s["w_state"],
+                                             s["b_state"], alpha, 1e-6, 1e-6, False)
+        assert_close(eager_states[k], want_st, what=f"state {k}")
+        cell = want_cell
+    eager = [eager_h.clone()] + [s.clone() for s in eager_states] + [eager_cell.clone()]
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        gh, gstates, gcell = step()
+    for replay in range(4):
+        for b, s in zip(dcase["bufs"], sentinel):
+            b.copy_(s)                       # eager work between replays: restore the untouched caches
+        gh.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_bulk_equal(dcase["bufs"], case["bufs"])
+        got = [gh] + list(gstates) + [gcell]
+        for a, b in zip(got, eager):
+            assert torch.equal(a, b), f"replay {replay} differs from the eager run"
+
+
+def test_direct_c_abi_calls(ops):
+    """Raw pointers straight into libarctic_mi355x.so (what another host language would do)."""
+    lib = _native.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator().manual_seed(12)
+    rows, hidden = 10, 512
+    x = torch.randn(rows, hidden, generator=g).to(torch.float16)
+    w = torch.randn(hidden, generator=g).to(torch.float16)
+    dx, dw = x.to(DEV), w.to(DEV)
+    out = torch.empty_like(dx)
+    rc = lib.arctic_speculator_ln(out.data_ptr(), dx.data_ptr(), dw.data_ptr(), None, rows, hidden, hidden, 1e-6,
+                                  _native.DTYPE_F16, stream)
+    assert rc == 0, lib.arctic_last_error()
+    torch.cuda.synchronize()
+    assert_close(out, oracle.speculator_ln(x, w, None, 1e-6), what="ln via C ABI")
+
+    case = make_bulk_case(T=20, L=3, H=2, D=64, bs=8, NB=4, kv_cache_dtype="fp8", seed=13, std=1.5, pad_fraction=0.2)
+    d = bulk_case_to(case, DEV)
+    L = 3
+    tab = lambda ts: (ctypes.c_void_p * L)(*[t.data_ptr() for t in ts])
+    rc = lib.arctic_reshape_and_cache_flash_bulk(
+        d["keys"].data_ptr(), d["values"].data_ptr(), d["keys"].stride(0), d["values"].stride(0),
+        tab(d["key_caches"]), tab(d["value_caches"]), tab(d["k_scales"]), tab(d["v_scales"]),
+        d["slot_mapping"].data_ptr(), 20, L, 2, 64, 8, d["key_caches"][0].stride(0), _native.DTYPE_BF16,
+        _native.KV_FP8_E4M3, stream)
+    assert rc == 0, lib.arctic_last_error()
+    torch.cuda.synchronize()
+    oracle.reshape_and_cache_flash_bulk(*bulk_args(case))
+    assert_bulk_equal(d["bufs"], case["bufs"])
+
+    c = make_lstm_case(rows=5, D=256, seed=14)
+    dc = {k: (None if v is None else v.to(DEV)) for k, v in c.items()}
+    st, ce = torch.empty(5, 256, dtype=torch.bfloat16, device=DEV), torch.empty(5, 256, dtype=torch.bfloat16, device=DEV)
+    rc = lib.arctic_sum_lstm(st.data_ptr(), ce.data_ptr(), dc["states"].data_ptr(), dc["z4"].data_ptr(),
+                             dc["prev_cell"].data_ptr(), dc["w_cell"].data_ptr(), dc["b_cell"].data_ptr(),
+                             dc["w_state"].data_ptr(), dc["b_state"].data_ptr(), 5, 256, 1024, 1024, 256, 256, 0.35,
+                             1e-6, 1e-6, 0, _native.DTYPE_BF16, stream)
+    assert rc == 0, lib.arctic_last_error()
+    torch.cuda.synchronize()
+    wst, wce = oracle.sum_lstm(c["states"], c["z4"], c["prev_cell"], c["w_cell"], c["b_cell"], c["w_state"],
+                               c["b_state"], 0.35, 1e-6, 1e-6, False)
+    assert_close(st, wst, what="state via C ABI")
+    assert_close(ce, wce, what="cell via C ABI")
+
+
+def test_side_stream(ops):
+    """The shim launches on torch's current stream, whichever that is."""
+    g = torch.Generator().manual_seed(15)
+    x = torch.randn(64, 2048, generator=g).to(torch.bfloat16)
+    dx = x.to(DEV)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        y = ops.speculator_ln(dx, None, None, 1e-6)
+    s.synchronize()
+    assert_close(y, oracle.speculator_ln(x, None, None, 1e-6), what="ln on a side stream")

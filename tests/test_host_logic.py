@@ -1,0 +1,98 @@
+"""Host side of the drop-in operator surface (runs without a GPU)."""
+import re
+
+import pytest
+import torch
+
+from arcticinference_amd import _native, py_custom_ops as ops
+
+# The schemas the reference registers (csrc/custom_ops/torch_bindings.cpp:7-49), whitespace-normalised.
+REFERENCE_SCHEMAS = {
+    "reshape_and_cache_flash_bulk":
+        "arctic_inference::reshape_and_cache_flash_bulk(Tensor keys, Tensor values, Tensor(c!)[] key_caches, "
+        "Tensor(d!)[] value_caches, Tensor slot_mapping, str kv_cache_dtype, Tensor(e)[] k_scales, "
+        "Tensor(f)[] v_scales, int num_heads, int head_size) -> ()",
+    "reshape_and_cache_flash_fp4":
+        "arctic_inference::reshape_and_cache_flash_fp4(Tensor key, Tensor value, Tensor(c!) key_cache, "
+        "Tensor(d!) value_cache, Tensor slot_mapping, str kv_cache_dtype, Tensor k_scale, Tensor v_scale, "
+        "Tensor(e!) key_scale_cache, Tensor(f!) value_scale_cache) -> ()",
+    "speculator_ln_cuda":
+        "arctic_inference::speculator_ln_cuda(Tensor input, Tensor? weight, Tensor? bias, float eps) -> Tensor",
+    "sum_lstm_cuda":
+        "arctic_inference::sum_lstm_cuda(Tensor states_4d, Tensor z4_4d, Tensor prev_cell_d, Tensor? w_cell, "
+        "Tensor? b_cell, Tensor? w_state, Tensor? b_state, float alpha, float eps_cell, float eps_state, "
+        "bool use_fast_gelu) -> (Tensor, Tensor)",
+}
+
+
+@pytest.fixture(scope="module")
+def loaded():
+    assert ops.try_load_torch_library(), "libarctic_mi355x.so is not built"
+    return ops
+
+
+def test_load_is_idempotent(loaded):
+    assert ops.try_load_torch_library() and ops.try_load_torch_library()
+    assert _native.is_loaded() and _native.loaded_path().endswith(".so")
+
+
+def test_schemas_match_the_reference(loaded):
+    for name, want in REFERENCE_SCHEMAS.items():
+        got = str(getattr(torch.ops.arctic_inference, name).default._schema)
+        assert re.sub(r"\s+", " ", got) == want
+
+
+def test_no_cpu_backend_and_no_fallback(loaded):
+    x = torch.randn(4, 64, dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError, match="CPU"):
+        ops.speculator_ln(x, None, None, 1e-6)
+    with pytest.raises(NotImplementedError, match="CPU"):
+        ops.sum_lstm(torch.randn(4, 256).bfloat16(), torch.randn(4, 256).bfloat16(), x, None, None, None, None, 1.0,
+                     1e-6, 1e-6, False)
+    with pytest.raises(NotImplementedError, match="CPU"):
+        ops.reshape_and_cache_flash_bulk(x, x, [x], [x], torch.zeros(4, dtype=torch.int64), "auto", [x], [x], 1, 64)
+
+
+def test_argument_checks_mirror_the_reference(loaded):
+    # the shims run the reference's TORCH_CHECKs before touching the device, so the
+    # ones that precede the device check can be exercised with CPU tensors
+    x32 = torch.randn(4, 64)
+    with pytest.raises(RuntimeError, match="speculator_ln: only fp16 and bf16 are supported."):
+        ops._speculator_ln_impl(x32, None, None, 1e-6)
+    with pytest.raises(RuntimeError, match="speculator_ln: input must be CUDA"):
+        ops._speculator_ln_impl(x32.bfloat16(), None, None, 1e-6)
+    with pytest.raises(RuntimeError, match="sum_lstm: only fp16 and bf16 are supported."):
+        ops._sum_lstm_impl(x32, x32, x32, None, None, None, None, 1.0, 1e-6, 1e-6, False)
+    with pytest.raises(RuntimeError, match="sum_lstm: inputs must be CUDA tensors"):
+        ops._sum_lstm_impl(x32.half(), x32.half(), x32.half(), None, None, None, None, 1.0, 1e-6, 1e-6, False)
+    with pytest.raises(RuntimeError, match="Unsupported data type of kv cache: nvfp4"):
+        ops._kv_dtype_code(torch.bfloat16, "nvfp4")
+    with pytest.raises(RuntimeError, match="Unsupported input type of kv cache"):
+        ops._kv_dtype_code(torch.int8, "auto")
+    assert ops._kv_dtype_code(torch.float16, "fp8") == (_native.DTYPE_F16, _native.KV_FP8_E4M3)
+    assert ops._kv_dtype_code(torch.float32, "fp8_e4m3") == (_native.DTYPE_F32, _native.KV_FP8_E4M3)
+    assert ops._kv_dtype_code(torch.bfloat16, "fp8_e5m2") == (_native.DTYPE_BF16, _native.KV_FP8_E5M2)
+    assert ops._kv_dtype_code(torch.bfloat16, "auto") == (_native.DTYPE_BF16, _native.KV_AUTO)
+    # empty layer list is a no-op (reference :87-89), mismatched list lengths are an error (:91-94)
+    ops._reshape_and_cache_flash_bulk_impl(x32, x32, [], [], torch.zeros(4, dtype=torch.int64), "auto", [], [], 1, 64)
+    with pytest.raises(RuntimeError, match="value_caches"):
+        ops._reshape_and_cache_flash_bulk_impl(x32, x32, [x32], [], torch.zeros(4, dtype=torch.int64), "auto", [x32],
+                                               [x32], 1, 64)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    """Without the shared object: try_load returns False (as the reference does) and the
+    operators raise; nothing falls back to another implementation."""
+    monkeypatch.setattr(_native, "library_path", lambda: None)
+    monkeypatch.setattr(_native, "_lib", None)
+    monkeypatch.setattr(ops, "_registered", False)
+    assert ops.try_load_torch_library() is False
+    x = torch.randn(4, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="not loaded"):
+        ops.speculator_ln(x, None, None, 1e-6)
+    with pytest.raises(RuntimeError, match="not loaded"):
+        ops.sum_lstm(x, x, x, None, None, None, None, 1.0, 1e-6, 1e-6, False)
+    with pytest.raises(RuntimeError, match="not loaded"):
+        ops.reshape_and_cache_flash_bulk(x, x, [x], [x], torch.zeros(4, dtype=torch.int64), "auto", [x], [x], 1, 64)
+    with pytest.raises(RuntimeError, match="not found"):
+        _native.load()

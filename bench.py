@@ -98,6 +98,19 @@ def event_times_us(fn, iters):
     return [s.elapsed_time(e) * 1e3 for s, e in zip(starts, ends)]
 
 
+def read_traffic(path):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by
+    a copy kernel of known size); the figure is kept next to the profile it came from."""
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.strip().startswith("hbm_bytes_per_launch"):
+                    return int(float(line.split("=")[1].split()[0]))
+    except OSError:
+        pass
+    return None
+
+
 def cpu_baseline_bulk(w: BulkWorkload, target_seconds=6.0):
     """Time the CPU oracle on a sample of the workload's tokens (all layers)."""
     import oracle
@@ -235,6 +248,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extras", action="store_true", help="skip the speculator / decode-mix measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (known bytes) so that a counter run of this "
+                         "command can scale FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path is built and measured on ONE GPU (every token, layer and row is "
@@ -265,11 +281,14 @@ def main():
     us = event_times_us(fn, args.steps)
     kernel_us = statistics.mean(us)
     achieved = w.bytes / kernel_us / 1e3
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
-        with open(tpath) as f:
-            traffic = json.load(f).get("kv_write_bulk_fp8_70b", {}).get("hbm_bytes_per_launch")
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    traffic = read_traffic(os.path.join(ROOT, "profiles", "kv_write_bulk_fp8_70b.traffic.txt"))
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "kernel": "kv_write_bulk_kernel<bf16, e4m3>", "kernel_us_mean": round(kernel_us, 2),

@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one bulk KV-cache write (one launch of the hot path) over the 70B
-SwiftKV shape of BASELINE.json (configs[2]): 16384 tokens, 40 layers, 8 KV heads
+SwiftKV shape (the benchmark's headline workload): 16384 tokens, 40 layers, 8 KV heads
 x 128, block 16, fp8-e4m3 cache with per-tensor amax/448 scales, 10 % of the
 slots are padding.  Inputs are resident in HBM before the timed region.  The
 last stdout line is ONE JSON object:
@@ -14,7 +14,7 @@ last stdout line is ONE JSON object:
                         stream it is launched on, against the 8 TB/s HBM peak
   cpu_baseline          the CPU oracle (a C port of the reference kernel, OpenMP)
                         timed on this machine's host cores on a bounded sample
-  extras                the other BASELINE configs (speculator ops, decode mix)
+  extras                the other workloads (8B prefill chunk, speculator ops, decode mix)
 
 Only one GPU is used; --gpus N with N > 1 is refused.
 """
@@ -148,7 +148,7 @@ def cpu_baseline_bulk(w: BulkWorkload, target_seconds=6.0):
 
 
 def bench_speculator(ops, dev, steps, warmup):
-    """BASELINE config 4: sum_lstm (3 chained steps) and the standalone LayerNorm at
+    """Speculator workload: sum_lstm (3 chained steps) and the standalone LayerNorm at
     T=512, H=4096, bf16.  Eight buffer sets (> 256 MB in total) are rotated so that
     the inputs do not stay resident in the last-level cache between launches."""
     T, Hd, sets = 512, 4096, 8
@@ -199,7 +199,7 @@ def bench_speculator(ops, dev, steps, warmup):
 
 
 def bench_decode_mix(ops, dev, steps):
-    """BASELINE config 5: 512 decode tokens; bulk fp8 KV write over 16 layers into
+    """Decode-step workload: 512 decode tokens; bulk fp8 KV write over 16 layers into
     32768-block caches, ln0, three sum_lstm steps; one HIP graph per step."""
     w = BulkWorkload("decode", 512, 16, 8, 128, 16, 32768, "fp8", 0.0, 4, 1.5, dev)
     T, Hd = 512, 4096
@@ -321,7 +321,7 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "fp8_e4m3",
         "data": "synthetic",
-        "config": {"workload": "BASELINE configs[2]: bulk KV write, 16384 tokens x 40 layers x 8 KV heads x 128, "
+        "config": {"workload": "bulk KV write at the 70B SwiftKV shape: 16384 tokens x 40 layers x 8 KV heads x 128, "
                                "block 16, 8192 blocks, fp8-e4m3 cache, amax/448 scales, 10% slots = -1",
                    "tokens": w.T, "valid_tokens": w.valid, "layers": w.L, "kv_heads": w.H, "head_size": w.D,
                    "block_size": w.bs, "num_blocks": w.NB, "parallelism": "single GPU"},

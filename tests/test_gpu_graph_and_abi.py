@@ -14,7 +14,7 @@ DEV = "cuda:0"
 
 
 def test_decode_step_in_one_graph(ops):
-    """BASELINE config 5 in miniature: bulk fp8 KV write, ln0 (no affine) and three chained
+    """The decode-step workload in miniature: bulk fp8 KV write, ln0 (no affine) and three chained
     sum_lstm steps captured as one graph.  The graph is replayed several times with eager
     work and synchronisation in between; every replay must equal the eager result and
     the oracle."""

@@ -23,7 +23,7 @@ def run_both(ops, case):
 
 
 def test_config1_bf16_passthrough(ops):
-    # BASELINE config 1: 256 tokens, 16 layers, 8 KV heads x 128, block 16, 512 blocks, bf16 cache
+    # the CPU-runnable benchmark shape: 256 tokens, 16 layers, 8 KV heads x 128, block 16, 512 blocks, bf16 cache
     case = make_bulk_case(T=256, L=16, H=8, D=128, bs=16, NB=512, seed=0)
     run_both(ops, case)
 
@@ -143,13 +143,13 @@ def test_fp8_from_fp32_rounding_boundaries(ops):
 
 
 def test_config2_fp8_prefill_chunk(ops):
-    # BASELINE config 2: 8192 tokens, 16 layers, fp8 cache with amax/448 scales
+    # the 8B prefill-chunk shape: 8192 tokens, 16 layers, fp8 cache with amax/448 scales
     case = make_bulk_case(T=8192, L=16, H=8, D=128, bs=16, NB=8192, kv_cache_dtype="fp8", seed=1, std=1.5)
     run_both(ops, case)
 
 
 def test_config3_shape_properties(ops):
-    """BASELINE config 3 at full size (16384 tokens, 40 layers, 10 % padding): too large
+    """The 70B SwiftKV shape at full size (16384 tokens, 40 layers, 10 % padding): too large
     for the CPU oracle in seconds, so it is checked through size-independent properties:
     rows of padded tokens and unaddressed slots keep their sentinel, a random sample of
     tokens matches the oracle bit for bit, and the write is idempotent."""

@@ -34,7 +34,7 @@ def test_reference_shapes(ops, shape, dtype, affine):
 
 @pytest.mark.parametrize("weight_only", [True, False])
 def test_config4_layernorm(ops, weight_only):
-    # BASELINE config 4's LayerNorm: [512, 4096] bf16, weight ~ N(1, .02), bias ~ N(0, .02), eps 1e-6
+    # the speculator benchmark shape: [512, 4096] bf16, weight ~ N(1, .02), bias ~ N(0, .02), eps 1e-6
     g = torch.Generator().manual_seed(3)
     x = torch.randn(512, 4096, generator=g).to(torch.bfloat16)
     w = (1 + 0.02 * torch.randn(4096, generator=g)).to(torch.bfloat16)

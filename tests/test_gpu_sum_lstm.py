@@ -56,7 +56,7 @@ def test_fast_gelu(ops, dtype):
 
 @pytest.mark.parametrize("alpha", [speculator_alpha(3, 4096), 1.0])
 def test_config4_three_steps(ops, alpha):
-    """BASELINE config 4: T=512, H=4096, bf16, 3 chained steps (cell_{k+1} = out_cell_k,
+    """The speculator benchmark shape: T=512, H=4096, bf16, 3 chained steps (cell_{k+1} = out_cell_k,
     fresh pre-activations per step)."""
     cell_gpu = cell_cpu = None
     for step in range(3):

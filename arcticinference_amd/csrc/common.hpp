@@ -133,6 +133,25 @@ __device__ __forceinline__ void store4_stream(void *p, uint32_t v) {
 #endif
 }
 
+// A lane's unit of work on the speculator paths: E consecutive 16-bit elements
+// moved with one access (E = 8: 16 bytes; narrower units measured slower).
+template <int E>
+struct Chunk;
+
+template <>
+struct Chunk<8> {
+  static constexpr int kBytes = 16;
+  uint4 v;
+  __device__ static __forceinline__ Chunk zero() { return Chunk{make_uint4(0, 0, 0, 0)}; }
+  __device__ static __forceinline__ Chunk load(const void *p) { return Chunk{load16(p)}; }
+  __device__ static __forceinline__ Chunk load_stream(const void *p) { return Chunk{load16_stream(p)}; }
+  __device__ __forceinline__ void store_stream(void *p) const { store16_stream(p, v); }
+  template <typename T>
+  __device__ __forceinline__ void unpack(float (&f)[8]) const { unpack8<T>(v, f); }
+  template <typename T>
+  __device__ static __forceinline__ Chunk pack(const float (&f)[8]) { return Chunk{pack8<T>(f)}; }
+};
+
 // ---- wave64 / workgroup reductions ------------------------------------------
 // DPP butterfly inside each row of 16 lanes, then the four row totals are read
 // with v_readlane.  Every lane returns the same wave total.

@@ -82,13 +82,14 @@ struct LstmParams {
 // in that order, so the first row sum, the candidate GELU and the early sigmoids
 // run while the later gates are still on their way, and only one sigmoid, one
 // multiply and the store remain after the last load has landed.
-template <typename T, int kChunksPerThread, bool kFastGelu, int kMaxThreads>
+template <typename T, int E, int kChunksPerThread, bool kFastGelu, int kMaxThreads>
 __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmParams p) {
   __shared__ float slots_cpre[16];
   __shared__ float slots_cnew[16];
   constexpr int K = kChunksPerThread;
+  using C = Chunk<E>;
   const int D = p.D;
-  const int chunks = D >> 3;
+  const int chunks = D / E;
   const int64_t row = blockIdx.x;
   const int64_t gate_bytes = (int64_t)D * 2;
   const char *s_row = p.states + row * p.s_stride * 2;
@@ -99,60 +100,60 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
 
   bool live[K];
   int64_t off[K];
-  uint4 sc[K], zc[K], sf[K], zf[K], si[K], zi[K], pc[K], so[K], zo[K];
-  uint4 wc[K], bc[K], ws[K], bs[K];
+  C sc[K], zc[K], sf[K], zf[K], si[K], zi[K], pc[K], so[K], zo[K];
+  C wc[K], bc[K], ws[K], bs[K];
 #pragma unroll
   for (int k = 0; k < K; ++k) {
     const int c = threadIdx.x + k * blockDim.x;
     live[k] = c < chunks;
-    off[k] = (int64_t)(live[k] ? c : 0) * 16;  // idle lanes re-read chunk 0 and discard it
+    off[k] = (int64_t)(live[k] ? c : 0) * C::kBytes;  // idle lanes re-read chunk 0 and discard it
   }
   // The scale / shift vectors are the same for every row (cache resident).  They
   // are requested first: memory returns loads in issue order, so asking for them
   // later would park the arithmetic behind the whole row.
 #pragma unroll
   for (int k = 0; k < K; ++k) {
-    if (p.w_cell) wc[k] = load16(p.w_cell + off[k]);
-    if (p.b_cell) bc[k] = load16(p.b_cell + off[k]);
-    if (p.w_state) ws[k] = load16(p.w_state + off[k]);
-    if (p.b_state) bs[k] = load16(p.b_state + off[k]);
+    if (p.w_cell) wc[k] = C::load(p.w_cell + off[k]);
+    if (p.b_cell) bc[k] = C::load(p.b_cell + off[k]);
+    if (p.w_state) ws[k] = C::load(p.w_state + off[k]);
+    if (p.b_state) bs[k] = C::load(p.b_state + off[k]);
   }
 #pragma unroll
   for (int k = 0; k < K; ++k) {
-    sc[k] = load16_stream(s_row + 3 * gate_bytes + off[k]);
-    zc[k] = load16_stream(z_row + 3 * gate_bytes + off[k]);
+    sc[k] = C::load_stream(s_row + 3 * gate_bytes + off[k]);
+    zc[k] = C::load_stream(z_row + 3 * gate_bytes + off[k]);
   }
 #pragma unroll
   for (int k = 0; k < K; ++k) {
-    sf[k] = load16_stream(s_row + off[k]);
-    zf[k] = load16_stream(z_row + off[k]);
+    sf[k] = C::load_stream(s_row + off[k]);
+    zf[k] = C::load_stream(z_row + off[k]);
   }
 #pragma unroll
-  for (int k = 0; k < K; ++k) pc[k] = load16_stream(pc_row + off[k]);
+  for (int k = 0; k < K; ++k) pc[k] = C::load_stream(pc_row + off[k]);
 #pragma unroll
   for (int k = 0; k < K; ++k) {
-    si[k] = load16_stream(s_row + gate_bytes + off[k]);
-    zi[k] = load16_stream(z_row + gate_bytes + off[k]);
+    si[k] = C::load_stream(s_row + gate_bytes + off[k]);
+    zi[k] = C::load_stream(z_row + gate_bytes + off[k]);
   }
 #pragma unroll
   for (int k = 0; k < K; ++k) {
-    so[k] = load16_stream(s_row + 2 * gate_bytes + off[k]);
-    zo[k] = load16_stream(z_row + 2 * gate_bytes + off[k]);
+    so[k] = C::load_stream(s_row + 2 * gate_bytes + off[k]);
+    zo[k] = C::load_stream(z_row + 2 * gate_bytes + off[k]);
   }
 
   // Lanes beyond the row take part in the sums with zeros.  (Each value is
   // cleared where it is first used, not here: touching pc now would wait for it.)
   // phase 1: pre_c and its sum of squares (reference :65-82); needs the cell gate only
-  float cact[K][8];
+  float cact[K][E];
   float ss = 0.f;
 #pragma unroll
   for (int k = 0; k < K; ++k) {
-    float a[8], b[8];
-    if (!live[k]) sc[k] = zc[k] = make_uint4(0, 0, 0, 0);
-    unpack8<T>(sc[k], a);
-    unpack8<T>(zc[k], b);
+    float a[E], b[E];
+    if (!live[k]) sc[k] = zc[k] = C::zero();
+    sc[k].template unpack<T>(a);
+    zc[k].template unpack<T>(b);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < E; ++j) {
       cact[k][j] = fmaf(p.alpha, b[j], a[j]);
       ss = fmaf(cact[k][j], cact[k][j], ss);
     }
@@ -161,12 +162,12 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
   // candidate = gelu(rmsnorm(pre_c)): runs while the other gates are still arriving
 #pragma unroll
   for (int k = 0; k < K; ++k) {
-    float w[8], b[8];
-    if (p.w_cell) unpack8<T>(wc[k], w);
-    if (p.b_cell) unpack8<T>(bc[k], b);
+    float w[E], b[E];
+    if (p.w_cell) wc[k].template unpack<T>(w);
+    if (p.b_cell) bc[k].template unpack<T>(b);
     const float mask = live[k] ? 1.f : 0.f;  // idle lanes must add nothing to the second sum
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < E; ++j) {
       float cn = cact[k][j] * inv_cpre;
       if (p.w_cell) cn *= w[j];
       if (p.b_cell) cn += b[j];
@@ -175,28 +176,28 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
   }
 
   // phase 2: cell update; write out_cell (reference :104-140)
-  float cell[K][8];  // ends up as the ROUNDED new cell, as the state phase must see it
+  float cell[K][E];  // ends up as the ROUNDED new cell, as the state phase must see it
   ss = 0.f;
 #pragma unroll
   for (int k = 0; k < K; ++k) {
-    float a[8], b[8], c[8];
-    unpack8<T>(sf[k], a);
-    unpack8<T>(zf[k], b);
-    if (!live[k]) pc[k] = make_uint4(0, 0, 0, 0);
-    unpack8<T>(pc[k], c);
+    float a[E], b[E], c[E];
+    sf[k].template unpack<T>(a);
+    zf[k].template unpack<T>(b);
+    if (!live[k]) pc[k] = C::zero();
+    pc[k].template unpack<T>(c);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) cell[k][j] = sigmoid_f(fmaf(p.alpha, b[j], a[j])) * c[j];
-    unpack8<T>(si[k], a);
-    unpack8<T>(zi[k], b);
+    for (int j = 0; j < E; ++j) cell[k][j] = sigmoid_f(fmaf(p.alpha, b[j], a[j])) * c[j];
+    si[k].template unpack<T>(a);
+    zi[k].template unpack<T>(b);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < E; ++j) {
       const float cnew = fmaf(cact[k][j], sigmoid_f(fmaf(p.alpha, b[j], a[j])), cell[k][j]);
       ss = fmaf(cnew, cnew, ss);  // unrounded, as in the reference (:136)
       cell[k][j] = cnew;
     }
-    const uint4 packed = pack8<T>(cell[k]);
-    if (live[k]) store16_stream(oc_row + off[k], packed);
-    unpack8<T>(packed, cell[k]);
+    const C packed = C::template pack<T>(cell[k]);
+    if (live[k]) packed.store_stream(oc_row + off[k]);
+    packed.template unpack<T>(cell[k]);
   }
   const float inv_cnew = rsqrtf(block_sum(ss, slots_cnew) * p.inv_D + p.eps_state);
 
@@ -204,22 +205,22 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
   // the output gate is the last load to arrive and is consumed last
 #pragma unroll
   for (int k = 0; k < K; ++k) {
-    float w[8], b[8], st[8];
-    if (p.w_state) unpack8<T>(ws[k], w);
-    if (p.b_state) unpack8<T>(bs[k], b);
+    float w[E], b[E], st[E];
+    if (p.w_state) ws[k].template unpack<T>(w);
+    if (p.b_state) bs[k].template unpack<T>(b);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < E; ++j) {
       float cn = cell[k][j] * inv_cnew;
       if (p.w_state) cn *= w[j];
       if (p.b_state) cn += b[j];
       st[j] = gelu<kFastGelu>(cn);
     }
-    float a[8], g[8];
-    unpack8<T>(so[k], a);
-    unpack8<T>(zo[k], g);
+    float a[E], g[E];
+    so[k].template unpack<T>(a);
+    zo[k].template unpack<T>(g);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) st[j] *= sigmoid_f(fmaf(p.alpha, g[j], a[j]));
-    if (live[k]) store16_stream(os_row + off[k], pack8<T>(st));
+    for (int j = 0; j < E; ++j) st[j] *= sigmoid_f(fmaf(p.alpha, g[j], a[j]));
+    if (live[k]) C::template pack<T>(st).store_stream(os_row + off[k]);
   }
 }
 
@@ -284,22 +285,18 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
                    aligned16(p.b_cell) && aligned16(p.w_state) && aligned16(p.b_state);
   const dim3 grid((unsigned)rows);
   if (vec) {
-    // one 16-byte chunk per lane up to 512 lanes (D <= 4096), two beyond that
-    int cpt = chunks > 512 ? 2 : 1;
-#ifdef ARCTIC_TUNING
-    if (const char *e = getenv("ARCTIC_LSTM_CPT")) cpt = atoi(e) == 2 ? 2 : 1;
-#endif
-    if (cpt == 1 && chunks > 1024) cpt = 2;
-    int threads = (chunks + cpt - 1) / cpt;
+    const int units = p.D / 8;
+    const int cpt = units > 512 ? 2 : 1;   // one 16-byte chunk per lane up to 512 lanes (D <= 4096)
+    int threads = (units + cpt - 1) / cpt;
     threads = std::max(64, (threads + 63) & ~63);
-    if (cpt == 1 && threads <= 512)
-      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 1, kFastGelu, 512>), grid, dim3(threads), 0, s, p);
-    else if (cpt == 1)
-      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 1, kFastGelu, 1024>), grid, dim3(threads), 0, s, p);
-    else if (threads <= 256)
-      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 2, kFastGelu, 256>), grid, dim3(threads), 0, s, p);
+    unsigned lds = 0;
+#ifdef ARCTIC_TUNING
+    if (const char *e = getenv("ARCTIC_LSTM_LDS")) lds = (unsigned)atoi(e);
+#endif
+    if (cpt == 1)
+      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512>), grid, dim3(threads), lds, s, p);
     else
-      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 2, kFastGelu, 1024>), grid, dim3(threads), 0, s, p);
+      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 2, kFastGelu, 1024>), grid, dim3(threads), lds, s, p);
   } else {
     hipLaunchKernelGGL((sum_lstm_scalar_kernel<T, kFastGelu>), grid, dim3(256), 0, s, p);
   }

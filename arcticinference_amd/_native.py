@@ -25,6 +25,7 @@ EXPORTED_SYMBOLS = (
     "arctic_abi_version",
     "arctic_last_error",
     "arctic_reshape_and_cache_flash_bulk",
+    "arctic_reshape_and_cache_flash_fp4",
     "arctic_speculator_ln",
     "arctic_sum_lstm",
 )
@@ -73,6 +74,9 @@ def _declare(lib: ctypes.CDLL) -> None:
         i32, i32, i32, i32,    # num_layers, num_heads, head_size, block_size
         i64, i32, i32, vp]     # block_stride, src_dtype, kv_cache_dtype, stream
     lib.arctic_reshape_and_cache_flash_bulk.restype = i32
+    lib.arctic_reshape_and_cache_flash_fp4.argtypes = [
+        vp, vp, i64, i64, vp, vp, vp, vp, vp, i64, i32, i32, i32, i64, i64, i64, i32, vp]
+    lib.arctic_reshape_and_cache_flash_fp4.restype = i32
     lib.arctic_speculator_ln.argtypes = [vp, vp, vp, vp, i64, i32, i64, f32, i32, vp]
     lib.arctic_speculator_ln.restype = i32
     lib.arctic_sum_lstm.argtypes = [vp] * 9 + [i64, i32, i64, i64, i64, i64, f32, f32, f32, i32, i32, vp]

@@ -179,10 +179,56 @@ def _reshape_and_cache_flash_bulk_impl(
     _native.check(rc)
 
 
-def _reshape_and_cache_flash_fp4_impl(*args, **kwargs) -> None:
-    raise NotImplementedError(
-        "arctic_inference::reshape_and_cache_flash_fp4 is not part of this library "
-        "(only the bulk KV write and the speculator ops are)")
+def _reshape_and_cache_flash_fp4_impl(
+    key: torch.Tensor,
+    value: torch.Tensor,
+    key_cache: torch.Tensor,
+    value_cache: torch.Tensor,
+    slot_mapping: torch.Tensor,
+    kv_cache_dtype: str,
+    k_scale: torch.Tensor,
+    v_scale: torch.Tensor,
+    key_scale_cache: torch.Tensor,
+    value_scale_cache: torch.Tensor,
+) -> None:
+    """Host side of the NVFP4-style cache write; layout detection and checks follow the
+    reference's launcher (csrc/custom_ops/reshape_and_cache_flash_fp4.cu:256-337).
+    kv_cache_dtype, k_scale and v_scale are accepted and unused, as in the reference."""
+    lib = _lib()
+    _check(key.dtype in _HALF_DTYPES,
+           "Unsupported input dtype for reshape_and_cache_fp4. Must be half or bfloat16.")
+    _check(key.dim() == 3 and value.dim() == 3, "reshape_and_cache_flash_fp4: key/value must be [tokens, heads, head_size]")
+    num_tokens = slot_mapping.size(0)
+    num_heads, head_size = key.size(1), key.size(2)
+    _check(key_cache.dim() == 4 and value_cache.dim() == 4, "KV cache must be rank-4")
+    is_nhd = key_cache.size(2) == num_heads
+    block_stride = key_cache.stride(0)
+    page_stride = key_cache.stride(1) if is_nhd else key_cache.stride(2)
+    head_stride = key_cache.stride(2) if is_nhd else key_cache.stride(1)
+    block_size = key_cache.size(1) if is_nhd else key_cache.size(2)
+    _check(value_cache.stride(0) == block_stride, "block_stride mismatch")
+    _check((value_cache.stride(1) if is_nhd else value_cache.stride(2)) == page_stride, "page_stride mismatch")
+    _check((value_cache.stride(2) if is_nhd else value_cache.stride(1)) == head_stride, "head_stride mismatch")
+    _check((value_cache.size(1) if is_nhd else value_cache.size(2)) == block_size,
+           "block_size mismatch between key_cache and value_cache")
+    # assumed, not checked, by the reference (it would write out of bounds instead)
+    _check(value.dtype == key.dtype and value.shape == key.shape, "reshape_and_cache_flash_fp4: key/value mismatch")
+    _check(key.stride(2) == 1 and key.stride(1) == head_size and value.stride(2) == 1 and
+           value.stride(1) == head_size, "reshape_and_cache_flash_fp4: heads of a token must be dense")
+    _check(slot_mapping.dtype == torch.int64, f"expected scalar type Long but found {slot_mapping.dtype}")
+    _check(all(t.element_size() == 1 for t in (key_cache, value_cache, key_scale_cache, value_scale_cache)),
+           "reshape_and_cache_flash_fp4: caches and scale caches must be byte tensors")
+    _check(key_cache.size(3) * 2 == head_size and key_cache.stride(3) == 1,
+           "reshape_and_cache_flash_fp4: cache last dim must be head_size / 2 packed bytes")
+    _check(key_scale_cache.numel() * 8 >= key_cache.numel() and value_scale_cache.numel() * 8 >= value_cache.numel(),
+           "reshape_and_cache_flash_fp4: scale cache too small (one byte per 16 elements)")
+    with _on_device_of(key):
+        rc = lib.arctic_reshape_and_cache_flash_fp4(
+            key.data_ptr(), value.data_ptr(), key.stride(0), value.stride(0), key_cache.data_ptr(),
+            value_cache.data_ptr(), key_scale_cache.data_ptr(), value_scale_cache.data_ptr(),
+            slot_mapping.data_ptr(), num_tokens, num_heads, head_size, int(block_size), int(block_stride),
+            int(page_stride), int(head_stride), _HALF_DTYPES[key.dtype], _stream_of(key))
+    _native.check(rc)
 
 
 def _speculator_ln_impl(input: torch.Tensor, weight: Optional[torch.Tensor],

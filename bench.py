@@ -198,6 +198,57 @@ def bench_speculator(ops, dev, steps, warmup):
     return out
 
 
+def bench_fp4(ops, dev, steps):
+    """NVFP4-style cache write, one call per layer as the model would issue them: 8192 tokens,
+    8 KV heads x 128, 16 layers (16 key/value tensors and caches, so nothing is re-used from cache).
+    Algorithmic bytes per token and layer: 2 x 2n read + 2 x (n/2 + n/16) written = 5248 B."""
+    T, H, D, bs, NB, L = 8192, 8, 128, 16, 8192, 16
+    g = torch.Generator(device=dev).manual_seed(5)
+    keys = [(torch.randn(T, H, D, generator=g, device=dev) * 0.5).to(torch.bfloat16) for _ in range(L)]
+    values = [(torch.randn(T, H, D, generator=g, device=dev) * 0.5).to(torch.bfloat16) for _ in range(L)]
+    kc = [torch.zeros(NB, bs, H, D // 2, dtype=torch.uint8, device=dev) for _ in range(L)]
+    vc = [torch.zeros(NB, bs, H, D // 2, dtype=torch.uint8, device=dev) for _ in range(L)]
+    ks = [torch.zeros(NB, bs, H, D // 16, dtype=torch.uint8, device=dev) for _ in range(L)]
+    vs = [torch.zeros(NB, bs, H, D // 16, dtype=torch.uint8, device=dev) for _ in range(L)]
+    slots = torch.randperm(NB * bs, generator=torch.Generator().manual_seed(5))[:T].to(dev)
+    z = torch.zeros((), device=dev)
+
+    def step():
+        for l in range(L):
+            ops.reshape_and_cache_flash_fp4(keys[l], values[l], kc[l], vc[l], ks[l], vs[l], slots, "fp4", z, z)
+
+    for _ in range(3):
+        step()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    graph.replay()
+    torch.cuda.synchronize()
+    med = statistics.median(event_times_us(graph.replay, max(10, steps // 2))) / L
+    nbytes = T * (4 * H * D + 2 * (H * D // 2 + H * D // 16))
+    return {"us_per_layer_graph": round(med, 2), "bytes_per_layer": nbytes, "GBps": round(nbytes / med / 1e3, 1),
+            "hbm_frac": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
+
+
+def box_reference(dev):
+    """What plain library kernels reach on this very GPU (boxes of one pool differ by up to 20 %):
+    a contiguous bf16 -> fp8 cast of 1.3 GB (the same 2:1 read:write mix as the bulk fp8 write, no
+    scatter, no scaling) and a 1 GiB device-to-device copy."""
+    x = torch.randn(1 << 26, device=dev).to(torch.bfloat16).repeat(10)
+    f = lambda: x.to(torch.float8_e4m3fn)
+    for _ in range(3):
+        f()
+    cast = statistics.median(event_times_us(f, 10))
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    g = lambda: dst.copy_(src)
+    for _ in range(3):
+        g()
+    copy = statistics.median(event_times_us(g, 10))
+    return {"torch_bf16_to_fp8_cast_GBps": round(x.numel() * 3 / cast / 1e3, 1),
+            "torch_copy_1GiB_GBps": round(2 * (1 << 30) / copy / 1e3, 1)}
+
+
 def bench_decode_mix(ops, dev, steps):
     """Decode-step workload: 512 decode tokens; bulk fp8 KV write over 16 layers into
     32768-block caches, ln0, three sum_lstm steps; one HIP graph per step."""
@@ -310,6 +361,9 @@ def main():
         extras["bulk_fp8_8b_prefill"] = {"kernel_us": round(m, 2), "GBps": round(w2.bytes / m / 1e3, 1),
                                          "hbm_frac": round(w2.bytes / m / 1e3 / HBM_PEAK_GBS, 4)}
         del w2, f2
+        torch.cuda.empty_cache()
+        extras["box_reference"] = box_reference(dev)
+        extras["fp4_write_8b_layer"] = bench_fp4(ops, dev, args.steps)
         torch.cuda.empty_cache()
         extras["speculator"] = bench_speculator(ops, dev, args.steps, args.warmup)
         extras["decode_mix"] = bench_decode_mix(ops, dev, args.steps)

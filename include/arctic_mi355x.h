@@ -93,6 +93,35 @@ int arctic_reshape_and_cache_flash_bulk(
     void *stream);
 
 /*
+ * NVFP4-style KV-cache write for ONE layer: e2m1 values, two per byte (first element
+ * in the low nibble), plus one e4m3 scale byte per 16 elements.  Replaces
+ *   reshape_and_cache_flash_fp4()             csrc/custom_ops/reshape_and_cache_flash_fp4.cu:256-337
+ *   reshape_and_cache_flash_kernel_fp4<>, quantize_16_to_fp4<>   :104-254
+ * (custom_ops.h:19-27, torch_bindings.cpp:20-32).
+ *
+ * For every token t with slot = slot_mapping[t] >= 0, head h and group g of 16 elements:
+ *   amax = max |x|;  scale byte = e4m3(amax / 6) (saturating);  SF = value of that byte
+ *   nibble_i = e2m1(x_i / SF), round to nearest even, saturating at +-6 (0 if SF == 0)
+ *   packed -> cache      + blk*block_stride     + off*page_stride     + h*head_stride     + g*8
+ *   scale  -> scale cache + blk*(block_stride/8) + off*(page_stride/8) + h*(head_stride/8) + g
+ * with blk = slot / block_size, off = slot % block_size.  Strides are in BYTES of the packed
+ * cache: NHD [NB, block_size, H, D/2] passes page_stride = stride(1), head_stride = stride(2);
+ * HND [NB, H, block_size, D/2] passes page_stride = stride(2), head_stride = stride(1).  The
+ * reference's per-tensor k_scale / v_scale and kv_cache_dtype arguments have no effect there
+ * and are not part of this call.  The two reciprocals (1/6, 1/SF) are correctly rounded here
+ * and approximate (rcp.approx.ftz) in the reference.
+ *
+ *   key, value   device; [num_tokens, num_heads*head_size] F16 or BF16, row strides in ELEMENTS,
+ *                16-byte aligned rows; head_size % 16 == 0
+ */
+int arctic_reshape_and_cache_flash_fp4(
+    const void *key, const void *value, int64_t key_stride, int64_t value_stride,
+    void *key_cache, void *value_cache, void *key_scale_cache,
+    void *value_scale_cache, const int64_t *slot_mapping, int64_t num_tokens,
+    int num_heads, int head_size, int block_size, int64_t block_stride,
+    int64_t page_stride, int64_t head_stride, int dtype, void *stream);
+
+/*
  * Speculator "LayerNorm" (an RMS norm with optional scale and shift).  Replaces
  *   speculator_ln_cuda()                      csrc/custom_ops/speculator_ln.cu:152-252
  *   spec_ln_vec_kernel<> / spec_ln_scalar_kernel<>   csrc/custom_ops/speculator_ln.cu:21-150

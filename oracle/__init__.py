@@ -66,6 +66,13 @@ def lib() -> ctypes.CDLL:
             vp, vp, i64, i64, vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i64,
             i32, i32]
         L.ao_reshape_and_cache_flash_bulk.restype = i32
+        L.ao_f32_to_e2m1.argtypes = [f32]
+        L.ao_f32_to_e2m1.restype = ctypes.c_uint8
+        L.ao_e2m1_to_f32.argtypes = [ctypes.c_uint8]
+        L.ao_e2m1_to_f32.restype = f32
+        L.ao_reshape_and_cache_flash_fp4.argtypes = [vp, vp, i64, i64, vp, vp, vp, vp, vp, i64, i32, i32, i32,
+                                                     i64, i64, i64, i32]
+        L.ao_reshape_and_cache_flash_fp4.restype = i32
         L.ao_speculator_ln.argtypes = [vp, vp, vp, vp, i64, i32, i64, f32, i32]
         L.ao_speculator_ln.restype = i32
         L.ao_sum_lstm.argtypes = [vp] * 9 + [i64, i32, i64, i64, i64, i64, f32,
@@ -154,6 +161,43 @@ def reshape_and_cache_flash_bulk(
         _SRC_DTYPE[keys.dtype], _KV_DTYPE[kv_cache_dtype])
     if rc != 0:
         raise RuntimeError("oracle: unsupported dtype combination")
+
+
+def fp4_layout(key: torch.Tensor, key_cache: torch.Tensor):
+    """(is_nhd, block_size, block_stride, page_stride, head_stride) exactly as the reference's
+    host code derives them (csrc/custom_ops/reshape_and_cache_flash_fp4.cu:266-280)."""
+    num_heads = key.size(1)
+    is_nhd = key_cache.size(2) == num_heads
+    block_stride = key_cache.stride(0)
+    page_stride = key_cache.stride(1) if is_nhd else key_cache.stride(2)
+    head_stride = key_cache.stride(2) if is_nhd else key_cache.stride(1)
+    block_size = key_cache.size(1) if is_nhd else key_cache.size(2)
+    return is_nhd, block_size, block_stride, page_stride, head_stride
+
+
+def reshape_and_cache_flash_fp4(keys: torch.Tensor, values: torch.Tensor, key_cache: torch.Tensor,
+                                value_cache: torch.Tensor, key_cache_scales: torch.Tensor,
+                                value_cache_scales: torch.Tensor, slot_mapping: torch.Tensor,
+                                kv_cache_dtype: str, k_scale: torch.Tensor, v_scale: torch.Tensor) -> None:
+    """In-place NVFP4-style cache write on CPU tensors; argument order of the reference's Python
+    wrapper (arctic_inference/py_custom_ops.py:76-90)."""
+    for t in (keys, values, key_cache, value_cache, key_cache_scales, value_cache_scales, slot_mapping):
+        _cpu(t, "tensor")
+    assert key_cache.dim() == 4 and value_cache.dim() == 4
+    _, block_size, block_stride, page_stride, head_stride = fp4_layout(keys, key_cache)
+    rc = lib().ao_reshape_and_cache_flash_fp4(
+        keys.data_ptr(), values.data_ptr(), keys.stride(0), values.stride(0), key_cache.data_ptr(),
+        value_cache.data_ptr(), key_cache_scales.data_ptr(), value_cache_scales.data_ptr(),
+        slot_mapping.data_ptr(), slot_mapping.size(0), keys.size(1), keys.size(2), block_size, block_stride,
+        page_stride, head_stride, _SRC_DTYPE[keys.dtype])
+    if rc != 0:
+        raise RuntimeError("oracle: fp4 cache write needs fp16/bf16 input and head_size % 16 == 0")
+
+
+def e2m1_decode(nibbles: torch.Tensor) -> torch.Tensor:
+    L = lib()
+    table = torch.tensor([L.ao_e2m1_to_f32(c) for c in range(16)], dtype=torch.float32)
+    return table[nibbles.to(torch.int64)]
 
 
 def speculator_ln(input: torch.Tensor, weight: Optional[torch.Tensor],

@@ -256,6 +256,94 @@ int ao_reshape_and_cache_flash_bulk(
   return 0;
 }
 
+/* ---- next row: NVFP4-style KV-cache write ----------------------------------
+ * Restates reshape_and_cache_flash_kernel_fp4 / quantize_16_to_fp4
+ * (csrc/custom_ops/reshape_and_cache_flash_fp4.cu:104-147,150-254), sm_100 branch:
+ * per group of 16 consecutive elements along head_size
+ *   amax   = max |x|                                   (:115-121, NaN ignored by __hmax)
+ *   sf     = amax * (1/6)                               (:122)
+ *   scale  = e4m3(sf), stored as one byte; SF = float(scale)   (:124-128)
+ *   inv    = SF != 0 ? 1/SF : 0                          (:131-132)
+ *   nibble = e2m1(x * inv), round to nearest even, saturating at +-6 (:64-76)
+ * two nibbles per byte, the first element in the low nibble (:88).
+ * The reference takes both reciprocals with rcp.approx.ftz (<= 1 ulp from the
+ * correctly rounded value); this restatement uses the correctly rounded ones, so
+ * PARITY IS UNPINNED where that last ulp decides a rounding, and for NaN inputs
+ * (PTX maps NaN to +6 there, the sm_90 fallback :36-38 to 0; here: +6).
+ * k_scale / v_scale / kv_cache_dtype are accepted and ignored, as in the reference.
+ * Strides are in bytes of the packed cache; the scale cache uses stride/8 (:185-187).
+ */
+uint8_t ao_f32_to_e2m1(float v) {
+  uint32_t u = f32_bits(v);
+  uint8_t sign = (uint8_t)((u >> 28) & 0x8u);
+  float x = fabsf(v);
+  uint8_t m;
+  if (x != x) return 0x7; /* NaN */
+  if (x > 5.0f) m = 7;           /* 6 */
+  else if (x >= 3.5f) m = 6;     /* 4; 3.5 ties to even (4) */
+  else if (x > 2.5f) m = 5;      /* 3; 2.5 ties to even (2) */
+  else if (x >= 1.75f) m = 4;    /* 2 */
+  else if (x > 1.25f) m = 3;     /* 1.5; 1.25 ties to even (1) */
+  else if (x >= 0.75f) m = 2;    /* 1 */
+  else if (x > 0.25f) m = 1;     /* 0.5; 0.25 ties to even (0) */
+  else m = 0;
+  return (uint8_t)(sign | m);
+}
+
+float ao_e2m1_to_f32(uint8_t c) {
+  static const float lut[8] = {0.f, 0.5f, 1.f, 1.5f, 2.f, 3.f, 4.f, 6.f};
+  float v = lut[c & 7];
+  return (c & 8) ? -v : v;
+}
+
+/* One group of 16: writes 8 packed bytes and 1 scale byte. */
+static void quantize_16_to_fp4(const void *src, int64_t first, int dtype, uint8_t *dst, uint8_t *scale_dst) {
+  float x[16];
+  float amax = 0.f;
+  for (int i = 0; i < 16; ++i) {
+    x[i] = load_as_f32(src, first + i, dtype);
+    float a = fabsf(x[i]);
+    if (a > amax) amax = a; /* NaN never wins the comparison */
+  }
+  volatile float sixth = 1.0f / 6.0f;
+  volatile float sf = amax * sixth;
+  const uint8_t code = ao_f32_to_e4m3fn(sf);
+  *scale_dst = code;
+  const float SF = ao_e4m3fn_to_f32(code);
+  volatile float inv = (SF != 0.0f) ? 1.0f / SF : 0.0f;
+  for (int i = 0; i < 8; ++i) {
+    volatile float a = x[2 * i] * inv, b = x[2 * i + 1] * inv;
+    dst[i] = (uint8_t)((ao_f32_to_e2m1(b) << 4) | ao_f32_to_e2m1(a));
+  }
+}
+
+int ao_reshape_and_cache_flash_fp4(const void *key, const void *value, int64_t key_stride, int64_t value_stride,
+                                   uint8_t *key_cache, uint8_t *value_cache, uint8_t *key_scale_cache,
+                                   uint8_t *value_scale_cache, const int64_t *slot_mapping, int64_t num_tokens,
+                                   int num_heads, int head_size, int block_size, int64_t block_stride,
+                                   int64_t page_stride, int64_t head_stride, int dtype) {
+  if (dtype != AO_F16 && dtype != AO_BF16) return -1;
+  if (head_size % 16) return -2;
+  const int groups = head_size / 16;
+#pragma omp parallel for schedule(static)
+  for (int64_t t = 0; t < num_tokens; ++t) {
+    const int64_t slot = slot_mapping[t];
+    if (slot < 0) continue;
+    const int64_t blk = slot / block_size, off = slot % block_size;
+    for (int h = 0; h < num_heads; ++h) {
+      const int64_t row = blk * block_stride + off * page_stride + (int64_t)h * head_stride;
+      const int64_t srow = blk * (block_stride / 8) + off * (page_stride / 8) + (int64_t)h * (head_stride / 8);
+      for (int g = 0; g < groups; ++g) {
+        quantize_16_to_fp4(key, t * key_stride + (int64_t)h * head_size + g * 16, dtype, key_cache + row + g * 8,
+                           key_scale_cache + srow + g);
+        quantize_16_to_fp4(value, t * value_stride + (int64_t)h * head_size + g * 16, dtype,
+                           value_cache + row + g * 8, value_scale_cache + srow + g);
+      }
+    }
+  }
+  return 0;
+}
+
 /* ---- Part B: speculator "LayerNorm" (an RMS norm) -------------------------
  * Restates spec_ln_vec_kernel / spec_ln_scalar_kernel
  * (csrc/custom_ops/speculator_ln.cu:21-150):

@@ -1,0 +1,82 @@
+"""GPU parity of the NVFP4-style cache write against the CPU oracle: bit-exact (the oracle and
+the kernel use the same correctly rounded reciprocals)."""
+import pytest
+import torch
+
+import oracle
+from test_oracle_fp4 import make_case
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+ZERO = torch.tensor(0.0)
+
+
+def run_both(ops, key, value, kc, vc, ksc, vsc, slots):
+    d = [t.to(DEV) for t in (key, value, kc, vc, ksc, vsc, slots)]
+    ops.reshape_and_cache_flash_fp4(d[0], d[1], d[2], d[3], d[4], d[5], d[6], "fp4", ZERO.to(DEV), ZERO.to(DEV))
+    torch.cuda.synchronize()
+    oracle.reshape_and_cache_flash_fp4(key, value, kc, vc, ksc, vsc, slots, "fp4", ZERO, ZERO)
+    for got, want, name in zip(d[2:6], (kc, vc, ksc, vsc), ("key cache", "value cache", "key scales", "value scales")):
+        g = got.cpu()
+        if not torch.equal(g, want):
+            bad = (g != want).nonzero()
+            raise AssertionError(f"{name}: {bad.shape[0]} bytes differ, first at {bad[0].tolist()}: "
+                                 f"got {int(g[tuple(bad[0])])} want {int(want[tuple(bad[0])])}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("nhd", [True, False])
+@pytest.mark.parametrize("shape", [
+    (64, 16, 128, 16, 4),      # the reference test's sizes (tests/unit_tests/test_reshape_and_cache_flash_nvfp4.py:85-90)
+    (256, 8, 64, 32, 8),
+    (33, 8, 128, 16, 3),
+    (5, 1, 16, 4, 3),
+])
+def test_random(ops, dtype, nhd, shape):
+    T, H, D, bs, NB = shape
+    run_both(ops, *make_case(T, H, D, bs, NB, dtype, nhd, seed=21))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_every_finite_sixteen_bit_value(ops, dtype):
+    """All 16-bit patterns as inputs (NaN patterns replaced by 0: the NaN nibble is unpinned),
+    in groups whose maximum is also forced through every magnitude."""
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype)
+    x = torch.where(torch.isnan(bits.float()), torch.zeros_like(bits), bits)
+    g = torch.Generator().manual_seed(5)
+    x = x[torch.randperm(65536, generator=g)]
+    T, H, D = 64, 8, 128
+    key = x.view(T, H, D).clone()
+    value = (x.float() * 3.0e-3).to(dtype).view(T, H, D)      # a second pass at a different magnitude
+    _, _, kc, vc, ksc, vsc, _ = make_case(T, H, D, 16, 4, dtype, True, seed=6, pad=0.0)
+    slots = torch.randperm(64, generator=g).to(torch.int64)
+    run_both(ops, key, value, kc, vc, ksc, vsc, slots)
+
+
+def test_rounding_ties(ops):
+    """Groups whose scale is an exact power of two, holding every e2m1 tie and its neighbours."""
+    ties = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0])
+    ulp = torch.tensor([-1, 0, 1], dtype=torch.int32)
+    pts = (ties.view(torch.int32)[:, None] + ulp[None, :]).view(torch.float32).reshape(-1)   # 21 values
+    pts = torch.cat([pts, -pts])[:30]
+    T, H, D = 8, 2, 32
+    key = torch.zeros(T * H * D // 16, 16)
+    for r in range(key.shape[0]):
+        k = r % 5 - 2
+        key[r, 0] = 6.0 * 2.0 ** k                      # forces SF = 2^k exactly
+        key[r, 1:] = pts[(torch.arange(15) + r) % 30] * 2.0 ** k
+    key = key.view(T, H, D)
+    for dtype in (torch.float16, torch.bfloat16):
+        _, _, kc, vc, ksc, vsc, _ = make_case(T, H, D, 8, 1, dtype, True, seed=8, pad=0.0)
+        run_both(ops, key.to(dtype), (-key).to(dtype), kc, vc, ksc, vsc, torch.arange(T, dtype=torch.int64))
+
+
+def test_errors(ops):
+    key, value, kc, vc, ksc, vsc, slots = [t.to(DEV) for t in make_case(4, 2, 32, 4, 2, torch.bfloat16, True, seed=1)]
+    z = ZERO.to(DEV)
+    with pytest.raises(RuntimeError, match="Must be half or bfloat16"):
+        ops.reshape_and_cache_flash_fp4(key.float(), value.float(), kc, vc, ksc, vsc, slots, "fp4", z, z)
+    with pytest.raises(RuntimeError, match="KV cache must be rank-4"):
+        ops.reshape_and_cache_flash_fp4(key, value, kc[0], vc[0], ksc, vsc, slots, "fp4", z, z)
+    with pytest.raises(RuntimeError, match="block_stride mismatch"):
+        ops.reshape_and_cache_flash_fp4(key, value, kc, torch.cat([vc, vc], dim=1), ksc, vsc, slots, "fp4", z, z)

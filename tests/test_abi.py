@@ -44,9 +44,12 @@ def test_abi_version_matches_header(lib):
 
 
 def test_no_torch_dependency():
-    out = subprocess.run(["ldd", _native.library_path()], capture_output=True, text=True).stdout
-    assert "torch" not in out and "c10" not in out and "python" not in out.lower()
-    assert "amdhip64" in out
+    # the NEEDED entries of the ELF file itself (ldd would also resolve transitive paths)
+    out = subprocess.run(["readelf", "-d", _native.library_path()], capture_output=True, text=True).stdout
+    needed = [l.split("[")[-1].rstrip("]") for l in out.splitlines() if "(NEEDED)" in l]
+    assert needed, out
+    assert not any(("torch" in n) or ("c10" in n) or ("python" in n.lower()) for n in needed), needed
+    assert any("amdhip64" in n for n in needed), needed
 
 
 def test_header_compiles_as_plain_c(tmp_path):

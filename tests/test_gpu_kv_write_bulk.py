@@ -148,6 +148,39 @@ def test_config2_fp8_prefill_chunk(ops):
     run_both(ops, case)
 
 
+@pytest.mark.parametrize("kv", ["fp8", "auto"])
+def test_long_prefill_launch_shape(ops, kv):
+    """4096 tokens x 32 layers: takes the 512-lane x 2-chunk kernel shape used for long
+    prefill launches; compared in full against the oracle."""
+    case = make_bulk_case(T=4096, L=32, H=8, D=128, bs=16, NB=512, kv_cache_dtype=kv, seed=12, std=1.5,
+                          pad_fraction=0.05)
+    run_both(ops, case)
+
+
+def test_random_configurations(ops):
+    """Seeded sweep over shapes, dtypes, layouts, pitches and padding: exercises the layer
+    grouping, the power-of-two and general row decompositions, the multi-launch split and
+    the element-wise fallback against the oracle."""
+    import random
+    rnd = random.Random(2024)
+    for it in range(40):
+        H = rnd.choice([1, 2, 3, 4, 8])
+        D = rnd.choice([16, 32, 64, 80, 96, 128, 20])
+        cfg = dict(T=rnd.choice([1, 2, 7, 33, 130, 600]), L=rnd.choice([1, 2, 5, 16, 33, 64, 65, 100]), H=H, D=D,
+                   bs=rnd.choice([1, 4, 16, 32]), NB=0,
+                   src_dtype=rnd.choice([torch.bfloat16, torch.float16, torch.float32]),
+                   kv_cache_dtype=rnd.choice(["auto", "fp8", "fp8_e5m2"]), seed=1000 + it, std=rnd.choice([0.1, 1.5, 30.0]),
+                   pad_fraction=rnd.choice([0.0, 0.1, 0.5]), layout=rnd.choice(["flash", "flashinfer"]),
+                   key_pad=rnd.choice([0, 0, 8, 24, 3]))
+        cfg["NB"] = (cfg["T"] + cfg["bs"] - 1) // cfg["bs"] + rnd.choice([0, 1, 5])
+        if cfg["T"] * cfg["L"] * H * D > 40_000_000:
+            cfg["L"] = max(1, 40_000_000 // (cfg["T"] * H * D))
+        try:
+            run_both(ops, make_bulk_case(**cfg))
+        except AssertionError as e:
+            raise AssertionError(f"configuration {it}: {cfg}: {e}") from None
+
+
 def test_config3_shape_properties(ops):
     """The 70B SwiftKV shape at full size (16384 tokens, 40 layers, 10 % padding): too large
     for the CPU oracle in seconds, so it is checked through size-independent properties:

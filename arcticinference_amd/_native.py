@@ -28,6 +28,7 @@ EXPORTED_SYMBOLS = (
     "arctic_reshape_and_cache_flash_fp4",
     "arctic_speculator_ln",
     "arctic_sum_lstm",
+    "arctic_sum_lstm_shared_z",
 )
 
 _lib: Optional[ctypes.CDLL] = None
@@ -81,6 +82,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.arctic_speculator_ln.restype = i32
     lib.arctic_sum_lstm.argtypes = [vp] * 9 + [i64, i32, i64, i64, i64, i64, f32, f32, f32, i32, i32, vp]
     lib.arctic_sum_lstm.restype = i32
+    lib.arctic_sum_lstm_shared_z.argtypes = lib.arctic_sum_lstm.argtypes
+    lib.arctic_sum_lstm_shared_z.restype = i32
 
 
 def load() -> ctypes.CDLL:

@@ -82,7 +82,11 @@ struct LstmParams {
 // in that order, so the first row sum, the candidate GELU and the early sigmoids
 // run while the later gates are still on their way, and only one sigmoid, one
 // multiply and the store remain after the last load has landed.
-template <typename T, int E, int kChunksPerThread, bool kFastGelu, int kMaxThreads>
+// kSharedZ: `z4` holds ONE gate-wide row per token ([rows, D]) that is added to all four
+// gates, as the speculator's z4 = emb.repeat(1, 1, 4) would; it is then read once, not four times.
+// kAllVectors: all four scale / shift vectors are given (the speculator always passes them)
+// AND every lane of the workgroup owns a chunk, so no select on either is needed.
+template <typename T, int E, int kChunksPerThread, bool kFastGelu, int kMaxThreads, bool kSharedZ, bool kAllVectors>
 __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmParams p) {
   __shared__ float slots_cpre[16];
   __shared__ float slots_cnew[16];
@@ -105,7 +109,7 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
 #pragma unroll
   for (int k = 0; k < K; ++k) {
     const int c = threadIdx.x + k * blockDim.x;
-    live[k] = c < chunks;
+    live[k] = kAllVectors || c < chunks;
     off[k] = (int64_t)(live[k] ? c : 0) * C::kBytes;  // idle lanes re-read chunk 0 and discard it
   }
   // The scale / shift vectors are the same for every row (cache resident).  They
@@ -113,32 +117,32 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
   // later would park the arithmetic behind the whole row.
 #pragma unroll
   for (int k = 0; k < K; ++k) {
-    if (p.w_cell) wc[k] = C::load(p.w_cell + off[k]);
-    if (p.b_cell) bc[k] = C::load(p.b_cell + off[k]);
-    if (p.w_state) ws[k] = C::load(p.w_state + off[k]);
-    if (p.b_state) bs[k] = C::load(p.b_state + off[k]);
+    if (kAllVectors || p.w_cell) wc[k] = C::load(p.w_cell + off[k]);
+    if (kAllVectors || p.b_cell) bc[k] = C::load(p.b_cell + off[k]);
+    if (kAllVectors || p.w_state) ws[k] = C::load(p.w_state + off[k]);
+    if (kAllVectors || p.b_state) bs[k] = C::load(p.b_state + off[k]);
   }
 #pragma unroll
   for (int k = 0; k < K; ++k) {
+    zc[k] = C::load_stream(z_row + (kSharedZ ? 0 : 3 * gate_bytes) + off[k]);
     sc[k] = C::load_stream(s_row + 3 * gate_bytes + off[k]);
-    zc[k] = C::load_stream(z_row + 3 * gate_bytes + off[k]);
   }
 #pragma unroll
   for (int k = 0; k < K; ++k) {
     sf[k] = C::load_stream(s_row + off[k]);
-    zf[k] = C::load_stream(z_row + off[k]);
+    zf[k] = kSharedZ ? zc[k] : C::load_stream(z_row + off[k]);
   }
 #pragma unroll
   for (int k = 0; k < K; ++k) pc[k] = C::load_stream(pc_row + off[k]);
 #pragma unroll
   for (int k = 0; k < K; ++k) {
     si[k] = C::load_stream(s_row + gate_bytes + off[k]);
-    zi[k] = C::load_stream(z_row + gate_bytes + off[k]);
+    zi[k] = kSharedZ ? zc[k] : C::load_stream(z_row + gate_bytes + off[k]);
   }
 #pragma unroll
   for (int k = 0; k < K; ++k) {
     so[k] = C::load_stream(s_row + 2 * gate_bytes + off[k]);
-    zo[k] = C::load_stream(z_row + 2 * gate_bytes + off[k]);
+    zo[k] = kSharedZ ? zc[k] : C::load_stream(z_row + 2 * gate_bytes + off[k]);
   }
 
   // Lanes beyond the row take part in the sums with zeros.  (Each value is
@@ -162,15 +166,20 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
   // candidate = gelu(rmsnorm(pre_c)): runs while the other gates are still arriving
 #pragma unroll
   for (int k = 0; k < K; ++k) {
+    // an absent scale / shift vector acts as 1 / 0 (exact), so the norm is one multiply and
+    // one fused multiply-add per element whichever vectors were given
     float w[E], b[E];
-    if (p.w_cell) wc[k].template unpack<T>(w);
-    if (p.b_cell) bc[k].template unpack<T>(b);
+#pragma unroll
+    for (int j = 0; j < E; ++j) {
+      w[j] = 1.f;
+      b[j] = 0.f;
+    }
+    if (kAllVectors || p.w_cell) wc[k].template unpack<T>(w);
+    if (kAllVectors || p.b_cell) bc[k].template unpack<T>(b);
     const float mask = live[k] ? 1.f : 0.f;  // idle lanes must add nothing to the second sum
 #pragma unroll
     for (int j = 0; j < E; ++j) {
-      float cn = cact[k][j] * inv_cpre;
-      if (p.w_cell) cn *= w[j];
-      if (p.b_cell) cn += b[j];
+      const float cn = fmaf(cact[k][j] * inv_cpre, w[j], b[j]);
       cact[k][j] = gelu<kFastGelu>(cn) * mask;
     }
   }
@@ -206,15 +215,15 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
 #pragma unroll
   for (int k = 0; k < K; ++k) {
     float w[E], b[E], st[E];
-    if (p.w_state) ws[k].template unpack<T>(w);
-    if (p.b_state) bs[k].template unpack<T>(b);
 #pragma unroll
     for (int j = 0; j < E; ++j) {
-      float cn = cell[k][j] * inv_cnew;
-      if (p.w_state) cn *= w[j];
-      if (p.b_state) cn += b[j];
-      st[j] = gelu<kFastGelu>(cn);
+      w[j] = 1.f;
+      b[j] = 0.f;
     }
+    if (kAllVectors || p.w_state) ws[k].template unpack<T>(w);
+    if (kAllVectors || p.b_state) bs[k].template unpack<T>(b);
+#pragma unroll
+    for (int j = 0; j < E; ++j) st[j] = gelu<kFastGelu>(fmaf(cell[k][j] * inv_cnew, w[j], b[j]));
     float a[E], g[E];
     so[k].template unpack<T>(a);
     zo[k].template unpack<T>(g);
@@ -227,7 +236,7 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
 // Any D, any alignment: element-wise, three passes like the reference's scalar
 // kernel (sum_lstm.cu:193-291).
 template <typename T, bool kFastGelu>
-__global__ __launch_bounds__(256) void sum_lstm_scalar_kernel(const LstmParams p) {
+__global__ __launch_bounds__(256) void sum_lstm_scalar_kernel(const LstmParams p, const int z_gate_stride) {
   __shared__ float slots_cpre[16];
   __shared__ float slots_cnew[16];
   const int D = p.D;
@@ -242,7 +251,7 @@ __global__ __launch_bounds__(256) void sum_lstm_scalar_kernel(const LstmParams p
 
   float ss = 0.f;
   for (int j = threadIdx.x; j < D; j += blockDim.x) {
-    const float c = T::lo(s[3 * (int64_t)D + j]) + p.alpha * T::lo(z[3 * (int64_t)D + j]);
+    const float c = T::lo(s[3 * (int64_t)D + j]) + p.alpha * T::lo(z[3 * (int64_t)z_gate_stride + j]);
     ss += c * c;
   }
   const float inv_cpre = rsqrtf(block_sum(ss, slots_cpre) * p.inv_D + p.eps_cell);
@@ -250,8 +259,8 @@ __global__ __launch_bounds__(256) void sum_lstm_scalar_kernel(const LstmParams p
   ss = 0.f;
   for (int j = threadIdx.x; j < D; j += blockDim.x) {
     const float pre_f = T::lo(s[j]) + p.alpha * T::lo(z[j]);
-    const float pre_i = T::lo(s[(int64_t)D + j]) + p.alpha * T::lo(z[(int64_t)D + j]);
-    const float cpre = T::lo(s[3 * (int64_t)D + j]) + p.alpha * T::lo(z[3 * (int64_t)D + j]);
+    const float pre_i = T::lo(s[(int64_t)D + j]) + p.alpha * T::lo(z[(int64_t)z_gate_stride + j]);
+    const float cpre = T::lo(s[3 * (int64_t)D + j]) + p.alpha * T::lo(z[3 * (int64_t)z_gate_stride + j]);
     float cn = cpre * inv_cpre;
     if (wc) cn *= T::lo(wc[j]);
     if (bc) cn += T::lo(bc[j]);
@@ -266,14 +275,14 @@ __global__ __launch_bounds__(256) void sum_lstm_scalar_kernel(const LstmParams p
     float cn = T::lo(oc[j]) * inv_cnew;
     if (ws) cn *= T::lo(ws[j]);
     if (bs) cn += T::lo(bs[j]);
-    const float pre_o = T::lo(s[2 * (int64_t)D + j]) + p.alpha * T::lo(z[2 * (int64_t)D + j]);
+    const float pre_o = T::lo(s[2 * (int64_t)D + j]) + p.alpha * T::lo(z[2 * (int64_t)z_gate_stride + j]);
     os[j] = (uint16_t)T::round_bits(gelu<kFastGelu>(cn) * sigmoid_f(pre_o));
   }
 }
 
 static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
-template <typename T, bool kFastGelu>
+template <typename T, bool kFastGelu, bool kSharedZ>
 static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
   const int chunks = p.D / 8;
   const bool multi = rows > 1;
@@ -285,20 +294,18 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
                    aligned16(p.b_cell) && aligned16(p.w_state) && aligned16(p.b_state);
   const dim3 grid((unsigned)rows);
   if (vec) {
-    const int units = p.D / 8;
-    const int cpt = units > 512 ? 2 : 1;   // one 16-byte chunk per lane up to 512 lanes (D <= 4096)
-    int threads = (units + cpt - 1) / cpt;
+    const int cpt = chunks > 512 ? 2 : 1;   // one 16-byte chunk per lane up to 512 lanes (D <= 4096)
+    int threads = (chunks + cpt - 1) / cpt;
     threads = std::max(64, (threads + 63) & ~63);
-    unsigned lds = 0;
-#ifdef ARCTIC_TUNING
-    if (const char *e = getenv("ARCTIC_LSTM_LDS")) lds = (unsigned)atoi(e);
-#endif
-    if (cpt == 1)
-      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512>), grid, dim3(threads), lds, s, p);
+    const bool all = p.w_cell && p.b_cell && p.w_state && p.b_state && threads * cpt == chunks;
+    if (cpt == 1 && all)
+      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, true>), grid, dim3(threads), 0, s, p);
+    else if (cpt == 1)
+      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, false>), grid, dim3(threads), 0, s, p);
     else
-      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 2, kFastGelu, 1024>), grid, dim3(threads), lds, s, p);
+      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 2, kFastGelu, 1024, kSharedZ, false>), grid, dim3(threads), 0, s, p);
   } else {
-    hipLaunchKernelGGL((sum_lstm_scalar_kernel<T, kFastGelu>), grid, dim3(256), 0, s, p);
+    hipLaunchKernelGGL((sum_lstm_scalar_kernel<T, kFastGelu>), grid, dim3(256), 0, s, p, kSharedZ ? 0 : p.D);
   }
 }
 
@@ -306,25 +313,23 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
 
 using namespace arctic;
 
-extern "C" int arctic_sum_lstm(void *out_state, void *out_cell, const void *states, const void *z4,
-                               const void *prev_cell, const void *w_cell, const void *b_cell,
-                               const void *w_state, const void *b_state, int64_t rows, int D,
-                               int64_t s_stride, int64_t z_stride, int64_t pc_stride, int64_t out_stride,
-                               float alpha, float eps_cell, float eps_state, int fast_gelu, int dtype,
-                               void *stream) {
-  const char *fn = "sum_lstm";
+static int sum_lstm_entry(const char *fn, bool shared_z, void *out_state, void *out_cell, const void *states,
+                          const void *z, const void *prev_cell, const void *w_cell, const void *b_cell,
+                          const void *w_state, const void *b_state, int64_t rows, int D, int64_t s_stride,
+                          int64_t z_stride, int64_t pc_stride, int64_t out_stride, float alpha, float eps_cell,
+                          float eps_state, int fast_gelu, int dtype, void *stream) {
   if (dtype != ARCTIC_DTYPE_F16 && dtype != ARCTIC_DTYPE_BF16)
     return fail(ARCTIC_ERR_UNSUPPORTED, "%s: only fp16 and bf16 are supported.", fn);
   if (D <= 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: last dim of states must be 4*D_gate", fn);
   if (rows < 0 || rows > 0x7fffffffLL) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: bad row count", fn);
   if (rows == 0) return ARCTIC_OK;
-  if (!out_state || !out_cell || !states || !z4 || !prev_cell)
+  if (!out_state || !out_cell || !states || !z || !prev_cell)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
   LstmParams p;
   p.out_state = (char *)out_state;
   p.out_cell = (char *)out_cell;
   p.states = (const char *)states;
-  p.z4 = (const char *)z4;
+  p.z4 = (const char *)z;
   p.prev_cell = (const char *)prev_cell;
   p.w_cell = (const char *)w_cell;
   p.b_cell = (const char *)b_cell;
@@ -340,12 +345,40 @@ extern "C" int arctic_sum_lstm(void *out_state, void *out_cell, const void *stat
   p.eps_cell = eps_cell;
   p.eps_state = eps_state;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == ARCTIC_DTYPE_BF16) {
-    if (fast_gelu) launch_lstm<BF16, true>(p, rows, s);
-    else launch_lstm<BF16, false>(p, rows, s);
-  } else {
-    if (fast_gelu) launch_lstm<F16, true>(p, rows, s);
-    else launch_lstm<F16, false>(p, rows, s);
-  }
+#define ARCTIC_LSTM_DISPATCH(TYPE)                                        \
+  do {                                                                    \
+    if (shared_z) {                                                       \
+      if (fast_gelu) launch_lstm<TYPE, true, true>(p, rows, s);           \
+      else launch_lstm<TYPE, false, true>(p, rows, s);                    \
+    } else {                                                              \
+      if (fast_gelu) launch_lstm<TYPE, true, false>(p, rows, s);          \
+      else launch_lstm<TYPE, false, false>(p, rows, s);                   \
+    }                                                                     \
+  } while (0)
+  if (dtype == ARCTIC_DTYPE_BF16) ARCTIC_LSTM_DISPATCH(BF16);
+  else ARCTIC_LSTM_DISPATCH(F16);
+#undef ARCTIC_LSTM_DISPATCH
   return check_launch(fn);
+}
+
+extern "C" int arctic_sum_lstm(void *out_state, void *out_cell, const void *states, const void *z4,
+                               const void *prev_cell, const void *w_cell, const void *b_cell,
+                               const void *w_state, const void *b_state, int64_t rows, int D,
+                               int64_t s_stride, int64_t z_stride, int64_t pc_stride, int64_t out_stride,
+                               float alpha, float eps_cell, float eps_state, int fast_gelu, int dtype,
+                               void *stream) {
+  return sum_lstm_entry("sum_lstm", false, out_state, out_cell, states, z4, prev_cell, w_cell, b_cell, w_state,
+                        b_state, rows, D, s_stride, z_stride, pc_stride, out_stride, alpha, eps_cell, eps_state,
+                        fast_gelu, dtype, stream);
+}
+
+extern "C" int arctic_sum_lstm_shared_z(void *out_state, void *out_cell, const void *states, const void *z,
+                                        const void *prev_cell, const void *w_cell, const void *b_cell,
+                                        const void *w_state, const void *b_state, int64_t rows, int D,
+                                        int64_t s_stride, int64_t z_stride, int64_t pc_stride,
+                                        int64_t out_stride, float alpha, float eps_cell, float eps_state,
+                                        int fast_gelu, int dtype, void *stream) {
+  return sum_lstm_entry("sum_lstm_shared_z", true, out_state, out_cell, states, z, prev_cell, w_cell, b_cell,
+                        w_state, b_state, rows, D, s_stride, z_stride, pc_stride, out_stride, alpha, eps_cell,
+                        eps_state, fast_gelu, dtype, stream);
 }

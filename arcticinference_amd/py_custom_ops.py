@@ -45,6 +45,14 @@ _SCHEMAS = {
         "float eps_state, bool use_fast_gelu) -> (Tensor, Tensor)",
 }
 
+# Operators that fuse a caller-side step into one of the above; the reference has no such schema.
+_EXTRA_SCHEMAS = {
+    "sum_lstm_shared_z_cuda":
+        "sum_lstm_shared_z_cuda(Tensor states_4d, Tensor z_d, Tensor prev_cell_d, Tensor? w_cell, "
+        "Tensor? b_cell, Tensor? w_state, Tensor? b_state, float alpha, float eps_cell, "
+        "float eps_state, bool use_fast_gelu) -> (Tensor, Tensor)",
+}
+
 _SRC_DTYPES = {
     torch.float32: _native.DTYPE_F32,
     torch.float16: _native.DTYPE_F16,
@@ -283,8 +291,10 @@ def _sum_lstm_impl(
     eps_cell: float,
     eps_state: float,
     use_fast_gelu: bool,
+    _shared_z: bool = False,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Host side of sum_lstm_cuda (csrc/custom_ops/sum_lstm.cu:293-473)."""
+    """Host side of sum_lstm_cuda (csrc/custom_ops/sum_lstm.cu:293-473).  With _shared_z the
+    second argument is the un-repeated [..., D] embedding row (see sum_lstm_shared_z)."""
     lib = _lib()
     dtype = states_4d.dtype
     _check(dtype in _HALF_DTYPES, "sum_lstm: only fp16 and bf16 are supported.")
@@ -295,7 +305,10 @@ def _sum_lstm_impl(
     hidden4 = states_4d.size(-1)
     _check(hidden4 > 0 and hidden4 % 4 == 0, "sum_lstm: last dim of states must be 4*D_gate")
     d_gate = hidden4 // 4
-    _check(z4_4d.size(-1) == hidden4, "sum_lstm: z4 must have last dim 4*D_gate")
+    if _shared_z:
+        _check(z4_4d.size(-1) == d_gate, "sum_lstm_shared_z: z must have last dim D_gate")
+    else:
+        _check(z4_4d.size(-1) == hidden4, "sum_lstm: z4 must have last dim 4*D_gate")
     d_cell = prev_cell_d.size(-1)
     _check(d_cell == d_gate,
            f"sum_lstm: prev_cell last dim must equal D_gate. Got {d_cell} vs expected {d_gate}.")
@@ -309,7 +322,7 @@ def _sum_lstm_impl(
             _check(t.is_contiguous(), f"sum_lstm: {name} must be contiguous")
 
     s2 = states_4d.view(-1, hidden4)
-    z2 = z4_4d.view(-1, hidden4)
+    z2 = z4_4d.view(-1, d_gate if _shared_z else hidden4)
     p2 = prev_cell_d.view(-1, d_cell)
     rows = s2.size(0)
     _check(z2.size(0) == rows and p2.size(0) == rows, "sum_lstm: row counts of the inputs differ")
@@ -325,8 +338,9 @@ def _sum_lstm_impl(
     def ptr(t):
         return t.data_ptr() if t is not None else None
 
+    entry = lib.arctic_sum_lstm_shared_z if _shared_z else lib.arctic_sum_lstm
     with _on_device_of(states_4d):
-        rc = lib.arctic_sum_lstm(
+        rc = entry(
             out_state.data_ptr(), out_cell.data_ptr(), s2.data_ptr(), z2.data_ptr(), p2.data_ptr(),
             ptr(w_cell), ptr(b_cell), ptr(w_state), ptr(b_state),
             rows, d_gate, s2.stride(0), z2.stride(0), p2.stride(0), out_cell.stride(0),
@@ -336,7 +350,14 @@ def _sum_lstm_impl(
     return out_state_orig, out_cell_orig
 
 
+def _sum_lstm_shared_z_impl(states_4d, z_d, prev_cell_d, w_cell, b_cell, w_state, b_state, alpha, eps_cell,
+                            eps_state, use_fast_gelu):
+    return _sum_lstm_impl(states_4d, z_d, prev_cell_d, w_cell, b_cell, w_state, b_state, alpha, eps_cell,
+                          eps_state, use_fast_gelu, _shared_z=True)
+
+
 _IMPLS = {
+    "sum_lstm_shared_z_cuda": _sum_lstm_shared_z_impl,
     "reshape_and_cache_flash_bulk": _reshape_and_cache_flash_bulk_impl,
     "reshape_and_cache_flash_fp4": _reshape_and_cache_flash_fp4_impl,
     "speculator_ln_cuda": _speculator_ln_impl,
@@ -351,7 +372,7 @@ def _register_ops() -> None:
     if _registered:
         return
     lib = torch.library.Library(_NAMESPACE, "DEF")
-    for name, schema in _SCHEMAS.items():
+    for name, schema in {**_SCHEMAS, **_EXTRA_SCHEMAS}.items():
         lib.define(schema)
         lib.impl(name, _IMPLS[name], "CUDA")
     _torch_lib = lib  # keep alive: dropping the Library object unregisters the ops
@@ -455,3 +476,24 @@ def sum_lstm(
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     return _ops().sum_lstm_cuda(states_4d, z4_4d, prev_cell_d, w_cell, b_cell, w_state, b_state,
                                 alpha, eps_cell, eps_state, use_fast_gelu)
+
+
+def sum_lstm_shared_z(
+    states_4d: torch.Tensor,
+    z_d: torch.Tensor,
+    prev_cell_d: torch.Tensor,
+    w_cell: Optional[torch.Tensor],
+    b_cell: Optional[torch.Tensor],
+    w_state: Optional[torch.Tensor],
+    b_state: Optional[torch.Tensor],
+    alpha: float,
+    eps_cell: float,
+    eps_state: float,
+    use_fast_gelu: bool,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``sum_lstm(states_4d, z_d.repeat(..., 4), ...)`` without building the repeated tensor:
+    the speculator's ``z4 = forget_emb(tokens).repeat(1, 1, 4)``
+    (arctic_inference/vllm/spec_dec/arctic_speculator.py:744) folded into the operator.
+    Bit-identical to the two-step form; reads 6*D fewer bytes per row."""
+    return _ops().sum_lstm_shared_z_cuda(states_4d, z_d, prev_cell_d, w_cell, b_cell, w_state, b_state,
+                                         alpha, eps_cell, eps_state, use_fast_gelu)

@@ -169,11 +169,20 @@ def bench_speculator(ops, dev, steps, warmup):
             _, cell = ops.sum_lstm(S[i % sets][k], Z[i % sets][k], cell, w_cell, b_cell, w_state, b_state,
                                    alpha, 1e-6, 1e-6, False)
 
+    def lstm3_shared_z(i):
+        # the same three steps with the embedding row passed once ([T, H]) instead of repeated four times
+        cell = C0[i % sets]
+        for k in range(3):
+            _, cell = ops.sum_lstm_shared_z(S[i % sets][k], Z[i % sets][k][:, :Hd], cell, w_cell, b_cell, w_state,
+                                            b_state, alpha, 1e-6, 1e-6, False)
+
     def ln(i):
         ops.speculator_ln(X[i % sets], w_cell, b_cell, 1e-6)
 
     out = {}
-    for name, fn, per_call, calls in (("sum_lstm", lstm3, 22 * Hd * T, 3), ("speculator_ln", ln, 4 * Hd * T, 1)):
+    for name, fn, per_call, calls in (("sum_lstm", lstm3, 22 * Hd * T, 3),
+                                      ("sum_lstm_shared_z", lstm3_shared_z, 16 * Hd * T, 3),
+                                      ("speculator_ln", ln, 4 * Hd * T, 1)):
         for i in range(warmup):
             fn(i)
         torch.cuda.synchronize()

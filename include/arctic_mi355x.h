@@ -170,6 +170,23 @@ int arctic_sum_lstm(void *out_state, void *out_cell, const void *states,
                     float alpha, float eps_cell, float eps_state, int fast_gelu,
                     int dtype, void *stream);
 
+/*
+ * sum_lstm with the embedding term given ONCE per token.  The speculator builds
+ *   z4 = forget_emb(tokens).repeat(1, 1, 4)       arctic_inference/vllm/spec_dec/arctic_speculator.py:744
+ * i.e. the same [rows, D] row under all four gates, and passes it to sum_lstm.  This entry
+ * point takes that [rows, D] row itself (z, rows z_stride ELEMENTS apart) and adds it to every
+ * gate; everything else, and every output bit, is as arctic_sum_lstm with z4 = repeat(z, 4).
+ * It fuses the caller's repeat() into the operator (6*D fewer bytes read per row and no z4
+ * tensor); the reference has no operator of this shape.
+ */
+int arctic_sum_lstm_shared_z(void *out_state, void *out_cell, const void *states,
+                             const void *z, const void *prev_cell, const void *w_cell,
+                             const void *b_cell, const void *w_state,
+                             const void *b_state, int64_t rows, int D, int64_t s_stride,
+                             int64_t z_stride, int64_t pc_stride, int64_t out_stride,
+                             float alpha, float eps_cell, float eps_state, int fast_gelu,
+                             int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

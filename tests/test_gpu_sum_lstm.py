@@ -71,6 +71,29 @@ def test_config4_three_steps(ops, alpha):
         assert same > 0.97, f"step {step}: only {same:.4f} of the cells are bit-identical to the oracle"
 
 
+@pytest.mark.parametrize("cfg", [dict(rows=64, D=512, pad4=16, padD=8), dict(rows=4, D=128, pad4=7, padD=3),
+                                 dict(rows=512, D=4096, pad4=0, padD=0), dict(rows=3, D=8200, pad4=0, padD=0)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_shared_z_equals_repeated_z(ops, cfg, dtype):
+    """sum_lstm_shared_z(states, z) must give the very bits of sum_lstm(states, z.repeat(1, 4)),
+    and both must match the oracle run on the repeated tensor."""
+    c = make_lstm_case(dtype=dtype, seed=99, repeat_z=True, **cfg)
+    D = cfg["D"]
+    z = c["z4"][:, :D].contiguous()
+    assert torch.equal(c["z4"], z.repeat(1, 4))
+    alpha = 0.35
+    args = [dev(c[k]) for k in ("prev_cell", "w_cell", "b_cell", "w_state", "b_state")]
+    st_r, ce_r = ops.sum_lstm(dev(c["states"]), dev(c["z4"]), *args, alpha, 1e-6, 1e-6, False)
+    st_s, ce_s = ops.sum_lstm_shared_z(dev(c["states"]), z.to(DEV), *args, alpha, 1e-6, 1e-6, False)
+    torch.cuda.synchronize()
+    assert st_s.stride() == c["prev_cell"].stride()
+    assert torch.equal(st_s, st_r) and torch.equal(ce_s, ce_r)
+    want_s, want_c = oracle.sum_lstm(c["states"], c["z4"], c["prev_cell"], c["w_cell"], c["b_cell"], c["w_state"],
+                                     c["b_state"], alpha, 1e-6, 1e-6, False)
+    assert_close(ce_s, want_c, RTOL, ATOL, "cell (shared z)")
+    assert_close(st_s, want_s, RTOL, ATOL, "state (shared z)")
+
+
 def test_rank3_inputs(ops):
     c = make_lstm_case(rows=6, D=256, seed=8)
     for k in ("states", "z4", "prev_cell"):

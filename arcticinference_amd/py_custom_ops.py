@@ -78,7 +78,14 @@ def _lib() -> ctypes.CDLL:
     return _native.load()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_of(t: torch.Tensor) -> int:
+    """hipStream_t of torch's current stream on the tensor's device (what
+    at::cuda::getCurrentCUDAStream() is to the reference)."""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
@@ -119,8 +126,11 @@ def _kv_dtype_code(src_dtype: torch.dtype, kv_cache_dtype: str) -> Tuple[int, in
     return _SRC_DTYPES[src_dtype], kv
 
 
+_data_ptr = torch.Tensor.data_ptr
+
+
 def _ptr_table(tensors: List[torch.Tensor]):
-    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+    return (ctypes.c_void_p * len(tensors))(*map(_data_ptr, tensors))
 
 
 def _reshape_and_cache_flash_bulk_impl(
@@ -170,12 +180,12 @@ def _reshape_and_cache_flash_bulk_impl(
            f"reshape_and_cache_flash_bulk: cache element size {cache_elem} does not match "
            f"kv_cache_dtype '{kv_cache_dtype}' (expected {want_elem})")
     if kv_code != _native.KV_AUTO:
-        _check(all(s.dtype == torch.float32 for s in k_scales) and
-               all(s.dtype == torch.float32 for s in v_scales),
+        _check({s.dtype for s in k_scales} == {torch.float32} and {s.dtype for s in v_scales} == {torch.float32},
                "reshape_and_cache_flash_bulk: k_scales / v_scales must be float32")
-    dev = keys.device
-    _check(all(t.device == dev for t in (values, slot_mapping, *key_caches, *value_caches)),
-           "reshape_and_cache_flash_bulk: all tensors must be on the same device")
+    devices = {t.device for t in key_caches}
+    devices.update(t.device for t in value_caches)
+    devices.update((values.device, slot_mapping.device, keys.device))
+    _check(len(devices) == 1, "reshape_and_cache_flash_bulk: all tensors must be on the same device")
 
     with _on_device_of(keys):
         rc = lib.arctic_reshape_and_cache_flash_bulk(

@@ -6,8 +6,20 @@
 A step is one bulk KV-cache write (one launch of the hot path) over the 70B
 SwiftKV shape (the benchmark's headline workload): 16384 tokens, 40 layers, 8 KV heads
 x 128, block 16, fp8-e4m3 cache with per-tensor amax/448 scales, 10 % of the
-slots are padding.  Inputs are resident in HBM before the timed region.  The
-last stdout line is ONE JSON object:
+slots are padding.  Inputs are resident in HBM before the timed region.
+
+The caches sit where they sit in the serving process the shape comes from
+(Llama-3.3-70B SwiftKV, fp8, one MI355X): the resident weights are allocated first
+(66 GiB, a placeholder that is never touched), then vLLM's paged KV pool, one
+[2, num_blocks, 16, 8, 128] tensor per layer for all 80 layers (65536 blocks =
+2 GiB per layer), and the bulk write fills the upper 40 layers, as
+llama_swiftkv.py:599-622 does.  This matters on MI355X: its HBM answers in three
+address regions of 96 GiB, stores into one region top out near 4.9 TB/s while stores
+spread over two or three reach 6.9 TB/s, so the same kernel is 15-20 % slower when
+every cache is packed into the first 13 GiB of an otherwise empty GPU.  That
+compact placement is measured too and reported under extras.
+
+The last stdout line is ONE JSON object:
 
   value / ms_per_step   wall clock around exactly K steps (sync on both sides)
   roofline              the kernel's own duration from HIP events recorded on the
@@ -50,7 +62,7 @@ def make_slots(num_tokens, num_slots, gen, pad_fraction):
 class BulkWorkload:
     """One bulk KV-write configuration, resident on the GPU."""
 
-    def __init__(self, name, T, L, H, D, bs, NB, kv, pad_fraction, seed, std, dev):
+    def __init__(self, name, T, L, H, D, bs, NB, kv, pad_fraction, seed, std, dev, bufs=None):
         self.name, self.T, self.L, self.H, self.D, self.bs, self.NB, self.kv = name, T, L, H, D, bs, NB, kv
         n = H * D
         self.n = n
@@ -68,7 +80,9 @@ class BulkWorkload:
         self.valid = int((self.slots_cpu >= 0).sum())
         quant = kv != "auto"
         cdt = torch.uint8 if quant else torch.bfloat16
-        self.bufs = [torch.zeros(2, NB, bs, H, D, dtype=cdt, device=dev) for _ in range(L)]
+        # bufs: the layers' [2, NB, bs, H, D] cache tensors when they already exist (a serving pool)
+        self.bufs = bufs if bufs is not None else [torch.zeros(2, NB, bs, H, D, dtype=cdt, device=dev) for _ in range(L)]
+        assert len(self.bufs) == L and tuple(self.bufs[0].shape) == (2, NB, bs, H, D) and self.bufs[0].dtype == cdt
         self.key_caches = [b[0] for b in self.bufs]
         self.value_caches = [b[1] for b in self.bufs]
         if quant:
@@ -84,6 +98,34 @@ class BulkWorkload:
     def args(self):
         return (self.keys, self.values, self.key_caches, self.value_caches, self.slots, self.kv,
                 self.k_scales, self.v_scales, self.H, self.D)
+
+
+class ServingMemoryMap:
+    """Device memory laid out as the serving process lays it out: resident weights first (a placeholder
+    that is never touched), then one [2, num_blocks, block, heads, head_size] cache tensor per model
+    layer, the way vLLM's FlashAttention backend allocates its paged pool.  SwiftKV's bulk write fills
+    the layers from num_key_value_layers up (llama_swiftkv.py:599-622)."""
+
+    def __init__(self, dev, weight_gib, model_layers, first_written_layer, NB, bs, H, D, cdt):
+        self.weight_gib, self.model_layers, self.first_written_layer, self.NB = weight_gib, model_layers, first_written_layer, NB
+        self.weights = torch.empty(weight_gib << 30, dtype=torch.uint8, device=dev)
+        self.pool = [torch.empty(2, NB, bs, H, D, dtype=cdt, device=dev) for _ in range(model_layers)]
+        self.pool_gib = sum(b.numel() * b.element_size() for b in self.pool) / 2 ** 30
+
+    def written_layers(self):
+        return self.pool[self.first_written_layer:]
+
+    def describe(self):
+        return (f"{self.weight_gib} GiB resident weights (placeholder) allocated first, then the paged KV pool of all "
+                f"{self.model_layers} layers, {self.NB} blocks = {self.pool_gib / self.model_layers:.0f} GiB per layer "
+                f"({self.pool_gib:.0f} GiB); layers {self.first_written_layer}-{self.model_layers - 1} are written; "
+                f"K/V source allocated after the pool")
+
+
+def kernel_stats(fn, steps, nbytes):
+    us = event_times_us(fn, steps)
+    m = statistics.median(us)
+    return {"kernel_us": round(m, 2), "GBps": round(nbytes / m / 1e3, 1), "hbm_frac": round(nbytes / m / 1e3 / HBM_PEAK_GBS, 4)}
 
 
 def event_times_us(fn, iters):
@@ -306,6 +348,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--weight-gib", type=int, default=66, help="resident-weights placeholder allocated before the KV pool")
+    ap.add_argument("--pool-blocks", type=int, default=65536, help="blocks per layer of the 80-layer KV pool")
     ap.add_argument("--no-extras", action="store_true", help="skip the speculator / decode-mix measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -325,7 +369,25 @@ def main():
     torch.cuda.set_device(dev)
     log(f"device: {torch.cuda.get_device_name(0)}; host cores: {os.cpu_count()}")
 
-    w = BulkWorkload("70B-SwiftKV", 16384, 40, 8, 128, 16, 8192, "fp8", 0.10, 2, 1.5, dev)
+    extras = {}
+    if not args.no_extras:
+        # the same shape with nothing else on the GPU: 40 caches of 8192 blocks (10 GiB) right behind the
+        # source, all inside one HBM region
+        wc = BulkWorkload("70B-SwiftKV-compact", 16384, 40, 8, 128, 16, 8192, "fp8", 0.10, 2, 1.5, dev)
+        fc = lambda: ops.reshape_and_cache_flash_bulk(*wc.args())
+        for _ in range(args.warmup):
+            fc()
+        extras["bulk_fp8_70b_compact_pool"] = dict(
+            kernel_stats(fc, args.steps, wc.bytes),
+            placement="source and 40 caches of 8192 blocks allocated alone on an empty GPU (13 GiB, one HBM region)")
+        log(f"compact placement: {extras['bulk_fp8_70b_compact_pool']}")
+        del wc, fc
+        torch.cuda.empty_cache()
+
+    mem = ServingMemoryMap(dev, args.weight_gib, 80, 40, args.pool_blocks, 16, 8, 128, torch.uint8)
+    log(f"memory map: {mem.describe()}")
+    w = BulkWorkload("70B-SwiftKV", 16384, 40, 8, 128, 16, args.pool_blocks, "fp8", 0.10, 2, 1.5, dev,
+                     bufs=mem.written_layers())
     fn = lambda: ops.reshape_and_cache_flash_bulk(*w.args())
     for _ in range(args.warmup):
         fn()
@@ -360,7 +422,15 @@ def main():
         cpu = cpu_baseline_bulk(w)
         log(f"cpu baseline: {cpu}")
 
-    extras = {}
+    workload_text = (f"bulk KV write at the 70B SwiftKV shape: {w.T} tokens x {w.L} layers x {w.H} KV heads x {w.D}, "
+                     f"block {w.bs}, fp8-e4m3 cache, amax/448 scales, 10% slots = -1, the rest distinct random "
+                     f"slots of a {w.NB}-block pool")
+    cfg = {"workload": workload_text, "tokens": w.T, "valid_tokens": w.valid, "layers": w.L, "kv_heads": w.H,
+           "head_size": w.D, "block_size": w.bs, "num_blocks": w.NB, "memory_map": mem.describe(),
+           "parallelism": "single GPU"}
+    del w, fn, mem
+    torch.cuda.empty_cache()
+
     if not args.no_extras:
         w2 = BulkWorkload("8B-prefill", 8192, 16, 8, 128, 16, 8192, "fp8", 0.0, 1, 1.5, dev)
         f2 = lambda: ops.reshape_and_cache_flash_bulk(*w2.args())
@@ -368,7 +438,8 @@ def main():
             f2()
         m = statistics.median(event_times_us(f2, args.steps))
         extras["bulk_fp8_8b_prefill"] = {"kernel_us": round(m, 2), "GBps": round(w2.bytes / m / 1e3, 1),
-                                         "hbm_frac": round(w2.bytes / m / 1e3 / HBM_PEAK_GBS, 4)}
+                                         "hbm_frac": round(w2.bytes / m / 1e3 / HBM_PEAK_GBS, 4),
+                                         "placement": "source and 16 caches of 8192 blocks allocated alone (one HBM region)"}
         del w2, f2
         torch.cuda.empty_cache()
         extras["box_reference"] = box_reference(dev)
@@ -384,10 +455,7 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "fp8_e4m3",
         "data": "synthetic",
-        "config": {"workload": "bulk KV write at the 70B SwiftKV shape: 16384 tokens x 40 layers x 8 KV heads x 128, "
-                               "block 16, 8192 blocks, fp8-e4m3 cache, amax/448 scales, 10% slots = -1",
-                   "tokens": w.T, "valid_tokens": w.valid, "layers": w.L, "kv_heads": w.H, "head_size": w.D,
-                   "block_size": w.bs, "num_blocks": w.NB, "parallelism": "single GPU"},
+        "config": cfg,
         "roofline": roofline, "cpu_baseline": cpu, "extras": extras,
     }
     print(json.dumps(result), flush=True)

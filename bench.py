@@ -343,6 +343,77 @@ def bench_decode_mix(ops, dev, steps):
             "GBps": round(nbytes / med / 1e3, 1), "hbm_frac": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
 
 
+def placement_sweep(ops, dev, steps):
+    """Where the caches sit in HBM against how fast the same launch runs.  The GPU's memory is taken in 32
+    chunks of 8 GiB (allocation order follows physical order on an otherwise empty GPU); the 70B-shape
+    source sits in one chunk and the 80 caches (4096 blocks each, 5 GiB) in another.  Scan 1 keeps the
+    source in chunk 0 and moves the caches through every chunk: the chunks that run slow share chunk 0's
+    region.  Scan 2 repeats that from the first fast chunk, which separates the other two regions.  The
+    last cases spread the caches of one launch over the regions found."""
+    T, L, H, D, bs, NB = 16384, 40, 8, 128, 16, 4096
+    n = H * D
+    nchunks, chunk_bytes = 32, 8 << 30
+    chunks = [torch.empty(chunk_bytes, dtype=torch.uint8, device=dev) for _ in range(nchunks)]
+    src_bytes, cache_bytes = T * L * n * 2, NB * bs * n
+    gd = torch.Generator(device=dev).manual_seed(2)
+    slots_cpu = make_slots(T, NB * bs, torch.Generator().manual_seed(2), 0.10)
+    slots = slots_cpu.to(dev)
+    nbytes = int((slots_cpu >= 0).sum()) * L * n * 6
+    scales = [torch.full((), 0.0134, device=dev) for _ in range(L)]
+
+    def source(c):
+        kv = chunks[c][:2 * src_bytes].view(torch.bfloat16).view(2, T, L * n)
+        for t0 in range(0, T, 512):
+            kv[:, t0:t0 + 512] = (torch.randn(2, 512, L * n, generator=gd, device=dev) * 1.5).to(torch.bfloat16)
+        return kv[0], kv[1]
+
+    def cache(c, index, base):
+        off = base + index * cache_bytes
+        return chunks[c][off:off + cache_bytes].view(NB, bs, H, D)
+
+    def timed(k, v, kc, vc):
+        f = lambda: ops.reshape_and_cache_flash_bulk(k, v, kc, vc, slots, "fp8", scales, scales, H, D)
+        for _ in range(3):
+            f()
+        return round(statistics.median(event_times_us(f, steps)), 1)
+
+    def scan(src_chunk):
+        k, v = source(src_chunk)
+        row = []
+        for c in range(nchunks):
+            base = 2 * src_bytes if c == src_chunk else 0
+            row.append(timed(k, v, [cache(c, 2 * l, base) for l in range(L)], [cache(c, 2 * l + 1, base) for l in range(L)]))
+        return row
+
+    scan0 = scan(0)
+    cut = (min(scan0) + max(scan0)) / 2
+    region_a = [c for c in range(nchunks) if scan0[c] > cut]
+    first_fast = next(c for c in range(nchunks) if scan0[c] <= cut)
+    scan1 = scan(first_fast)
+    cut1 = (min(scan1) + max(scan1)) / 2
+    region_b = [c for c in range(nchunks) if scan1[c] > cut1]
+    region_c = [c for c in range(nchunks) if c not in region_a and c not in region_b]
+    out = {"chunk_gib": 8, "us_source_in_chunk_0": scan0, f"us_source_in_chunk_{first_fast}": scan1,
+           "regions": [region_a, region_b, region_c], "bytes_per_launch": nbytes}
+    if region_a and region_b and region_c:
+        k, v = source(0)
+        reps = [region_a[len(region_a) // 2], region_b[len(region_b) // 2], region_c[len(region_c) // 2]]
+        base = 2 * src_bytes
+        cases = {
+            "one_region (source's own)": [reps[0]] * L,
+            "one_region (another)": [reps[1]] * L,
+            "layers_alternate_over_2_regions": [reps[l % 2] for l in range(L)],
+            "layers_alternate_over_3_regions": [reps[l % 3] for l in range(L)],
+            "lower_half_in_one_upper_half_in_another": [reps[1] if l < L // 2 else reps[2] for l in range(L)],
+        }
+        out["spread_cases_us"] = {
+            name: timed(k, v, [cache(where[l], 2 * l, base) for l in range(L)],
+                        [cache(where[l], 2 * l + 1, base) for l in range(L)])
+            for name, where in cases.items()}
+        out["spread_cases_GBps"] = {name: round(nbytes / us / 1e3) for name, us in out["spread_cases_us"].items()}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -352,6 +423,9 @@ def main():
     ap.add_argument("--pool-blocks", type=int, default=65536, help="blocks per layer of the 80-layer KV pool")
     ap.add_argument("--no-extras", action="store_true", help="skip the speculator / decode-mix measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--placement-sweep", action="store_true",
+                    help="instead of the benchmark, time the 70B-shape launch with the caches in each 8 GiB chunk "
+                         "of the GPU's memory and spread over its regions; prints one JSON object")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) so that a counter run of this "
                          "command can scale FETCH_SIZE / WRITE_SIZE")
@@ -368,6 +442,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     log(f"device: {torch.cuda.get_device_name(0)}; host cores: {os.cpu_count()}")
+
+    if args.placement_sweep:
+        print(json.dumps({"placement_sweep": placement_sweep(ops, dev, max(5, args.steps // 5))}), flush=True)
+        return
 
     extras = {}
     if not args.no_extras:

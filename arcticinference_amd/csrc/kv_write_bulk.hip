@@ -374,18 +374,25 @@ extern "C" int arctic_reshape_and_cache_flash_bulk(
     p.chunk_shift = -1;
     if (vec && (p.chunks_per_row & (p.chunks_per_row - 1)) == 0) p.chunk_shift = __builtin_ctz(p.chunks_per_row);
 
-    // One workgroup per token is best when there are thousands of tokens.  With
-    // few tokens (decode) a token's layers are split over several workgroups so
-    // that about eight workgroups per CU exist, each still moving at least one
-    // full batch of 1024 chunks.
+    // A token's layers are split over `groups` workgroups.  Measured best on gfx950: the 512-lane shape
+    // with 2-5 batches of 1024 chunks per workgroup (20 layers of 8 x 128 bf16 at most) and at least
+    // about 1024 workgroups; when so few tokens come that a workgroup would get less than two batches
+    // (decode), the 256-lane shape with about 2048 workgroups of at least one batch each.
     int groups = 1;
     bool wide = false;
     if (vec) {
       const int64_t chunks_per_layer = 2LL * p.chunks_per_row;
-      const int min_layers = (int)std::max<int64_t>(1, (1024 + chunks_per_layer - 1) / chunks_per_layer);
-      const int64_t want = (2048 + num_tokens - 1) / num_tokens;
-      groups = (int)std::max<int64_t>(1, std::min<int64_t>(want, count / min_layers));
-      wide = num_tokens >= 4096 && chunks_per_layer * count >= 8 * 1024;
+      int64_t g = std::max<int64_t>((1024 + num_tokens - 1) / num_tokens, (chunks_per_layer * count + 5119) / 5120);
+      g = std::max<int64_t>(1, std::min<int64_t>(g, count));
+      const int64_t layers_per_group = (count + g - 1) / g;
+      if (layers_per_group * chunks_per_layer >= 2048) {
+        wide = true;
+        groups = (int)g;
+      } else {
+        const int min_layers = (int)std::max<int64_t>(1, (1024 + chunks_per_layer - 1) / chunks_per_layer);
+        const int64_t want = (2048 + num_tokens - 1) / num_tokens;
+        groups = (int)std::max<int64_t>(1, std::min<int64_t>(want, count / min_layers));
+      }
     } else {
       groups = (int)std::max<int64_t>(1, std::min<int64_t>(count, (2048 + num_tokens - 1) / num_tokens));
     }

@@ -157,6 +157,20 @@ def test_long_prefill_launch_shape(ops, kv):
     run_both(ops, case)
 
 
+@pytest.mark.parametrize("T,L,kv", [
+    (300, 41, "fp8"),    # three layer groups per token, the last one a layer short (14 + 14 + 13)
+    (300, 41, "auto"),
+    (96, 70, "fp8"),     # two launches (64 + 6 layers); the first splits into four groups of 16
+    (2100, 23, "fp8_e5m2"),   # two groups of 12 and 11 layers
+])
+def test_layer_groups_with_a_ragged_tail(ops, T, L, kv):
+    """Layers of one token split over several workgroups of the 512-lane shape, layer count not a
+    multiple of the group size; compared in full against the oracle."""
+    case = make_bulk_case(T=T, L=L, H=8, D=128, bs=16, NB=(T + 15) // 16 + 3, kv_cache_dtype=kv, seed=31, std=1.5,
+                          pad_fraction=0.1)
+    run_both(ops, case)
+
+
 def test_random_configurations(ops):
     """Seeded sweep over shapes, dtypes, layouts, pitches and padding: exercises the layer
     grouping, the power-of-two and general row decompositions, the multi-launch split and

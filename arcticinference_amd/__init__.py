@@ -9,7 +9,9 @@ __version__ = "0.1.0"
 from . import py_custom_ops  # noqa: F401
 from .py_custom_ops import (  # noqa: F401
     reshape_and_cache_flash_bulk,
+    speculator_add_ln_gelu,
     speculator_ln,
+    speculator_ln_scaled,
     sum_lstm,
     try_load_jit_library,
     try_load_torch_library,

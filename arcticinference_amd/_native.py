@@ -27,6 +27,7 @@ EXPORTED_SYMBOLS = (
     "arctic_reshape_and_cache_flash_bulk",
     "arctic_reshape_and_cache_flash_fp4",
     "arctic_speculator_ln",
+    "arctic_speculator_add_ln_act",
     "arctic_sum_lstm",
     "arctic_sum_lstm_shared_z",
 )
@@ -80,6 +81,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.arctic_reshape_and_cache_flash_fp4.restype = i32
     lib.arctic_speculator_ln.argtypes = [vp, vp, vp, vp, i64, i32, i64, f32, i32, vp]
     lib.arctic_speculator_ln.restype = i32
+    lib.arctic_speculator_add_ln_act.argtypes = [vp, vp, vp, vp, vp, i64, i32, i64, i64, f32, f32, i32, f32, i32, vp]
+    lib.arctic_speculator_add_ln_act.restype = i32
     lib.arctic_sum_lstm.argtypes = [vp] * 9 + [i64, i32, i64, i64, i64, i64, f32, f32, f32, i32, i32, vp]
     lib.arctic_sum_lstm.restype = i32
     lib.arctic_sum_lstm_shared_z.argtypes = lib.arctic_sum_lstm.argtypes

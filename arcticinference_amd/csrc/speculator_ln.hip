@@ -7,19 +7,48 @@
 // chunks of the row in registers between the sum of squares and the scaling, so
 // the row is read from HBM once (the reference reads it twice); the sum is a DPP
 // wave reduction followed by a small LDS combine.
+//
+// The same kernel also carries the element-wise steps the speculator runs around
+// this norm (arctic_speculator.py:296-307,733-734,809-816), each with the rounding
+// of the separate PyTorch op it stands for:
+//   x   = round(in + alpha * z)        states.add_(z, alpha=...)      (optional)
+//   y   = round(x * inv_rms * w + b)   speculator_ln
+//   y   = round(gelu(y))               nn.GELU()                      (optional)
+//   out = round(y * out_scale)         ln0(x) / sqrt(2)               (optional)
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
 
+#include "activations.hpp"
 #include "common.hpp"
 
 namespace arctic {
 
-template <typename T, int kChunksPerThread>
+// What surrounds the norm; all fields are uniform over the launch.
+struct LnGlue {
+  const char *z;            // nullptr: no add
+  int64_t z_row_stride_bytes;
+  float alpha;
+  int activation;           // ARCTIC_ACT_*
+  float out_scale;          // applied when != 1
+};
+
+template <typename T>
+__device__ __forceinline__ float glue_tail(float y, const LnGlue &g) {
+  if (g.activation != ARCTIC_ACT_NONE) {
+    y = T::requant(y);
+    y = g.activation == ARCTIC_ACT_GELU ? gelu_erf(y) : gelu_tanh(y);
+  }
+  if (g.out_scale != 1.0f) y = T::requant(y) * g.out_scale;
+  return y;
+}
+
+template <typename T, int kChunksPerThread, bool kGlue>
 __global__ __launch_bounds__(1024) void spec_ln_vec_kernel(
     char *__restrict__ out, const char *__restrict__ in, const char *__restrict__ weight,
-    const char *__restrict__ bias, int64_t in_row_stride_bytes, int hidden, float inv_hidden, float eps) {
+    const char *__restrict__ bias, int64_t in_row_stride_bytes, int hidden, float inv_hidden, float eps,
+    LnGlue glue) {
   __shared__ float slots[16];
   const int chunks = hidden >> 3;
   const char *row_in = in + (int64_t)blockIdx.x * in_row_stride_bytes;
@@ -40,6 +69,25 @@ __global__ __launch_bounds__(1024) void spec_ln_vec_kernel(
     const int c = threadIdx.x + k * blockDim.x;
     raw[k] = make_uint4(0, 0, 0, 0);
     if (c < chunks) raw[k] = load16_stream(row_in + (int64_t)c * 16);
+  }
+  if (kGlue && glue.z) {
+    const char *row_z = glue.z + (int64_t)blockIdx.x * glue.z_row_stride_bytes;
+    uint4 zr[kChunksPerThread];
+#pragma unroll
+    for (int k = 0; k < kChunksPerThread; ++k) {
+      const int c = threadIdx.x + k * blockDim.x;
+      zr[k] = make_uint4(0, 0, 0, 0);
+      if (c < chunks) zr[k] = load16_stream(row_z + (int64_t)c * 16);
+    }
+#pragma unroll
+    for (int k = 0; k < kChunksPerThread; ++k) {
+      float x[8], z[8];
+      unpack8<T>(raw[k], x);
+      unpack8<T>(zr[k], z);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[j] = fmaf(glue.alpha, z[j], x[j]);
+      raw[k] = pack8<T>(x);   // the sum stands in the tensor's own type, as after the in-place add
+    }
   }
 #pragma unroll
   for (int k = 0; k < kChunksPerThread; ++k) {
@@ -71,6 +119,10 @@ __global__ __launch_bounds__(1024) void spec_ln_vec_kernel(
 #pragma unroll
       for (int j = 0; j < 8; ++j) x[j] += b[j];
     }
+    if (kGlue) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[j] = glue_tail<T>(x[j], glue);
+    }
     store16_stream(row_out + (int64_t)c * 16, pack8<T>(x));
   }
 }
@@ -79,22 +131,30 @@ __global__ __launch_bounds__(1024) void spec_ln_vec_kernel(
 template <typename T>
 __global__ __launch_bounds__(256) void spec_ln_scalar_kernel(
     uint16_t *__restrict__ out, const uint16_t *__restrict__ in, const uint16_t *__restrict__ weight,
-    const uint16_t *__restrict__ bias, int64_t in_row_stride, int hidden, float inv_hidden, float eps) {
+    const uint16_t *__restrict__ bias, int64_t in_row_stride, int hidden, float inv_hidden, float eps,
+    LnGlue glue) {
   __shared__ float slots[16];
   const uint16_t *row_in = in + (int64_t)blockIdx.x * in_row_stride;
+  const uint16_t *row_z =
+      glue.z ? (const uint16_t *)(glue.z + (int64_t)blockIdx.x * glue.z_row_stride_bytes) : nullptr;
   uint16_t *row_out = out + (int64_t)blockIdx.x * hidden;
+  auto element = [&](int j) {
+    float x = T::lo(row_in[j]);
+    if (row_z) x = T::requant(fmaf(glue.alpha, T::lo(row_z[j]), x));
+    return x;
+  };
   float ss = 0.f;
   for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
-    const float x = T::lo(row_in[j]);
+    const float x = element(j);
     ss += x * x;
   }
   const float total = block_sum(ss, slots);
   const float inv = rsqrtf(total * inv_hidden + eps);
   for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
-    float y = T::lo(row_in[j]) * inv;
+    float y = element(j) * inv;
     if (weight) y *= T::lo(weight[j]);
     if (bias) y += T::lo(bias[j]);
-    row_out[j] = (uint16_t)T::round_bits(y);
+    row_out[j] = (uint16_t)T::round_bits(glue_tail<T>(y, glue));
   }
 }
 
@@ -102,11 +162,13 @@ static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 template <typename T>
 static void launch_ln(void *out, const void *in, const void *w, const void *b, int64_t rows, int hidden,
-                      int64_t in_row_stride, float eps, hipStream_t s) {
+                      int64_t in_row_stride, float eps, const LnGlue &glue, hipStream_t s) {
   const int chunks = hidden / 8;
   const float inv_hidden = 1.0f / (float)hidden;
   const bool vec = (hidden % 8 == 0) && (in_row_stride % 8 == 0 || rows == 1) && aligned16(in) &&
-                   aligned16(out) && (!w || aligned16(w)) && (!b || aligned16(b)) && chunks <= 8 * 1024;
+                   aligned16(out) && (!w || aligned16(w)) && (!b || aligned16(b)) && chunks <= 8 * 1024 &&
+                   (!glue.z || (aligned16(glue.z) && (glue.z_row_stride_bytes % 16 == 0 || rows == 1)));
+  const bool plain = !glue.z && glue.activation == ARCTIC_ACT_NONE && glue.out_scale == 1.0f;
   const dim3 grid((unsigned)rows);
   if (vec) {
     int cpt = 1;
@@ -114,9 +176,17 @@ static void launch_ln(void *out, const void *in, const void *w, const void *b, i
     int threads = (chunks + cpt - 1) / cpt;
     threads = std::max(64, (threads + 63) & ~63);
     const int64_t stride_bytes = in_row_stride * 2;
-#define ARCTIC_LN_LAUNCH(CPT)                                                                         \
-  hipLaunchKernelGGL((spec_ln_vec_kernel<T, CPT>), grid, dim3(threads), 0, s, (char *)out,             \
-                     (const char *)in, (const char *)w, (const char *)b, stride_bytes, hidden, inv_hidden, eps)
+#define ARCTIC_LN_LAUNCH(CPT)                                                                              \
+  do {                                                                                                     \
+    if (plain)                                                                                             \
+      hipLaunchKernelGGL((spec_ln_vec_kernel<T, CPT, false>), grid, dim3(threads), 0, s, (char *)out,       \
+                         (const char *)in, (const char *)w, (const char *)b, stride_bytes, hidden,          \
+                         inv_hidden, eps, glue);                                                           \
+    else                                                                                                   \
+      hipLaunchKernelGGL((spec_ln_vec_kernel<T, CPT, true>), grid, dim3(threads), 0, s, (char *)out,        \
+                         (const char *)in, (const char *)w, (const char *)b, stride_bytes, hidden,          \
+                         inv_hidden, eps, glue);                                                           \
+  } while (0)
     switch (cpt) {
       case 1: ARCTIC_LN_LAUNCH(1); break;
       case 2: ARCTIC_LN_LAUNCH(2); break;
@@ -127,7 +197,7 @@ static void launch_ln(void *out, const void *in, const void *w, const void *b, i
   } else {
     hipLaunchKernelGGL((spec_ln_scalar_kernel<T>), grid, dim3(256), 0, s, (uint16_t *)out,
                        (const uint16_t *)in, (const uint16_t *)w, (const uint16_t *)b, in_row_stride, hidden,
-                       inv_hidden, eps);
+                       inv_hidden, eps, glue);
   }
 }
 
@@ -135,20 +205,38 @@ static void launch_ln(void *out, const void *in, const void *w, const void *b, i
 
 using namespace arctic;
 
-extern "C" int arctic_speculator_ln(void *out, const void *in, const void *weight, const void *bias,
-                                    int64_t rows, int hidden, int64_t in_row_stride, float eps, int dtype,
-                                    void *stream) {
-  const char *fn = "speculator_ln";
+static int ln_entry(const char *fn, void *out, const void *in, const void *weight, const void *bias,
+                    int64_t rows, int hidden, int64_t in_row_stride, float eps, const LnGlue &glue, int dtype,
+                    void *stream) {
   if (dtype != ARCTIC_DTYPE_F16 && dtype != ARCTIC_DTYPE_BF16)
     return fail(ARCTIC_ERR_UNSUPPORTED, "%s: only fp16 and bf16 are supported.", fn);
   if (hidden <= 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: hidden size must be > 0", fn);
   if (rows < 0 || rows > 0x7fffffffLL) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: bad row count", fn);
+  if (glue.activation != ARCTIC_ACT_NONE && glue.activation != ARCTIC_ACT_GELU &&
+      glue.activation != ARCTIC_ACT_GELU_TANH)
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: unknown activation %d", fn, glue.activation);
   if (rows == 0) return ARCTIC_OK;
   if (!out || !in) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
   hipStream_t s = (hipStream_t)stream;
   if (dtype == ARCTIC_DTYPE_BF16)
-    launch_ln<BF16>(out, in, weight, bias, rows, hidden, in_row_stride, eps, s);
+    launch_ln<BF16>(out, in, weight, bias, rows, hidden, in_row_stride, eps, glue, s);
   else
-    launch_ln<F16>(out, in, weight, bias, rows, hidden, in_row_stride, eps, s);
+    launch_ln<F16>(out, in, weight, bias, rows, hidden, in_row_stride, eps, glue, s);
   return check_launch(fn);
+}
+
+extern "C" int arctic_speculator_ln(void *out, const void *in, const void *weight, const void *bias,
+                                    int64_t rows, int hidden, int64_t in_row_stride, float eps, int dtype,
+                                    void *stream) {
+  const LnGlue none = {nullptr, 0, 0.0f, ARCTIC_ACT_NONE, 1.0f};
+  return ln_entry("speculator_ln", out, in, weight, bias, rows, hidden, in_row_stride, eps, none, dtype, stream);
+}
+
+extern "C" int arctic_speculator_add_ln_act(void *out, const void *in, const void *z, const void *weight,
+                                            const void *bias, int64_t rows, int hidden, int64_t in_row_stride,
+                                            int64_t z_row_stride, float alpha, float eps, int activation,
+                                            float out_scale, int dtype, void *stream) {
+  const LnGlue glue = {(const char *)z, z_row_stride * 2, alpha, activation, out_scale};
+  return ln_entry("speculator_add_ln_act", out, in, weight, bias, rows, hidden, in_row_stride, eps, glue, dtype,
+                  stream);
 }

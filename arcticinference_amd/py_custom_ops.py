@@ -43,6 +43,9 @@ _SCHEMAS = {
         "sum_lstm_cuda(Tensor states_4d, Tensor z4_4d, Tensor prev_cell_d, Tensor? w_cell, "
         "Tensor? b_cell, Tensor? w_state, Tensor? b_state, float alpha, float eps_cell, "
         "float eps_state, bool use_fast_gelu) -> (Tensor, Tensor)",
+    "speculator_add_ln_act_cuda":
+        "speculator_add_ln_act_cuda(Tensor input, Tensor? z, Tensor? weight, Tensor? bias, float alpha, "
+        "float eps, str activation, float out_scale) -> Tensor",
 }
 
 # Operators that fuse a caller-side step into one of the above; the reference has no such schema.
@@ -51,6 +54,9 @@ _EXTRA_SCHEMAS = {
         "sum_lstm_shared_z_cuda(Tensor states_4d, Tensor z_d, Tensor prev_cell_d, Tensor? w_cell, "
         "Tensor? b_cell, Tensor? w_state, Tensor? b_state, float alpha, float eps_cell, "
         "float eps_state, bool use_fast_gelu) -> (Tensor, Tensor)",
+    "speculator_add_ln_act_cuda":
+        "speculator_add_ln_act_cuda(Tensor input, Tensor? z, Tensor? weight, Tensor? bias, float alpha, "
+        "float eps, str activation, float out_scale) -> Tensor",
 }
 
 _SRC_DTYPES = {
@@ -249,17 +255,22 @@ def _reshape_and_cache_flash_fp4_impl(
     _native.check(rc)
 
 
-def _speculator_ln_impl(input: torch.Tensor, weight: Optional[torch.Tensor],
-                        bias: Optional[torch.Tensor], eps: float) -> torch.Tensor:
-    """Host side of speculator_ln_cuda (csrc/custom_ops/speculator_ln.cu:152-252)."""
+_ACTIVATIONS = {"none": 0, "gelu": 1, "gelu_tanh": 2}
+
+
+def _ln_common(fn: str, input: torch.Tensor, z: Optional[torch.Tensor], weight: Optional[torch.Tensor],
+               bias: Optional[torch.Tensor], alpha: float, eps: float, activation: str,
+               out_scale: float) -> torch.Tensor:
+    """Argument checks and launch shared by speculator_ln_cuda and speculator_add_ln_act_cuda
+    (the checks are those of csrc/custom_ops/speculator_ln.cu:152-201)."""
     lib = _lib()
-    _check(input.dtype in _HALF_DTYPES, "speculator_ln: only fp16 and bf16 are supported.")
-    _check(input.is_cuda, "speculator_ln: input must be CUDA")
+    _check(input.dtype in _HALF_DTYPES, f"{fn}: only fp16 and bf16 are supported.")
+    _check(input.is_cuda, f"{fn}: input must be CUDA")
     dtype = input.dtype
     hidden = input.size(-1)
-    _check(hidden > 0, "speculator_ln: hidden size must be > 0")
+    _check(hidden > 0, f"{fn}: hidden size must be > 0")
     _check(input.stride(-1) == 1,
-           "speculator_ln: last dimension must be contiguous (stride -1 == 1)")
+           f"{fn}: last dimension must be contiguous (stride -1 == 1)")
     if weight is not None:
         _check(weight.is_cuda, "weight must be CUDA")
         _check(weight.dtype == dtype, "weight dtype must match input dtype")
@@ -270,23 +281,50 @@ def _speculator_ln_impl(input: torch.Tensor, weight: Optional[torch.Tensor],
         _check(bias.dtype == dtype, "bias dtype must match input dtype")
         _check(bias.dim() == 1 and bias.numel() == hidden, "bias must be 1D of size hidden")
         _check(bias.is_contiguous(), "bias must be contiguous")
+    _check(activation in _ACTIVATIONS, f"{fn}: activation must be one of {sorted(_ACTIVATIONS)}")
 
     in_2d = input.view(-1, hidden)
     rows = in_2d.size(0)
     row_stride = in_2d.stride(0)
+    z_2d = None
+    if z is not None:
+        _check(z.is_cuda and z.device == input.device, "z must be CUDA, on the input's device")
+        _check(z.dtype == dtype, "z dtype must match input dtype")
+        _check(z.shape == input.shape, "z must have the input's shape")
+        _check(z.stride(-1) == 1, f"{fn}: last dimension of z must be contiguous")
+        z_2d = z.view(-1, hidden)
     out = torch.empty_like(input)
     out_2d = out.view(-1, hidden)  # rows are written dense, `hidden` apart
     if rows == 0:
         return out
-    _check(out_2d.stride(0) == hidden or rows == 1, "speculator_ln: internal - output rows must be dense")
+    _check(out_2d.stride(0) == hidden or rows == 1, f"{fn}: internal - output rows must be dense")
+    w_ptr = weight.data_ptr() if weight is not None else None
+    b_ptr = bias.data_ptr() if bias is not None else None
     with _on_device_of(input):
-        rc = lib.arctic_speculator_ln(
-            out_2d.data_ptr(), in_2d.data_ptr(),
-            weight.data_ptr() if weight is not None else None,
-            bias.data_ptr() if bias is not None else None,
-            rows, hidden, row_stride, float(eps), _HALF_DTYPES[dtype], _stream_of(input))
+        if z is None and activation == "none" and out_scale == 1.0:
+            rc = lib.arctic_speculator_ln(out_2d.data_ptr(), in_2d.data_ptr(), w_ptr, b_ptr, rows, hidden,
+                                          row_stride, float(eps), _HALF_DTYPES[dtype], _stream_of(input))
+        else:
+            rc = lib.arctic_speculator_add_ln_act(
+                out_2d.data_ptr(), in_2d.data_ptr(), z_2d.data_ptr() if z_2d is not None else None, w_ptr, b_ptr,
+                rows, hidden, row_stride, z_2d.stride(0) if z_2d is not None else 0, float(alpha), float(eps),
+                _ACTIVATIONS[activation], float(out_scale), _HALF_DTYPES[dtype], _stream_of(input))
     _native.check(rc)
     return out
+
+
+def _speculator_ln_impl(input: torch.Tensor, weight: Optional[torch.Tensor],
+                        bias: Optional[torch.Tensor], eps: float) -> torch.Tensor:
+    """Host side of speculator_ln_cuda (csrc/custom_ops/speculator_ln.cu:152-252)."""
+    return _ln_common("speculator_ln", input, None, weight, bias, 0.0, eps, "none", 1.0)
+
+
+def _speculator_add_ln_act_impl(input: torch.Tensor, z: Optional[torch.Tensor], weight: Optional[torch.Tensor],
+                                bias: Optional[torch.Tensor], alpha: float, eps: float, activation: str,
+                                out_scale: float) -> torch.Tensor:
+    """The norm with the speculator's element-wise steps around it in one launch
+    (arctic_inference/vllm/spec_dec/arctic_speculator.py:296-307, 733-734, 809-816)."""
+    return _ln_common("speculator_add_ln_act", input, z, weight, bias, alpha, eps, activation, out_scale)
 
 
 def _sum_lstm_impl(
@@ -368,6 +406,7 @@ def _sum_lstm_shared_z_impl(states_4d, z_d, prev_cell_d, w_cell, b_cell, w_state
 
 _IMPLS = {
     "sum_lstm_shared_z_cuda": _sum_lstm_shared_z_impl,
+    "speculator_add_ln_act_cuda": _speculator_add_ln_act_impl,
     "reshape_and_cache_flash_bulk": _reshape_and_cache_flash_bulk_impl,
     "reshape_and_cache_flash_fp4": _reshape_and_cache_flash_fp4_impl,
     "speculator_ln_cuda": _speculator_ln_impl,
@@ -507,3 +546,31 @@ def sum_lstm_shared_z(
     Bit-identical to the two-step form; reads 6*D fewer bytes per row."""
     return _ops().sum_lstm_shared_z_cuda(states_4d, z_d, prev_cell_d, w_cell, b_cell, w_state, b_state,
                                          alpha, eps_cell, eps_state, use_fast_gelu)
+
+
+def speculator_add_ln_gelu(
+    states: torch.Tensor,
+    z: torch.Tensor,
+    weight: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor],
+    alpha: float,
+    eps: float,
+) -> torch.Tensor:
+    """``gelu(ln(states + alpha * z))`` in one launch: the MLP / sum_rnn speculator's
+    ``states.add_(z, alpha=emb_weight / state_weight); activation(ln(states))``
+    (arctic_inference/vllm/spec_dec/arctic_speculator.py:300-307, 809-816), rounded after each
+    step like the three separate ops.  ``states`` is left unchanged."""
+    return _ops().speculator_add_ln_act_cuda(states, z, weight, bias, alpha, eps, "gelu", 1.0)
+
+
+def speculator_ln_scaled(
+    input: torch.Tensor,
+    weight: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor],
+    eps: float,
+    out_scale: float,
+) -> torch.Tensor:
+    """``speculator_ln(input, weight, bias, eps) * out_scale`` in one launch: the speculator's
+    ``ln0(previous_hidden_states) / SQRT2`` with ``out_scale = 1 / SQRT2``
+    (arctic_inference/vllm/spec_dec/arctic_speculator.py:296-297, 733-734)."""
+    return _ops().speculator_add_ln_act_cuda(input, None, weight, bias, 0.0, eps, "none", out_scale)

@@ -221,10 +221,21 @@ def bench_speculator(ops, dev, steps, warmup):
     def ln(i):
         ops.speculator_ln(X[i % sets], w_cell, b_cell, 1e-6)
 
+    def add_ln_gelu(i):
+        # the MLP / sum_rnn speculator's states.add_(z, alpha); gelu(ln(states)) in one launch
+        ops.speculator_add_ln_gelu(X[i % sets], C0[i % sets], w_cell, b_cell, alpha, 1e-6)
+
+    def add_ln_gelu_separate(i):
+        s = X[i % sets]
+        s.add_(C0[i % sets], alpha=1e-3)
+        torch.nn.functional.gelu(ops.speculator_ln(s, w_cell, b_cell, 1e-6))
+
     out = {}
     for name, fn, per_call, calls in (("sum_lstm", lstm3, 22 * Hd * T, 3),
                                       ("sum_lstm_shared_z", lstm3_shared_z, 16 * Hd * T, 3),
-                                      ("speculator_ln", ln, 4 * Hd * T, 1)):
+                                      ("speculator_ln", ln, 4 * Hd * T, 1),
+                                      ("speculator_add_ln_gelu", add_ln_gelu, 6 * Hd * T, 1),
+                                      ("add_ln_gelu_as_three_ops", add_ln_gelu_separate, 6 * Hd * T, 1)):
         for i in range(warmup):
             fn(i)
         torch.cuda.synchronize()

@@ -39,6 +39,11 @@ extern "C" {
 #define ARCTIC_KV_FP8_E4M3 1
 #define ARCTIC_KV_FP8_E5M2 2
 
+/* activation codes of arctic_speculator_add_ln_act */
+#define ARCTIC_ACT_NONE 0
+#define ARCTIC_ACT_GELU 1      /* erf form, nn.GELU() */
+#define ARCTIC_ACT_GELU_TANH 2 /* tanh form */
+
 #define ARCTIC_OK 0
 #define ARCTIC_ERR_INVALID_ARGUMENT 1
 #define ARCTIC_ERR_UNSUPPORTED 2
@@ -138,6 +143,31 @@ int arctic_speculator_ln(void *out, const void *in, const void *weight,
                          const void *bias, int64_t rows, int hidden,
                          int64_t in_row_stride, float eps, int dtype,
                          void *stream);
+
+/*
+ * The same norm with the element-wise steps the speculator runs around it folded
+ * in.  No single function of the reference corresponds to it; it stands for the
+ * PyTorch sequences
+ *   states.add_(z, alpha=emb_weight / state_weight); activation(ln(states))
+ *        arctic_inference/vllm/spec_dec/arctic_speculator.py:296-307, 809-816
+ *   ln0(previous_hidden_states) / SQRT2
+ *        arctic_inference/vllm/spec_dec/arctic_speculator.py:296-297, 733-734
+ * and rounds to `dtype` wherever those sequences hold a tensor of that type:
+ *   x = z ? round(in + alpha * z) : in
+ *   y = round(x * rsqrt(mean(x^2) + eps) [* weight] [+ bias])
+ *   if (activation) y = round(gelu(y));   if (out_scale != 1) y = round(y * out_scale)
+ * `in` is not modified.
+ *
+ *   z            device; rows of `hidden` elements, z_row_stride ELEMENTS apart, or NULL
+ *   activation   ARCTIC_ACT_*
+ *   other arguments as arctic_speculator_ln
+ */
+int arctic_speculator_add_ln_act(void *out, const void *in, const void *z,
+                                 const void *weight, const void *bias,
+                                 int64_t rows, int hidden, int64_t in_row_stride,
+                                 int64_t z_row_stride, float alpha, float eps,
+                                 int activation, float out_scale, int dtype,
+                                 void *stream);
 
 /*
  * Fused LSTM-style gate / cell / state update.  Replaces

@@ -75,6 +75,8 @@ def lib() -> ctypes.CDLL:
         L.ao_reshape_and_cache_flash_fp4.restype = i32
         L.ao_speculator_ln.argtypes = [vp, vp, vp, vp, i64, i32, i64, f32, i32]
         L.ao_speculator_ln.restype = i32
+        L.ao_speculator_add_ln_act.argtypes = [vp, vp, vp, vp, vp, i64, i32, i64, i64, f32, f32, i32, f32, i32]
+        L.ao_speculator_add_ln_act.restype = i32
         L.ao_sum_lstm.argtypes = [vp] * 9 + [i64, i32, i64, i64, i64, i64, f32,
                                              f32, f32, i32, i32]
         L.ao_sum_lstm.restype = i32
@@ -217,6 +219,37 @@ def speculator_ln(input: torch.Tensor, weight: Optional[torch.Tensor],
         in2.stride(0) if in2.size(0) > 1 else hidden, float(eps), _SRC_DTYPE[input.dtype])
     if rc != 0:
         raise RuntimeError("oracle: speculator_ln supports fp16/bf16 only")
+    return out
+
+
+_ACTIVATION = {"none": 0, "gelu": 1, "gelu_tanh": 2}
+
+
+def speculator_add_ln_act(input: torch.Tensor, z: Optional[torch.Tensor], weight: Optional[torch.Tensor],
+                          bias: Optional[torch.Tensor], alpha: float, eps: float, activation: str,
+                          out_scale: float) -> torch.Tensor:
+    """``act(ln(input + alpha * z)) * out_scale`` with the roundings of the separate PyTorch ops
+    (arctic_inference/vllm/spec_dec/arctic_speculator.py:296-307, 733-734, 809-816)."""
+    _cpu(input, "input")
+    hidden = input.size(-1)
+    assert input.stride(-1) == 1
+    in2 = input.view(-1, hidden)
+    z2 = None
+    if z is not None:
+        _cpu(z, "z")
+        assert z.shape == input.shape and z.dtype == input.dtype and z.stride(-1) == 1
+        z2 = z.view(-1, hidden)
+    out = torch.empty(input.shape, dtype=input.dtype)
+    w = weight.contiguous() if weight is not None else None
+    b = bias.contiguous() if bias is not None else None
+    rows = in2.size(0)
+    rc = lib().ao_speculator_add_ln_act(
+        out.data_ptr(), in2.data_ptr(), z2.data_ptr() if z2 is not None else None,
+        w.data_ptr() if w is not None else None, b.data_ptr() if b is not None else None, rows, hidden,
+        in2.stride(0) if rows > 1 else hidden, (z2.stride(0) if rows > 1 else hidden) if z2 is not None else 0,
+        float(alpha), float(eps), _ACTIVATION[activation], float(out_scale), _SRC_DTYPE[input.dtype])
+    if rc != 0:
+        raise RuntimeError("oracle: speculator_add_ln_act supports fp16/bf16 and activations none/gelu/gelu_tanh")
     return out
 
 

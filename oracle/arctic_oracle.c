@@ -122,6 +122,11 @@ static inline uint16_t store_half(float v, int dtype) {
   return dtype == AO_F16 ? ao_f32_to_f16(v) : ao_f32_to_bf16(v);
 }
 
+/* value of v after a round trip through the 16-bit type */
+static inline float requant(float v, int dtype) {
+  return dtype == AO_F16 ? ao_f16_to_f32(ao_f32_to_f16(v)) : ao_bf16_to_f32(ao_f32_to_bf16(v));
+}
+
 /* ---- fp8 encode / decode --------------------------------------------------
  * The reference's scaled_vec_conversion<uint8_t, *> ends in
  *   __nv_cvt_float_to_fp8(x / scale, __NV_SATFINITE, __NV_E4M3 | __NV_E5M2)
@@ -385,6 +390,49 @@ static inline float gelu_erf(float x) {
 static inline float gelu_tanh(float x) {
   return 0.5f * x *
          (1.0f + tanhf(0.79788456080286535588f * (x + 0.044715f * x * x * x)));
+}
+
+/* The speculator's element-wise steps around its norm, as one function: the
+ * PyTorch sequences of arctic_inference/vllm/spec_dec/arctic_speculator.py
+ *   :300-307, :809-816   states.add_(z, alpha=a); activation(ln(states))
+ *   :296-297, :733-734   ln0(previous_hidden_states) / SQRT2
+ * Every PyTorch op of those sequences leaves a 16-bit tensor, so the value is
+ * rounded to the 16-bit type after the add, after the norm (ao_speculator_ln's own
+ * rounding), after the GELU and after the scaling.  The add is a + alpha*b with a
+ * single rounding in fp32 (what the GPU's add kernel computes); nn.GELU() is the
+ * erf form evaluated in fp32; a tensor divided by a Python scalar is multiplied by
+ * the fp32 reciprocal, which the caller passes as out_scale.
+ * activation: 0 none, 1 erf GELU, 2 tanh GELU. */
+int ao_speculator_add_ln_act(void *out, const void *in, const void *z, const void *w,
+                             const void *b, int64_t rows, int hidden,
+                             int64_t in_row_stride, int64_t z_row_stride, float alpha,
+                             float eps, int activation, float out_scale, int dtype) {
+  if (dtype != AO_F16 && dtype != AO_BF16) return -1;
+  if (activation < 0 || activation > 2) return -2;
+  uint16_t *o = (uint16_t *)out;
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    float *x = (float *)malloc(sizeof(float) * (size_t)hidden);
+    float ss = 0.f;
+    for (int j = 0; j < hidden; ++j) {
+      float v = load_as_f32(in, r * in_row_stride + j, dtype);
+      if (z) v = requant(fmaf(alpha, load_as_f32(z, r * z_row_stride + j, dtype), v), dtype);
+      x[j] = v;
+      ss += v * v;
+    }
+    const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
+    for (int j = 0; j < hidden; ++j) {
+      float y = x[j] * inv;
+      if (w) y *= load_as_f32(w, j, dtype);
+      if (b) y += load_as_f32(b, j, dtype);
+      y = requant(y, dtype);
+      if (activation) y = requant(activation == 1 ? gelu_erf(y) : gelu_tanh(y), dtype);
+      if (out_scale != 1.0f) y = requant(y * out_scale, dtype);
+      o[r * (int64_t)hidden + j] = store_half(y, dtype);
+    }
+    free(x);
+  }
+  return 0;
 }
 
 /* Restates sum_lstm_vec_kernel / sum_lstm_scalar_kernel

@@ -79,3 +79,90 @@ def test_errors(ops):
         ops.speculator_ln(xb, torch.ones(64, device=DEV, dtype=torch.bfloat16), None, 1e-6)
     with pytest.raises(RuntimeError, match="bias must be 1D of size hidden"):
         ops.speculator_ln(xb, None, torch.ones(1, 128, device=DEV, dtype=torch.bfloat16), 1e-6)
+
+
+# --------------------------------------------------------------------------- #
+# speculator_add_ln_act: add + norm + GELU / scaling in one launch
+# --------------------------------------------------------------------------- #
+def glue_inputs(rows, hidden, dtype, seed, pad=0):
+    g = torch.Generator().manual_seed(seed)
+    x = pitched(rows, hidden, pad, dtype, g, std=1.3)
+    z = pitched(rows, hidden, pad, dtype, g)
+    w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    return x, z, w, b
+
+
+def same_fraction(a, b):
+    return (a.cpu().view(torch.int16) == b.cpu().view(torch.int16)).float().mean().item()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,hidden,pad", [(512, 4096, 0), (33, 1024, 8), (7, 513, 0), (5, 260, 3), (3, 12288, 0)])
+@pytest.mark.parametrize("activation", ["gelu", "gelu_tanh"])
+def test_add_ln_gelu_against_oracle(ops, dtype, rows, hidden, pad, activation):
+    x, z, w, b = glue_inputs(rows, hidden, dtype, 21, pad)
+    alpha = 2.3716
+    xd, zd = to_device_pitched(x, DEV), to_device_pitched(z, DEV)
+    before = xd.clone()
+    got = torch.ops.arctic_inference.speculator_add_ln_act_cuda(xd, zd, w.to(DEV), b.to(DEV), alpha, 1e-6,
+                                                                activation, 1.0)
+    torch.cuda.synchronize()
+    want = oracle.speculator_add_ln_act(x, z, w, b, alpha, 1e-6, activation, 1.0)
+    assert got.shape == x.shape and got.dtype == dtype and got.is_contiguous()
+    assert torch.equal(xd, before), "the input must stay untouched"
+    assert_close(got, want, RTOL, ATOL, "speculator_add_ln_act")
+    assert same_fraction(got, want) > 0.97
+    if activation == "gelu":
+        got2 = ops.speculator_add_ln_gelu(xd, zd, w.to(DEV), b.to(DEV), alpha, 1e-6)
+        assert torch.equal(got2, got)
+
+
+def test_add_ln_gelu_against_the_three_separate_gpu_ops(ops):
+    """states.add_(z, alpha=...); gelu(speculator_ln(states)) run as the speculator runs them
+    (arctic_inference/vllm/spec_dec/arctic_speculator.py:300-307) on the GPU."""
+    x, z, w, b = glue_inputs(512, 4096, torch.bfloat16, 22)
+    alpha = 2.3716
+    xd, zd, wd, bd = x.to(DEV), z.to(DEV), w.to(DEV), b.to(DEV)
+    fused = ops.speculator_add_ln_gelu(xd, zd, wd, bd, alpha, 1e-6)
+    s = xd.clone()
+    s.add_(zd, alpha=alpha)
+    separate = torch.nn.functional.gelu(ops.speculator_ln(s, wd, bd, 1e-6))
+    assert_close(fused, separate.cpu(), RTOL, ATOL, "fused vs separate")
+    assert same_fraction(fused, separate) > 0.99
+
+
+@pytest.mark.parametrize("affine", [False, True])
+def test_ln_scaled_is_ln_then_scale(ops, affine):
+    # ln0(x) / SQRT2 of the speculator (arctic_speculator.py:296-297): no affine terms there
+    x, _, w, b = glue_inputs(512, 4096, torch.bfloat16, 23)
+    w, b = (w, b) if affine else (None, None)
+    wd, bd = (w.to(DEV), b.to(DEV)) if affine else (None, None)
+    inv = float(torch.tensor(1.0) / torch.tensor(2 ** 0.5))
+    xd = x.to(DEV)
+    got = ops.speculator_ln_scaled(xd, wd, bd, 1e-6, inv)
+    # bit-identical to the product's own norm followed by a multiplication in fp32, rounded once more
+    two_step = (ops.speculator_ln(xd, wd, bd, 1e-6).float() * inv).to(torch.bfloat16)
+    assert torch.equal(got, two_step)
+    assert_close(got, oracle.speculator_add_ln_act(x, None, w, b, 0.0, 1e-6, "none", inv), RTOL, ATOL, "ln_scaled")
+    # and within an ulp of what torch's division gives
+    assert same_fraction(got, ops.speculator_ln(xd, wd, bd, 1e-6) / 2 ** 0.5) > 0.99
+
+
+def test_add_ln_act_degenerate_and_errors(ops):
+    x, z, w, b = glue_inputs(9, 512, torch.bfloat16, 24)
+    xd, zd, wd, bd = x.to(DEV), z.to(DEV), w.to(DEV), b.to(DEV)
+    op = torch.ops.arctic_inference.speculator_add_ln_act_cuda
+    plain = ops.speculator_ln(xd, wd, bd, 1e-6)
+    assert torch.equal(op(xd, None, wd, bd, 0.0, 1e-6, "none", 1.0), plain)
+    assert torch.equal(op(xd, zd, wd, bd, 0.0, 1e-6, "none", 1.0), plain)       # alpha = 0
+    assert torch.equal(op(xd, None, wd, bd, 0.0, 1e-6, "none", 0.5), plain / 2)  # exact scaling
+    assert op(torch.empty(0, 64, dtype=torch.bfloat16, device=DEV), None, None, None, 0.0, 1e-6, "gelu", 1.0).shape == (0, 64)
+    with pytest.raises(RuntimeError, match="activation must be one of"):
+        op(xd, zd, wd, bd, 1.0, 1e-6, "relu", 1.0)
+    with pytest.raises(RuntimeError, match="z must have the input's shape"):
+        op(xd, zd[:4], wd, bd, 1.0, 1e-6, "gelu", 1.0)
+    with pytest.raises(RuntimeError, match="z dtype must match"):
+        op(xd, zd.half(), wd, bd, 1.0, 1e-6, "gelu", 1.0)
+    with pytest.raises(RuntimeError, match="only fp16 and bf16"):
+        op(xd.float(), None, None, None, 1.0, 1e-6, "gelu", 1.0)

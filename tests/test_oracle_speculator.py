@@ -12,7 +12,7 @@ import torch
 import torch.nn.functional as F
 
 import oracle
-from helpers import make_lstm_case, pitched
+from helpers import assert_close, make_lstm_case, pitched
 
 GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
 # largest relative error of ONE round-to-nearest into the format (half a unit in the last place)
@@ -201,3 +201,91 @@ def test_lstm_degenerate_cases():
     # tanh and erf GELU differ
     f_ = oracle.sum_lstm(s4, z4, pc, None, None, None, None, 0.35, 1e-6, 1e-6, True)
     assert not torch.equal(f_[0], d[0])
+
+
+# --------------------------------------------------------------------------- #
+# ao_speculator_add_ln_act: the element-wise steps around the norm
+# (arctic_inference/vllm/spec_dec/arctic_speculator.py:296-307, 733-734, 809-816)
+# --------------------------------------------------------------------------- #
+def glue_case(rows, hidden, dtype, seed, pad=0):
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(rows, hidden + pad, generator=g) * 1.3).to(dtype)[:, :hidden]
+    z = torch.randn(rows, hidden + pad, generator=g).to(dtype)[:, :hidden]
+    w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    return x, z, w, b
+
+
+def same_fraction(a, b):
+    return (a.view(torch.int16) == b.view(torch.int16)).float().mean().item()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hidden,pad", [(4096, 0), (260, 0), (513, 3)])
+def test_glue_equals_the_separate_torch_ops(dtype, hidden, pad):
+    """states.add_(z, alpha); gelu(ln(states)) with torch's GELU around the pinned ao_speculator_ln.
+    The add is written out in fp32 (one rounding into the tensor's type): torch's CPU add_ rounds alpha
+    to the tensor's type and rounds alpha*z once more in its scalar tail, which the GPU kernel the
+    speculator runs on does not.  alpha = 0.75 makes alpha*z exact in fp32, so the sum does not depend
+    on fused or separate multiply-add either."""
+    x, z, w, b = glue_case(24, hidden, dtype, 7, pad)
+    alpha = 0.75
+    s = (x.float() + alpha * z.float()).to(dtype)
+    t = x.clone()
+    t.add_(z, alpha=alpha)
+    assert same_fraction(s, t) > 0.99                 # torch's own in-place add agrees but for its tail elements
+    want = torch.nn.functional.gelu(oracle.speculator_ln(s, w, b, 1e-6))
+    got = oracle.speculator_add_ln_act(x, z, w, b, alpha, 1e-6, "gelu", 1.0)
+    # torch's vectorised erf and libm's differ in the last fp32 bits now and then; fp16 keeps three more of them
+    assert same_fraction(got, want) > (0.999 if dtype == torch.bfloat16 else 0.997)
+    assert_close(got, want, 8e-3 if dtype == torch.bfloat16 else 1.1e-3, 1e-6, "glue vs separate ops (one ulp)")
+    # the tanh form against torch's
+    want_t = torch.nn.functional.gelu(oracle.speculator_ln(s, w, b, 1e-6).float(), approximate="tanh").to(dtype)
+    got_t = oracle.speculator_add_ln_act(x, z, w, b, alpha, 1e-6, "gelu_tanh", 1.0)
+    assert same_fraction(got_t, want_t) > (0.999 if dtype == torch.bfloat16 else 0.997)
+
+
+def test_glue_float64_closed_form_with_general_alpha():
+    x, z, w, b = glue_case(16, 1024, torch.bfloat16, 8)
+    alpha = 2.3716
+    a32 = float(torch.tensor(alpha, dtype=torch.float32))
+    s = (x.double() + a32 * z.double()).to(torch.bfloat16)          # rounding after the in-place add
+    y = rms_norm_ref(s.double(), 1e-6, w.double(), b.double()).to(torch.bfloat16)
+    want = torch.nn.functional.gelu(y.double()).to(torch.bfloat16)
+    got = oracle.speculator_add_ln_act(x, z, w, b, alpha, 1e-6, "gelu", 1.0)
+    assert same_fraction(got, want) > 0.995
+    # an add that lands on the other side of a rounding boundary moves the end result by a few ulps
+    assert_close(got, want, 1e-2, 2e-2, "glue vs float64")
+
+
+def test_glue_degenerate_cases():
+    x, z, w, b = glue_case(9, 512, torch.bfloat16, 9)
+    plain = oracle.speculator_ln(x, w, b, 1e-6)
+    # nothing switched on: the norm itself, bit for bit
+    assert torch.equal(oracle.speculator_add_ln_act(x, None, w, b, 0.0, 1e-6, "none", 1.0), plain)
+    # alpha = 0: z must not matter
+    assert torch.equal(oracle.speculator_add_ln_act(x, z, w, b, 0.0, 1e-6, "none", 1.0), plain)
+    # scaling by a power of two is exact: ln(x) * 0.5 == ln(x) / 2
+    assert torch.equal(oracle.speculator_add_ln_act(x, None, w, b, 0.0, 1e-6, "none", 0.5), plain / 2)
+    # ln0(x) / SQRT2 (no affine) against torch's division, which the GPU turns into a multiplication
+    inv = float(torch.tensor(1.0, dtype=torch.float32) / torch.tensor(2 ** 0.5, dtype=torch.float32))
+    got = oracle.speculator_add_ln_act(x, None, None, None, 0.0, 1e-6, "none", inv)
+    want = oracle.speculator_ln(x, None, None, 1e-6) / 2 ** 0.5
+    assert same_fraction(got, want) > 0.995
+    assert_close(got, want, 8e-3, 1e-6, "ln0 / sqrt2")
+    # the order is norm -> activation -> scale: the other orders give something else
+    a = oracle.speculator_add_ln_act(x, z, w, b, 1.5, 1e-6, "gelu", 0.5)
+    ln = oracle.speculator_ln((x.float() + 1.5 * z.float()).to(torch.bfloat16), w, b, 1e-6)
+    assert_close(a, torch.nn.functional.gelu(ln) * 0.5, 8e-3, 1e-6, "order")
+    wrong = torch.nn.functional.gelu(ln * 0.5)
+    assert (a.float() - wrong.float()).abs().max() > 0.05
+    # the sign of alpha matters
+    assert not torch.equal(oracle.speculator_add_ln_act(x, z, w, b, -1.5, 1e-6, "gelu", 0.5), a)
+
+
+def test_glue_rejects_unknown_modes():
+    x = torch.zeros(2, 8)
+    with pytest.raises(RuntimeError):
+        oracle.speculator_add_ln_act(x, None, None, None, 0.0, 1e-6, "none", 1.0)   # fp32
+    with pytest.raises(KeyError):
+        oracle.speculator_add_ln_act(x.bfloat16(), None, None, None, 0.0, 1e-6, "relu", 1.0)

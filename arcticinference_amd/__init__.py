@@ -8,7 +8,9 @@ __version__ = "0.1.0"
 
 from . import py_custom_ops  # noqa: F401
 from .py_custom_ops import (  # noqa: F401
+    gather_rows,
     reshape_and_cache_flash_bulk,
+    scatter_rows,
     speculator_add_ln_gelu,
     speculator_ln,
     speculator_ln_scaled,

@@ -30,6 +30,7 @@ EXPORTED_SYMBOLS = (
     "arctic_speculator_add_ln_act",
     "arctic_sum_lstm",
     "arctic_sum_lstm_shared_z",
+    "arctic_gather_rows",
 )
 
 _lib: Optional[ctypes.CDLL] = None
@@ -87,6 +88,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.arctic_sum_lstm.restype = i32
     lib.arctic_sum_lstm_shared_z.argtypes = lib.arctic_sum_lstm.argtypes
     lib.arctic_sum_lstm_shared_z.restype = i32
+    lib.arctic_gather_rows.argtypes = [i32, vp, vp, vp, vp, vp, vp, i32, i64, i64, i32, vp]
+    lib.arctic_gather_rows.restype = i32
 
 
 def load() -> ctypes.CDLL:

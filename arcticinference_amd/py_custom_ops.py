@@ -43,6 +43,8 @@ _SCHEMAS = {
         "sum_lstm_cuda(Tensor states_4d, Tensor z4_4d, Tensor prev_cell_d, Tensor? w_cell, "
         "Tensor? b_cell, Tensor? w_state, Tensor? b_state, float alpha, float eps_cell, "
         "float eps_state, bool use_fast_gelu) -> (Tensor, Tensor)",
+    "gather_rows": "gather_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
+    "scatter_rows": "scatter_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
     "speculator_add_ln_act_cuda":
         "speculator_add_ln_act_cuda(Tensor input, Tensor? z, Tensor? weight, Tensor? bias, float alpha, "
         "float eps, str activation, float out_scale) -> Tensor",
@@ -54,6 +56,8 @@ _EXTRA_SCHEMAS = {
         "sum_lstm_shared_z_cuda(Tensor states_4d, Tensor z_d, Tensor prev_cell_d, Tensor? w_cell, "
         "Tensor? b_cell, Tensor? w_state, Tensor? b_state, float alpha, float eps_cell, "
         "float eps_state, bool use_fast_gelu) -> (Tensor, Tensor)",
+    "gather_rows": "gather_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
+    "scatter_rows": "scatter_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
     "speculator_add_ln_act_cuda":
         "speculator_add_ln_act_cuda(Tensor input, Tensor? z, Tensor? weight, Tensor? bias, float alpha, "
         "float eps, str activation, float out_scale) -> Tensor",
@@ -404,7 +408,59 @@ def _sum_lstm_shared_z_impl(states_4d, z_d, prev_cell_d, w_cell, b_cell, w_state
                           eps_state, use_fast_gelu, _shared_z=True)
 
 
+def _move_rows_impl(fn: str, sources: List[torch.Tensor], indices: torch.Tensor, outs: List[torch.Tensor],
+                    scatter: bool) -> None:
+    lib = _lib()
+    _check(len(sources) == len(outs), f"{fn}: {len(sources)} sources but {len(outs)} outputs")
+    _check(indices.is_cuda and indices.dim() == 1 and indices.is_contiguous(),
+           f"{fn}: indices must be a contiguous 1-D CUDA tensor")
+    _check(indices.dtype in (torch.int32, torch.int64), f"{fn}: indices must be int32 or int64")
+    n = indices.numel()
+    if n == 0 or not sources:
+        return
+    indexed_rows = None
+    row_bytes, src_stride, dst_stride = [], [], []
+    for k, (src, dst) in enumerate(zip(sources, outs)):
+        _check(src.is_cuda and dst.is_cuda and src.device == indices.device and dst.device == indices.device,
+               f"{fn}: tensor {k}: sources, outputs and indices must be on one CUDA device")
+        _check(src.dtype == dst.dtype, f"{fn}: tensor {k}: source and output dtypes differ")
+        _check(src.dim() >= 1 and src.shape[1:] == dst.shape[1:], f"{fn}: tensor {k}: row shapes differ")
+        _check(src.size(0) == 0 or src[0].is_contiguous(), f"{fn}: tensor {k}: source rows must be contiguous")
+        _check(dst.size(0) == 0 or dst[0].is_contiguous(), f"{fn}: tensor {k}: output rows must be contiguous")
+        indexed, linear = (dst, src) if scatter else (src, dst)
+        _check(linear.size(0) >= n, f"{fn}: tensor {k}: {n} indices but only {linear.size(0)} rows")
+        _check(indexed_rows in (None, indexed.size(0)), f"{fn}: indexed tensors differ in their number of rows")
+        indexed_rows = indexed.size(0)
+        es = src.element_size()
+        row = 1
+        for d in src.shape[1:]:
+            row *= d
+        row_bytes.append(row * es)
+        src_stride.append(src.stride(0) * es)
+        dst_stride.append(dst.stride(0) * es)
+    i64s = lambda v: (ctypes.c_int64 * len(v))(*v)
+    with _on_device_of(indices):
+        rc = lib.arctic_gather_rows(len(sources), _ptr_table(sources), _ptr_table(outs), i64s(row_bytes),
+                                    i64s(src_stride), i64s(dst_stride), indices.data_ptr(), indices.element_size(),
+                                    n, indexed_rows, 1 if scatter else 0, _stream_of(indices))
+    _native.check(rc)
+
+
+def _gather_rows_impl(sources: List[torch.Tensor], indices: torch.Tensor, outs: List[torch.Tensor]) -> None:
+    """outs[k][r] = sources[k][indices[r]]: the index_select calls of swiftkv_select
+    (arctic_inference/vllm/swiftkv/llama_swiftkv.py:663-679) in one launch."""
+    _move_rows_impl("gather_rows", sources, indices, outs, False)
+
+
+def _scatter_rows_impl(sources: List[torch.Tensor], indices: torch.Tensor, outs: List[torch.Tensor]) -> None:
+    """outs[k][indices[r]] = sources[k][r]: `orig_hidden_states[logits_indices] = hidden_states[:batch_size]`
+    (arctic_inference/vllm/swiftkv/llama_swiftkv.py:733-742)."""
+    _move_rows_impl("scatter_rows", sources, indices, outs, True)
+
+
 _IMPLS = {
+    "gather_rows": _gather_rows_impl,
+    "scatter_rows": _scatter_rows_impl,
     "sum_lstm_shared_z_cuda": _sum_lstm_shared_z_impl,
     "speculator_add_ln_act_cuda": _speculator_add_ln_act_impl,
     "reshape_and_cache_flash_bulk": _reshape_and_cache_flash_bulk_impl,
@@ -574,3 +630,25 @@ def speculator_ln_scaled(
     ``ln0(previous_hidden_states) / SQRT2`` with ``out_scale = 1 / SQRT2``
     (arctic_inference/vllm/spec_dec/arctic_speculator.py:296-297, 733-734)."""
     return _ops().speculator_add_ln_act_cuda(input, None, weight, bias, 0.0, eps, "none", out_scale)
+
+
+def gather_rows(sources: List[torch.Tensor], indices: torch.Tensor,
+                outs: Optional[List[Optional[torch.Tensor]]] = None) -> List[torch.Tensor]:
+    """``torch.index_select(sources[k], 0, indices, out=outs[k][:indices.numel()])`` for every k in one
+    launch: the five ``index_fn`` calls of ``swiftkv_select``
+    (arctic_inference/vllm/swiftkv/llama_swiftkv.py:663-679).  A missing output is allocated, like
+    ``tensor.index_select(0, indices)``.  Returns the outputs (whole buffers, as passed)."""
+    n = indices.numel()
+    outs = list(outs) if outs is not None else [None] * len(sources)
+    for k, src in enumerate(sources):
+        if outs[k] is None:
+            outs[k] = torch.empty((n,) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
+    _ops().gather_rows(list(sources), indices, outs)
+    return outs
+
+
+def scatter_rows(sources: List[torch.Tensor], indices: torch.Tensor, outs: List[torch.Tensor]) -> None:
+    """``outs[k][indices] = sources[k][:indices.numel()]`` for every k in one launch: the write-back
+    ``orig_hidden_states[logits_indices] = hidden_states[:batch_size]``
+    (arctic_inference/vllm/swiftkv/llama_swiftkv.py:733-742)."""
+    _ops().scatter_rows(list(sources), indices, list(outs))

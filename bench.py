@@ -292,6 +292,42 @@ def bench_fp4(ops, dev, steps):
             "hbm_frac": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
 
 
+def bench_row_gather(ops, dev, steps):
+    """swiftkv_select of a decode-only batch at the 70B shape (llama_swiftkv.py:663-679): 512 rows of
+    hidden_states and residual (8192 bf16), positions (int64), k_states and v_states (40 layers x 1024 bf16)
+    gathered by logits_indices into the decode buffers; one launch against torch's five index_select calls.
+    Four rotating sets (800 MB) keep the rows out of the last-level cache."""
+    T, hidden, kvw, sets = 512, 8192, 40 * 1024, 4
+    g = torch.Generator(device=dev).manual_seed(6)
+    rn = lambda *s: torch.randn(*s, generator=g, device=dev).to(torch.bfloat16)
+    src = [[rn(T, hidden), rn(T, hidden), torch.arange(T, device=dev), rn(T, kvw), rn(T, kvw)] for _ in range(sets)]
+    dst = [[torch.empty_like(t) for t in s] for s in src]
+    idx = torch.arange(T, device=dev)
+    nbytes = 2 * sum(t.numel() * t.element_size() for t in src[0])
+
+    def fused(i):
+        ops.gather_rows(src[i % sets], idx, dst[i % sets])
+
+    def separate(i):
+        for t, o in zip(src[i % sets], dst[i % sets]):
+            torch.index_select(t, 0, idx, out=o)
+
+    out = {"bytes_per_call": nbytes}
+    for name, fn in (("gather_rows", fused), ("five_index_select", separate)):
+        for i in range(3):
+            fn(i)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(sets):
+                fn(i)
+        graph.replay()
+        torch.cuda.synchronize()
+        med = statistics.median(event_times_us(graph.replay, max(10, steps // 2))) / sets
+        out[name] = {"us_per_call_graph": round(med, 2), "GBps": round(nbytes / med / 1e3, 1),
+                     "hbm_frac": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
+    return out
+
+
 def box_reference(dev):
     """What plain library kernels reach on this very GPU (boxes of one pool differ by up to 20 %):
     a contiguous bf16 -> fp8 cast of 1.3 GB (the same 2:1 read:write mix as the bulk fp8 write, no
@@ -536,6 +572,7 @@ def main():
         torch.cuda.empty_cache()
         extras["speculator"] = bench_speculator(ops, dev, args.steps, args.warmup)
         extras["decode_mix"] = bench_decode_mix(ops, dev, args.steps)
+        extras["swiftkv_select_decode_70b"] = bench_row_gather(ops, dev, args.steps)
         log(f"extras: {extras}")
 
     result = {

@@ -217,6 +217,35 @@ int arctic_sum_lstm_shared_z(void *out_state, void *out_cell, const void *states
                              float alpha, float eps_cell, float eps_state, int fast_gelu,
                              int dtype, void *stream);
 
+/*
+ * Row gather / scatter over up to 8 tensors in one launch.  No native function of
+ * the reference corresponds to it; it stands for the PyTorch calls either side of
+ * the bulk KV write in LlamaSwiftKVModel:
+ *   gather   torch.index_select(tensor, 0, logits_indices, out=buffer[:batch]) for
+ *            hidden_states, residual, positions, k_states, v_states
+ *            arctic_inference/vllm/swiftkv/llama_swiftkv.py:663-679
+ *   scatter  orig_hidden_states[logits_indices] = hidden_states[:batch_size]
+ *            arctic_inference/vllm/swiftkv/llama_swiftkv.py:733-742
+ *
+ * gather  (scatter == 0): dst_t row r           <- src_t row indices[r]
+ * scatter (scatter != 0): dst_t row indices[r]  <- src_t row r
+ * for r in [0, num_indices) and every tensor t.  Bytes are copied as they are.  An
+ * index outside [0, num_indexed_rows) moves nothing (torch raises a device-side
+ * assertion there).  Equal indices in a scatter race, as in torch.
+ *
+ *   src, dst            HOST arrays [num_tensors] of device pointers (row 0 of each tensor)
+ *   row_bytes           HOST array: bytes per row of each tensor (0 skips the tensor)
+ *   *_row_stride_bytes  HOST arrays: bytes between rows
+ *   indices             device, num_indices entries of index_bytes (4 or 8) each, signed
+ *   num_indices         at most 65535
+ *   num_indexed_rows    rows of the indexed side (sources of a gather, destinations of a scatter)
+ */
+int arctic_gather_rows(int num_tensors, const void *const *src, void *const *dst,
+                       const int64_t *row_bytes, const int64_t *src_row_stride_bytes,
+                       const int64_t *dst_row_stride_bytes, const void *indices,
+                       int index_bytes, int64_t num_indices, int64_t num_indexed_rows,
+                       int scatter, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -284,3 +284,33 @@ def sum_lstm(states_4d: torch.Tensor, z4_4d: torch.Tensor, prev_cell_d: torch.Te
     if rc != 0:
         raise RuntimeError("oracle: sum_lstm supports fp16/bf16 only")
     return out_state.view(prev_cell_d.shape), out_cell.view(prev_cell_d.shape)
+
+
+def gather_rows(sources, indices: torch.Tensor, outs=None):
+    """The reference's own expression on the CPU: ``torch.index_select(t, 0, indices, out=buf[:n])`` per
+    tensor (arctic_inference/vllm/swiftkv/llama_swiftkv.py:663-679).  Rows whose index is out of range
+    are left as they are (torch raises there; the kernel skips)."""
+    n = indices.numel()
+    idx = indices.to(torch.int64)
+    result = []
+    for k, src in enumerate(sources):
+        _cpu(src, "source")
+        out = outs[k] if outs is not None and outs[k] is not None else torch.zeros(
+            (n,) + tuple(src.shape[1:]), dtype=src.dtype)
+        ok = (idx >= 0) & (idx < src.size(0))
+        rows = torch.nonzero(ok).flatten()
+        out[rows] = src.index_select(0, idx[rows])
+        result.append(out)
+    return result
+
+
+def scatter_rows(sources, indices: torch.Tensor, outs) -> None:
+    """``out[indices] = src[:n]`` per tensor (arctic_inference/vllm/swiftkv/llama_swiftkv.py:733-742);
+    out-of-range indices are skipped."""
+    n = indices.numel()
+    idx = indices.to(torch.int64)
+    for src, out in zip(sources, outs):
+        _cpu(src, "source")
+        ok = (idx >= 0) & (idx < out.size(0))
+        rows = torch.nonzero(ok).flatten()
+        out[idx[rows]] = src[:n][rows]

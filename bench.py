@@ -509,7 +509,18 @@ def main():
         del wc, fc
         torch.cuda.empty_cache()
 
-    mem = ServingMemoryMap(dev, args.weight_gib, 80, 40, args.pool_blocks, 16, 8, 128, torch.uint8)
+    # the map needs 66 + 160 GiB of the 268; should less be free, halve the pool rather than fail
+    mem, pool_blocks = None, args.pool_blocks
+    while mem is None:
+        try:
+            mem = ServingMemoryMap(dev, args.weight_gib, 80, 40, pool_blocks, 16, 8, 128, torch.uint8)
+        except torch.OutOfMemoryError:
+            torch.cuda.empty_cache()
+            if pool_blocks <= 2048:
+                raise
+            pool_blocks //= 2
+            log(f"not enough free device memory for the pool; retrying with {pool_blocks} blocks per layer")
+    args.pool_blocks = pool_blocks
     log(f"memory map: {mem.describe()}")
     w = BulkWorkload("70B-SwiftKV", 16384, 40, 8, 128, 16, args.pool_blocks, "fp8", 0.10, 2, 1.5, dev,
                      bufs=mem.written_layers())

@@ -515,11 +515,12 @@ def main():
         try:
             mem = ServingMemoryMap(dev, args.weight_gib, 80, 40, pool_blocks, 16, 8, 128, torch.uint8)
         except torch.OutOfMemoryError:
-            torch.cuda.empty_cache()
             if pool_blocks <= 2048:
                 raise
             pool_blocks //= 2
             log(f"not enough free device memory for the pool; retrying with {pool_blocks} blocks per layer")
+        if mem is None:
+            torch.cuda.empty_cache()   # after the handler, when the half-built map is no longer referenced
     args.pool_blocks = pool_blocks
     log(f"memory map: {mem.describe()}")
     w = BulkWorkload("70B-SwiftKV", 16384, 40, 8, 128, 16, args.pool_blocks, "fp8", 0.10, 2, 1.5, dev,

@@ -189,6 +189,20 @@ def cpu_baseline_bulk(w: BulkWorkload, target_seconds=6.0):
     }
 
 
+def load_floor_kernels():
+    """bench_floor.so: bare kernels that move the same bytes as the library's and compute nothing
+    (built by __graft_entry__.build()).  None when it has not been built."""
+    import ctypes
+    path = os.path.join(ROOT, "bench_floor.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    lib.floor_lstm_traffic.argtypes = [vp, vp, vp, vp, vp, i64, i32, vp]
+    lib.floor_stream.argtypes = [vp, i32, vp, i32, i64, i32, vp, vp]
+    return lib
+
+
 def bench_speculator(ops, dev, steps, warmup):
     """Speculator workload: sum_lstm (3 chained steps) and the standalone LayerNorm at
     T=512, H=4096, bf16.  Eight buffer sets (> 256 MB in total) are rotated so that
@@ -230,12 +244,25 @@ def bench_speculator(ops, dev, steps, warmup):
         s.add_(C0[i % sets], alpha=1e-3)
         torch.nn.functional.gelu(ops.speculator_ln(s, w_cell, b_cell, 1e-6))
 
+    floor = load_floor_kernels()
+    OS = [torch.empty(T, Hd, dtype=torch.bfloat16, device=dev) for _ in range(2)]
+
+    def lstm3_traffic_only(i):
+        # the loads and stores of the three sum_lstm calls with no arithmetic between them
+        stream = torch.cuda.current_stream().cuda_stream
+        for k in range(3):
+            floor.floor_lstm_traffic(S[i % sets][k].data_ptr(), Z[i % sets][k].data_ptr(), C0[i % sets].data_ptr(),
+                                     OS[0].data_ptr(), OS[1].data_ptr(), T, Hd, stream)
+
+    cases = [("sum_lstm", lstm3, 22 * Hd * T, 3),
+             ("sum_lstm_shared_z", lstm3_shared_z, 16 * Hd * T, 3),
+             ("speculator_ln", ln, 4 * Hd * T, 1),
+             ("speculator_add_ln_gelu", add_ln_gelu, 6 * Hd * T, 1),
+             ("add_ln_gelu_as_three_ops", add_ln_gelu_separate, 6 * Hd * T, 1)]
+    if floor is not None:
+        cases.insert(1, ("sum_lstm_traffic_only_floor", lstm3_traffic_only, 22 * Hd * T, 3))
     out = {}
-    for name, fn, per_call, calls in (("sum_lstm", lstm3, 22 * Hd * T, 3),
-                                      ("sum_lstm_shared_z", lstm3_shared_z, 16 * Hd * T, 3),
-                                      ("speculator_ln", ln, 4 * Hd * T, 1),
-                                      ("speculator_add_ln_gelu", add_ln_gelu, 6 * Hd * T, 1),
-                                      ("add_ln_gelu_as_three_ops", add_ln_gelu_separate, 6 * Hd * T, 1)):
+    for name, fn, per_call, calls in cases:
         for i in range(warmup):
             fn(i)
         torch.cuda.synchronize()
@@ -458,6 +485,29 @@ def placement_sweep(ops, dev, steps):
                         [cache(where[l], 2 * l + 1, base) for l in range(L)])
             for name, where in cases.items()}
         out["spread_cases_GBps"] = {name: round(nbytes / us / 1e3) for name, us in out["spread_cases_us"].items()}
+        floor = load_floor_kernels()
+        if floor is not None:
+            # bare streams of 64 KiB pieces dealt over one, two or three regions: 3 GiB loaded, stored, or
+            # loaded with half as much stored (the byte mix of the fp8 write)
+            import ctypes
+            pieces = 3 * 16384
+            sink = torch.zeros(1, dtype=torch.int32, device=dev)
+            ptrs = lambda offs: (ctypes.c_void_p * 3)(*[chunks[c].data_ptr() + offs for c in reps])
+            low, high = ptrs(0), ptrs(4 << 30)
+            stream = torch.cuda.current_stream().cuda_stream
+
+            def stream_GBps(mode, nsrc, ndst, moved):
+                f = lambda: floor.floor_stream(low, nsrc, high, ndst, pieces, mode, sink.data_ptr(), stream)
+                for _ in range(2):
+                    f()
+                return round(moved / statistics.median(event_times_us(f, steps)) / 1e3)
+
+            out["bare_stream_GBps"] = {
+                "load_only": {f"{n}_regions": stream_GBps(0, n, 1, pieces * 65536) for n in (1, 2, 3)},
+                "store_only": {f"{n}_regions": stream_GBps(1, 1, n, pieces * 65536) for n in (1, 2, 3)},
+                "load_2_store_1, loads from one region": {
+                    f"stores_to_{n}_regions": stream_GBps(2, 1, n, pieces * 98304) for n in (1, 2, 3)},
+            }
     return out
 
 

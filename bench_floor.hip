@@ -1,0 +1,75 @@
+// Bare kernels that bench.py times next to the library's kernels: what the same bytes cost on this GPU
+// when nothing is computed.  Measurement aid only; nothing in the package uses it.
+//
+//   floor_lstm_traffic   the loads and stores of sum_lstm (nine 16-byte loads per lane from the rows of
+//                        states, z4 and prev_cell, two 16-byte stores), one workgroup per row, no arithmetic
+//   floor_stream         load-only, store-only or a 2:1 load:store stream in 64 KiB pieces, the pieces dealt
+//                        round robin over up to three buffers (which the caller places in different regions
+//                        of the HBM)
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+__global__ void lstm_traffic_kernel(const char *s, const char *z, const char *pc, char *out_state, char *out_cell,
+                                    int D) {
+  const int chunks = D / 8;
+  const int c = threadIdx.x;
+  if (c >= chunks) return;
+  const size_t row4 = (size_t)blockIdx.x * 4 * D * 2, row1 = (size_t)blockIdx.x * D * 2;
+  u32x4 v[9];
+  for (int g = 0; g < 4; ++g) {
+    v[g] = __builtin_nontemporal_load((const u32x4 *)(s + row4 + (size_t)g * D * 2) + c);
+    v[4 + g] = __builtin_nontemporal_load((const u32x4 *)(z + row4 + (size_t)g * D * 2) + c);
+  }
+  v[8] = __builtin_nontemporal_load((const u32x4 *)(pc + row1) + c);
+  const u32x4 a = v[0] ^ v[1] ^ v[2] ^ v[3] ^ v[8], b = v[4] ^ v[5] ^ v[6] ^ v[7];
+  __builtin_nontemporal_store(a, (u32x4 *)(out_cell + row1) + c);
+  __builtin_nontemporal_store(b, (u32x4 *)(out_state + row1) + c);
+}
+
+struct Three {
+  char *p[3];
+};
+
+// mode 0: load 64 KiB pieces; 1: store 64 KiB pieces; 2: load 64 KiB, store 32 KiB
+__global__ void stream_kernel(Three src, int nsrc, Three dst, int ndst, int64_t pieces, int mode, unsigned *sink) {
+  unsigned acc = 0;
+  for (int64_t k = blockIdx.x; k < pieces; k += gridDim.x) {
+    const u32x4 *from = (const u32x4 *)(src.p[k % nsrc] + (k / nsrc) * 65536);
+    for (int i = threadIdx.x; i < 4096; i += blockDim.x) {
+      u32x4 v = {1u, 2u, 3u, (unsigned)i};
+      if (mode != 1) v = __builtin_nontemporal_load(from + i);
+      if (mode == 0) acc ^= v.x ^ v.y ^ v.z ^ v.w;
+      if (mode == 1) __builtin_nontemporal_store(v, (u32x4 *)(dst.p[k % ndst] + (k / ndst) * 65536) + i);
+      if (mode == 2) {
+        const u32x2 w = {v.x ^ v.z, v.y ^ v.w};
+        __builtin_nontemporal_store(w, (u32x2 *)(dst.p[k % ndst] + (k / ndst) * 32768) + i);
+      }
+    }
+  }
+  if (mode == 0 && acc == 0x12345677u) *sink = acc;
+}
+
+extern "C" int floor_lstm_traffic(const void *s, const void *z, const void *pc, void *out_state, void *out_cell,
+                                  int64_t rows, int D, void *stream) {
+  if (rows <= 0 || D <= 0 || D % 8 != 0 || D / 8 > 1024) return 1;
+  hipLaunchKernelGGL(lstm_traffic_kernel, dim3((unsigned)rows), dim3((unsigned)((D / 8 + 63) & ~63)), 0,
+                     (hipStream_t)stream, (const char *)s, (const char *)z, (const char *)pc, (char *)out_state,
+                     (char *)out_cell, D);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+// Each buffer must hold ceil(pieces / n) * 64 KiB.  `sink` is 4 bytes of device memory.
+extern "C" int floor_stream(void *const *src, int nsrc, void *const *dst, int ndst, int64_t pieces, int mode,
+                            void *sink, void *stream) {
+  if (nsrc < 1 || nsrc > 3 || ndst < 1 || ndst > 3 || pieces <= 0 || mode < 0 || mode > 2 || !sink) return 1;
+  Three a = {}, b = {};
+  for (int i = 0; i < nsrc; ++i) a.p[i] = (char *)src[i];
+  for (int i = 0; i < ndst; ++i) b.p[i] = (char *)dst[i];
+  hipLaunchKernelGGL(stream_kernel, dim3(8192), dim3(256), 0, (hipStream_t)stream, a, nsrc, b, ndst, pieces, mode,
+                     (unsigned *)sink);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}

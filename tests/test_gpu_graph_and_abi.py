@@ -74,6 +74,53 @@ def test_decode_step_in_one_graph(ops):
             assert torch.equal(a, b), f"replay {replay} differs from the eager run"
 
 
+def test_next_row_operators_in_one_graph(ops):
+    """gather_rows, the bulk write, ln0 / sqrt2, add + norm + GELU, sum_lstm with the shared embedding row
+    and scatter_rows captured as one graph; every replay must equal the eager run bit for bit."""
+    T, D, n_sel = 96, 1024, 40
+    g = torch.Generator().manual_seed(77)
+    case = make_bulk_case(T=T, L=4, H=8, D=128, bs=16, NB=16, kv_cache_dtype="fp8", seed=5, std=1.5)
+    dcase = bulk_case_to(case, DEV)
+    rn = lambda *sh: torch.randn(*sh, generator=g).to(torch.bfloat16).to(DEV)
+    hidden, residual = rn(T, D), rn(T, D)
+    positions = torch.randint(0, 4096, (T,), generator=g).to(DEV)
+    idx = torch.sort(torch.randperm(T, generator=g)[:n_sel]).values.to(DEV)
+    bufs = [torch.zeros(64, D, dtype=torch.bfloat16, device=DEV), torch.zeros(64, D, dtype=torch.bfloat16, device=DEV),
+            torch.zeros(64, dtype=torch.int64, device=DEV)]
+    z, w, b = rn(64, D), rn(D), rn(D)
+    s4, pc = rn(64, 4 * D), rn(64, D)
+    orig = rn(T, D)
+    alpha = speculator_alpha(3, D)
+
+    def step():
+        h, r, p = ops.gather_rows([hidden, residual, positions], idx, bufs)
+        ops.reshape_and_cache_flash_bulk(*bulk_args(dcase))
+        x0 = ops.speculator_ln_scaled(h, None, None, 1e-6, 0.70710678)
+        act = ops.speculator_add_ln_gelu(x0, z, w, b, alpha, 1e-6)
+        st, cell = ops.sum_lstm_shared_z(s4, act, pc, w, b, w, b, alpha, 1e-6, 1e-6, False)
+        out = orig.clone()
+        ops.scatter_rows([st], idx, [out])
+        return x0, act, st, cell, out, p
+
+    eager = [t.clone() for t in step()]
+    torch.cuda.synchronize()
+    want = orig.clone()
+    want[idx] = eager[2][:n_sel]
+    assert torch.equal(eager[4], want)
+    assert torch.equal(eager[5][:n_sel], positions[idx])
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for replay in range(3):
+        for t in bufs:
+            t.zero_()                          # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, e in zip(outs, eager):
+            assert torch.equal(a, e), f"replay {replay} differs from the eager run"
+
+
 def test_direct_c_abi_calls(ops):
     """Raw pointers straight into libarctic_mi355x.so (what another host language would do)."""
     lib = _native.load()

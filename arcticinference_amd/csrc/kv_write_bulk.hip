@@ -109,7 +109,8 @@ __device__ __forceinline__ void emit_chunk(const uint4 &v, const RowDesc &d, int
 }
 
 // kBulkThreads x kUnroll 16-byte chunks form one batch of a workgroup.  Two shapes
-// are built: 512 x 2 (long prefill launches) and 256 x 4 (few tokens).
+// are built: 512 x 2 (a workgroup moves two batches or more) and 256 x 4 (decode:
+// few tokens, a single batch per workgroup).
 template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll>
 __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
     const BulkParams p, const LayerTables tab) {

@@ -6,8 +6,12 @@
 //
 //  * Nodes, child buckets and endpoint records live in three arenas and refer to each other by 32-bit
 //    index (the reference uses heap nodes, unique_ptr children maps and shared_ptr groups).
-//  * One open-addressing table per tree maps (parent, first token) -> child, another (node, sequence)
-//    -> endpoint record; the reference keeps a hash map inside every node.
+//  * One open-addressing table per tree maps (parent, first token) -> child; the reference keeps a hash
+//    map inside every node.  The endpoints of a node (which suffixes end there) are a short linked list
+//    of records; a suffix that is still growing carries its record along, so the hot path never searches
+//    for it, and only a node that collects many endpoints gets them indexed in a second table.
+//  * Sequences sit in numbered slots; nodes and endpoint records name a slot, not a sequence id, so
+//    reading a node's tokens takes no hash lookup.
 //  * The children of a node are kept in decreasing order of count as a list of buckets, one per
 //    distinct count, each holding its nodes in order (the O(1) frequency-list layout).  The reference
 //    keeps one sibling list plus "group" records that point at the first node of each run of equal
@@ -122,7 +126,7 @@ struct Node {
   int64_t count = 0;          // suffixes that end at or pass through this node
   int32_t token = 0;          // first token of the node's label
   int32_t length = 0;         // tokens in the label
-  int32_t ref_seq = 0;        // the label is tokens [ref_idx, ref_idx + length) of sequence ref_seq
+  int32_t ref_seq = 0;        // the label is tokens [ref_idx, ref_idx + length) of the sequence in slot ref_seq
   int32_t ref_idx = -1;
   uint32_t parent = NIL;
   uint32_t first_bucket = NIL;  // children, highest count first
@@ -133,17 +137,21 @@ struct Node {
   uint32_t first_endpoint = NIL;
   uint32_t num_children = 0;
   uint32_t num_endpoints = 0;
+  bool endpoints_indexed = false;  // true once the node held more than kIndexAbove endpoints
 };
+
+constexpr uint32_t kIndexAbove = 16;
 
 // The children of one node that share one count, in order.
 struct Bucket {
+  int64_t count = 0;
   uint32_t head = NIL;
   uint32_t tail = NIL;
   uint32_t next = NIL;  // bucket with the next lower count
   uint32_t prev = NIL;
 };
 
-// "A suffix of sequence seq ends in this node, at position end of the sequence."
+// "A suffix of the sequence in slot seq ends in this node, at position end of the sequence."
 struct Endpoint {
   uint32_t node = NIL;
   int32_t seq = 0;
@@ -152,9 +160,16 @@ struct Endpoint {
   uint32_t prev = NIL;
 };
 
+// Where one of the last max_depth suffixes of a sequence currently ends, and its endpoint record.
+struct Growing {
+  uint32_t node;
+  uint32_t endpoint;
+};
+
 struct Sequence {
+  int32_t id = 0;
   std::vector<int32_t> tokens;
-  std::deque<uint32_t> active;  // nodes where the last max_depth suffixes currently end, oldest first
+  std::deque<Growing> active;  // oldest (deepest) first
 };
 
 struct Draft {
@@ -195,8 +210,13 @@ inline uint64_t pair_key(uint32_t a, int32_t b) { return ((uint64_t)a << 32) | (
 
 struct arctic_suffix_tree {
   explicit arctic_suffix_tree(int max_depth) : max_depth_(max_depth) { root_ = nodes_.make(); }
+  ~arctic_suffix_tree() {
+    for (Sequence *s : slots_) delete s;
+  }
+  arctic_suffix_tree(const arctic_suffix_tree &) = delete;
+  arctic_suffix_tree &operator=(const arctic_suffix_tree &) = delete;
 
-  int num_seqs() const { return (int)seqs_.size(); }
+  int num_seqs() const { return (int)slot_of_.size(); }
   void append(int seq_id, int32_t token);
   void remove(int seq_id);
   Draft speculate(const int32_t *context, int64_t n, int max_spec_tokens, float max_spec_factor,
@@ -205,52 +225,120 @@ struct arctic_suffix_tree {
   size_t estimate_memory() const;
 
  private:
+  // ---- sequences ---------------------------------------------------------------------------------
+  int32_t slot_for(int seq_id) {
+    auto it = slot_of_.find(seq_id);
+    if (it != slot_of_.end()) return it->second;
+    int32_t slot;
+    if (!free_slots_.empty()) {
+      slot = free_slots_.back();
+      free_slots_.pop_back();
+    } else {
+      slot = (int32_t)slots_.size();
+      slots_.push_back(nullptr);
+    }
+    slots_[slot] = new Sequence();
+    slots_[slot]->id = seq_id;
+    slot_of_.emplace(seq_id, slot);
+    return slot;
+  }
+  const int32_t *label(uint32_t node) const {
+    const Node &n = nodes_[node];
+    return slots_[n.ref_seq]->tokens.data() + n.ref_idx;
+  }
+
   // ---- children table --------------------------------------------------------------------------
   uint32_t child_of(uint32_t parent, int32_t token) const { return children_.find(pair_key(parent, token)); }
+  // the same answer without touching the table where the node itself tells it
+  uint32_t find_child(uint32_t parent, int32_t token) const {
+    const Node &p = nodes_[parent];
+    if (p.num_children == 0) return NIL;
+    if (p.num_children == 1) {
+      const uint32_t only = buckets_[p.first_bucket].head;
+      return nodes_[only].token == token ? only : NIL;
+    }
+    return child_of(parent, token);
+  }
   void set_child(uint32_t parent, int32_t token, uint32_t child) { children_.set(pair_key(parent, token), child); }
   void drop_child_key(uint32_t parent, int32_t token) { children_.erase(pair_key(parent, token)); }
 
   // ---- endpoints -------------------------------------------------------------------------------
-  uint32_t endpoint_of(uint32_t node, int32_t seq) const { return endpoint_index_.find(pair_key(node, seq)); }
-  void set_endpoint(uint32_t node, int32_t seq, int32_t end) {
-    uint32_t e = endpoint_of(node, seq);
-    if (e == NIL) {
-      e = endpoints_.make();
-      Endpoint &r = endpoints_[e];
-      r.node = node;
-      r.seq = seq;
-      r.next = nodes_[node].first_endpoint;
-      if (r.next != NIL) endpoints_[r.next].prev = e;
-      nodes_[node].first_endpoint = e;
-      nodes_[node].num_endpoints++;
-      endpoint_index_.set(pair_key(node, seq), e);
-    }
-    endpoints_[e].end = end;
+  uint32_t find_endpoint(uint32_t node, int32_t slot) const {
+    const Node &n = nodes_[node];
+    if (n.endpoints_indexed) return endpoint_index_.find(pair_key(node, slot));
+    for (uint32_t e = n.first_endpoint; e != NIL; e = endpoints_[e].next)
+      if (endpoints_[e].seq == slot) return e;
+    return NIL;
   }
-  bool drop_endpoint(uint32_t node, int32_t seq) {
-    const uint32_t e = endpoint_of(node, seq);
-    if (e == NIL) return false;
-    const Endpoint r = endpoints_[e];
-    if (r.prev != NIL) endpoints_[r.prev].next = r.next; else nodes_[node].first_endpoint = r.next;
+  void link_endpoint(uint32_t e, uint32_t node) {
+    Endpoint &r = endpoints_[e];
+    Node &n = nodes_[node];
+    r.node = node;
+    r.prev = NIL;
+    r.next = n.first_endpoint;
+    if (r.next != NIL) endpoints_[r.next].prev = e;
+    n.first_endpoint = e;
+    n.num_endpoints++;
+    if (n.endpoints_indexed) {
+      endpoint_index_.set(pair_key(node, r.seq), e);
+    } else if (n.num_endpoints > kIndexAbove) {
+      n.endpoints_indexed = true;
+      for (uint32_t x = n.first_endpoint; x != NIL; x = endpoints_[x].next)
+        endpoint_index_.set(pair_key(node, endpoints_[x].seq), x);
+    }
+  }
+  void unlink_endpoint(uint32_t e) {
+    const Endpoint &r = endpoints_[e];
+    Node &n = nodes_[r.node];
+    if (r.prev != NIL) endpoints_[r.prev].next = r.next; else n.first_endpoint = r.next;
     if (r.next != NIL) endpoints_[r.next].prev = r.prev;
-    nodes_[node].num_endpoints--;
-    endpoint_index_.erase(pair_key(node, seq));
+    n.num_endpoints--;
+    if (n.endpoints_indexed) endpoint_index_.erase(pair_key(r.node, r.seq));
+  }
+  // a record for a suffix that (the caller knows) has none in `node` yet
+  uint32_t add_endpoint(uint32_t node, int32_t slot, int32_t end) {
+    const uint32_t e = endpoints_.make();
+    endpoints_[e].seq = slot;
+    endpoints_[e].end = end;
+    link_endpoint(e, node);
+    return e;
+  }
+  void drop_endpoint(uint32_t e) {
+    unlink_endpoint(e);
     endpoints_.release(e);
-    return true;
+  }
+  // The growing suffix `g` now ends in `node` at `end`.  A node holds one record per sequence: if an
+  // earlier suffix of the same sequence already ended there (possible only at the depth limit, where
+  // suffixes stop growing), that record is taken over, as assigning endpoints[seq] does in the reference.
+  void move_endpoint(Growing &g, uint32_t node, int32_t end, bool may_exist) {
+    if (may_exist) {
+      const uint32_t there = find_endpoint(node, endpoints_[g.endpoint].seq);
+      if (there != NIL) {
+        drop_endpoint(g.endpoint);
+        g.endpoint = there;
+        endpoints_[there].end = end;
+        g.node = node;
+        return;
+      }
+    }
+    unlink_endpoint(g.endpoint);
+    endpoints_[g.endpoint].end = end;
+    link_endpoint(g.endpoint, node);
+    g.node = node;
   }
   void drop_all_endpoints(uint32_t node) {
-    for (uint32_t e = nodes_[node].first_endpoint; e != NIL;) {
+    Node &n = nodes_[node];
+    for (uint32_t e = n.first_endpoint; e != NIL;) {
       const uint32_t next = endpoints_[e].next;
-      endpoint_index_.erase(pair_key(node, endpoints_[e].seq));
+      if (n.endpoints_indexed) endpoint_index_.erase(pair_key(node, endpoints_[e].seq));
       endpoints_.release(e);
       e = next;
     }
-    nodes_[node].first_endpoint = NIL;
-    nodes_[node].num_endpoints = 0;
+    n.first_endpoint = NIL;
+    n.num_endpoints = 0;
   }
 
   // ---- ordered children ------------------------------------------------------------------------
-  int64_t bucket_count(uint32_t b) const { return nodes_[buckets_[b].head].count; }
   uint32_t head_child(uint32_t node) const {
     const uint32_t b = nodes_[node].first_bucket;
     return b == NIL ? NIL : buckets_[b].head;
@@ -265,6 +353,7 @@ struct arctic_suffix_tree {
   void bucket_alone(uint32_t parent, uint32_t node, uint32_t before, uint32_t after) {
     const uint32_t b = buckets_.make();
     Bucket &k = buckets_[b];
+    k.count = nodes_[node].count;
     k.head = k.tail = node;
     k.prev = before;
     k.next = after;
@@ -319,7 +408,7 @@ struct arctic_suffix_tree {
   }
   void add_last_child(uint32_t parent, uint32_t node) {  // node.count == 1
     const uint32_t last = nodes_[parent].last_bucket;
-    if (last != NIL && bucket_count(last) == 1) bucket_push_back(last, node);
+    if (last != NIL && buckets_[last].count == 1) bucket_push_back(last, node);
     else bucket_alone(parent, node, last, NIL);
     nodes_[parent].num_children++;
   }
@@ -327,10 +416,6 @@ struct arctic_suffix_tree {
   void count_down(uint32_t node);
 
   void release_subtree(uint32_t top);
-  const int32_t *label(uint32_t node) const {
-    const Node &n = nodes_[node];
-    return seqs_.find(n.ref_seq)->second.tokens.data() + n.ref_idx;
-  }
   bool match(const int32_t *context, int64_t n, uint32_t &node, int &idx) const;
   Draft draft_path(uint32_t node, int idx, int max_tokens, float min_token_prob) const;
   Draft draft_tree(uint32_t node, int idx, int max_tokens, float min_token_prob) const;
@@ -341,30 +426,33 @@ struct arctic_suffix_tree {
   Arena<Bucket> buckets_;
   Arena<Endpoint> endpoints_;
   FlatMap children_;
-  FlatMap endpoint_index_;
-  std::unordered_map<int32_t, Sequence> seqs_;
+  FlatMap endpoint_index_;                        // (node, slot) -> record, for nodes with many endpoints
+  std::vector<Sequence *> slots_;                 // sequences by slot; nullptr = free
+  std::vector<int32_t> free_slots_;
+  std::unordered_map<int32_t, int32_t> slot_of_;  // sequence id -> slot
 };
 
 // count c -> c+1 (suffix_tree.cc:171-215)
 void arctic_suffix_tree::count_up(uint32_t node) {
   Node &n = nodes_[node];
   const uint32_t b = n.bucket;
-  const uint32_t above = buckets_[b].prev;
-  const bool first = buckets_[b].head == node;
-  const bool alone = first && buckets_[b].tail == node;
-  const bool joins = above != NIL && bucket_count(above) == n.count + 1;
+  Bucket &k = buckets_[b];
+  const uint32_t above = k.prev;
+  const bool first = k.head == node;
+  const bool alone = first && k.tail == node;
+  const bool joins = above != NIL && buckets_[above].count == n.count + 1;
   if (alone && !joins) {  // nothing to reorder
     n.count += 1;
+    k.count += 1;
     return;
   }
   const uint32_t parent = n.parent;
-  // where a bucket of its own would go: right above b (b survives: it holds other nodes unless `joins`)
   unlink(node);
   nodes_[node].count += 1;
   if (joins) {
     if (first) bucket_push_front(above, node); else bucket_push_back(above, node);
   } else {
-    bucket_alone(parent, node, above, b);
+    bucket_alone(parent, node, above, b);  // b survives: it holds other nodes
   }
 }
 
@@ -372,11 +460,13 @@ void arctic_suffix_tree::count_up(uint32_t node) {
 void arctic_suffix_tree::count_down(uint32_t node) {
   Node &n = nodes_[node];
   const uint32_t b = n.bucket;
-  const uint32_t below = buckets_[b].next;
-  const bool alone = buckets_[b].head == node && buckets_[b].tail == node;
-  const bool joins = below != NIL && bucket_count(below) == n.count - 1;
+  Bucket &k = buckets_[b];
+  const uint32_t below = k.next;
+  const bool alone = k.head == node && k.tail == node;
+  const bool joins = below != NIL && buckets_[below].count == n.count - 1;
   if (alone && !joins) {
     n.count -= 1;
+    k.count -= 1;
     return;
   }
   const uint32_t parent = n.parent;
@@ -408,38 +498,43 @@ void arctic_suffix_tree::release_subtree(uint32_t top) {
 
 // suffix_tree.cc:297-490
 void arctic_suffix_tree::append(int seq_id, int32_t token) {
-  Sequence &seq = seqs_[seq_id];
+  const int32_t slot = slot_for(seq_id);
+  Sequence &seq = *slots_[slot];
   // a new suffix starts at the root
-  seq.active.push_back(root_);
-  set_endpoint(root_, seq_id, (int32_t)seq.tokens.size());
+  seq.active.push_back(Growing{root_, add_endpoint(root_, slot, (int32_t)seq.tokens.size())});
   nodes_[root_].count += 1;
-  if (seq.active.size() > (size_t)max_depth_) seq.active.pop_front();  // it keeps its endpoint: truncated suffix
+  if (seq.active.size() > (size_t)max_depth_) seq.active.pop_front();  // keeps its endpoint: a truncated suffix
   seq.tokens.push_back(token);
   const int32_t len = (int32_t)seq.tokens.size();
+  // only the oldest suffix of a full window reaches the depth limit, where records of the same
+  // sequence can already be waiting
+  const bool window_full = seq.active.size() == (size_t)max_depth_;
 
-  for (uint32_t &slot : seq.active) {
-    const uint32_t node = slot;
-    const uint32_t child = child_of(node, token);
+  bool oldest = true;
+  for (Growing &g : seq.active) {
+    const bool at_limit = oldest && window_full;
+    oldest = false;
+    const uint32_t node = g.node;
+    if (nodes_[node].count == 1 && node != root_) {
+      // only this suffix ends here and nothing passes through: a leaf, which grows by one token
+      nodes_[node].length += 1;
+      endpoints_[g.endpoint].end += 1;
+      continue;
+    }
+    const uint32_t child = find_child(node, token);
     if (child == NIL) {
-      Node &n = nodes_[node];
-      if (n.count == 1 && node != root_) {
-        // only this suffix ends here and nothing passes through: a leaf, which grows by one token
-        n.length += 1;
-        endpoints_[endpoint_of(node, seq_id)].end += 1;
-      } else {
+      {
         const uint32_t fresh = nodes_.make();
         Node &f = nodes_[fresh];
         f.count = 1;
         f.token = token;
         f.length = 1;
-        f.ref_seq = seq_id;
+        f.ref_seq = slot;
         f.ref_idx = len - 1;
         f.parent = node;
-        set_endpoint(fresh, seq_id, len);
         set_child(node, token, fresh);
-        drop_endpoint(node, seq_id);
+        move_endpoint(g, fresh, len, false);
         add_last_child(node, fresh);
-        slot = fresh;
       }
     } else if (nodes_[node].count == nodes_[child].count + 1 && node != root_) {
       // this suffix is the only one that ends here; every other one continues into the single child
@@ -447,30 +542,27 @@ void arctic_suffix_tree::append(int seq_id, int32_t token) {
       Node &c = nodes_[child];
       if (c.length == 1) {
         // with the new token the suffix covers the child entirely: the two nodes become one
-        c.count += 1;
+        c.count += 1;  // now equal to the node's count, whose place it takes
         c.token = n.token;
         c.length = n.length + 1;
-        c.ref_seq = seq_id;
+        c.ref_seq = slot;
         c.ref_idx = len - c.length;
-        set_endpoint(child, seq_id, len);
         c.parent = n.parent;
+        buckets_.release(n.first_bucket);
         take_place(node, child);
         drop_child_key(node, token);
         set_child(c.parent, c.token, child);  // overwrites the entry that led to `node`
-        // `node` is gone: its only bucket held `child`, its only endpoint was this suffix
-        buckets_.release(n.first_bucket);
-        drop_all_endpoints(node);
-        nodes_.release(node);
-        slot = child;
+        move_endpoint(g, child, len, at_limit);
+        nodes_.release(node);                 // its only endpoint was this suffix's, now moved
       } else {
         // the node takes over the child's first token
         n.length += 1;
-        endpoints_[endpoint_of(node, seq_id)].end += 1;
-        n.ref_seq = seq_id;
+        endpoints_[g.endpoint].end += 1;
+        n.ref_seq = slot;
         n.ref_idx = len - n.length;
         c.length -= 1;
         c.ref_idx += 1;
-        const int32_t first = seqs_.find(c.ref_seq)->second.tokens[c.ref_idx];
+        const int32_t first = slots_[c.ref_seq]->tokens[c.ref_idx];
         if (first != token) {
           drop_child_key(node, token);
           set_child(node, first, child);
@@ -480,10 +572,8 @@ void arctic_suffix_tree::append(int seq_id, int32_t token) {
     } else {
       // the suffix moves down into the child
       if (nodes_[child].length == 1) {
-        drop_endpoint(node, seq_id);
-        set_endpoint(child, seq_id, len);
+        move_endpoint(g, child, len, at_limit);
         count_up(child);
-        slot = child;
       } else {
         // the child's first token splits off into a node of its own, which the suffix enters
         const uint32_t mid = nodes_.make();
@@ -492,22 +582,20 @@ void arctic_suffix_tree::append(int seq_id, int32_t token) {
         m.count = c.count;
         m.token = token;
         m.length = 1;
-        m.ref_seq = seq_id;
+        m.ref_seq = slot;
         m.ref_idx = len - 1;
         m.parent = node;
         take_place(child, mid);
         set_child(node, token, mid);
         c.length -= 1;
         c.ref_idx += 1;
-        c.token = seqs_.find(c.ref_seq)->second.tokens[c.ref_idx];
+        c.token = slots_[c.ref_seq]->tokens[c.ref_idx];
         c.parent = mid;
         set_child(mid, c.token, child);
         bucket_alone(mid, child, NIL, NIL);
         m.num_children = 1;
-        drop_endpoint(node, seq_id);
-        set_endpoint(mid, seq_id, len);
+        move_endpoint(g, mid, len, false);
         count_up(mid);
-        slot = mid;
       }
     }
   }
@@ -515,9 +603,10 @@ void arctic_suffix_tree::append(int seq_id, int32_t token) {
 
 // suffix_tree.cc:500-581
 void arctic_suffix_tree::remove(int seq_id) {
-  auto found = seqs_.find(seq_id);
-  if (found == seqs_.end()) return;
-  const std::vector<int32_t> &seq = found->second.tokens;
+  auto found = slot_of_.find(seq_id);
+  if (found == slot_of_.end()) return;
+  const int32_t slot = found->second;
+  const std::vector<int32_t> &seq = slots_[slot]->tokens;
   const int32_t len = (int32_t)seq.size();
   std::vector<uint32_t> path;
   for (int32_t start = 0; start < len; ++start) {
@@ -527,7 +616,7 @@ void arctic_suffix_tree::remove(int seq_id) {
     path.clear();
     while (idx < len) {
       const int32_t token = seq[idx];
-      const uint32_t child = child_of(node, token);
+      const uint32_t child = find_child(node, token);
       if (child == NIL) break;
       if (nodes_[child].count > 1) {
         count_down(child);
@@ -539,7 +628,8 @@ void arctic_suffix_tree::remove(int seq_id) {
         release_subtree(child);
         break;
       }
-      drop_endpoint(child, seq_id);
+      const uint32_t e = find_endpoint(child, slot);
+      if (e != NIL) drop_endpoint(e);
       idx += nodes_[child].length;
       node = child;
       path.push_back(node);
@@ -555,9 +645,9 @@ void arctic_suffix_tree::remove(int seq_id) {
         c.length += n.length;
         c.ref_idx -= n.length;
         c.parent = n.parent;
+        buckets_.release(n.first_bucket);
         take_place(node, child);
         set_child(c.parent, c.token, child);
-        buckets_.release(n.first_bucket);
         drop_all_endpoints(node);
         nodes_.release(node);
         path.back() = node = child;
@@ -571,7 +661,7 @@ void arctic_suffix_tree::remove(int seq_id) {
       leaf = c;
       distance += nodes_[leaf].length;
     }
-    if (nodes_[leaf].num_endpoints == 0 || endpoint_of(leaf, seq_id) != NIL) continue;  // comes by again later
+    if (nodes_[leaf].num_endpoints == 0 || find_endpoint(leaf, slot) != NIL) continue;  // comes by again later
     const Endpoint &ref = endpoints_[nodes_[leaf].first_endpoint];
     const int32_t ref_seq = ref.seq;
     int32_t ref_idx = ref.end - distance;
@@ -579,25 +669,30 @@ void arctic_suffix_tree::remove(int seq_id) {
       Node &n = nodes_[path.back()];
       path.pop_back();
       ref_idx -= n.length;
-      if (n.ref_seq == seq_id) {
+      if (n.ref_seq == slot) {
         n.ref_seq = ref_seq;
         n.ref_idx = ref_idx;
       }
     }
   }
-  seqs_.erase(found);
+  delete slots_[slot];
+  slots_[slot] = nullptr;
+  free_slots_.push_back(slot);
+  slot_of_.erase(found);
 }
 
 // Walk `context` down from the root (suffix_tree.cc:815-838).
 bool arctic_suffix_tree::match(const int32_t *context, int64_t n, uint32_t &node, int &idx) const {
   node = root_;
   idx = 0;
+  int32_t length = 0;
   const int32_t *text = nullptr;
   for (int64_t i = 0; i < n; ++i) {
-    if (idx >= nodes_[node].length) {
-      node = child_of(node, context[i]);
+    if (idx >= length) {
+      node = find_child(node, context[i]);
       if (node == NIL) return false;
       text = label(node);
+      length = nodes_[node].length;
       idx = 0;
     }
     if (text[idx] != context[i]) return false;
@@ -668,23 +763,46 @@ Draft arctic_suffix_tree::draft_tree(uint32_t node, int idx, int max_tokens, flo
   return d;
 }
 
-// suffix_tree.cc:583-612
+// suffix_tree.cc:583-612.  The reference tries every suffix of the context from the shortest up, stops at
+// the first that is not in the tree, and keeps the draft with the highest score, the longest match
+// winning a tie.  The same answer with less work: the suffixes that are in the tree are exactly those up
+// to some length (a tree of suffixes holds every tail of what it holds), found by bisection; the drafts
+// are then built from the longest match down, a shorter one replacing the best only with a strictly
+// higher score, and the walk ends as soon as no remaining token budget could reach that score (a score
+// is a sum of probabilities, so it never exceeds the number of tokens).
 Draft arctic_suffix_tree::speculate(const int32_t *context, int64_t n, int max_spec_tokens, float max_spec_factor,
                                     float max_spec_offset, float min_token_prob, bool use_tree_spec) {
   Draft best;
-  for (int64_t match_len = 1; match_len < n; ++match_len) {
-    uint32_t node;
-    int idx;
-    if (!match(context + (n - match_len), match_len, node, idx)) break;
-    int max_tokens =
-        std::min(max_spec_tokens, static_cast<int>((int)match_len * max_spec_factor + max_spec_offset + 1e-6));
-    max_tokens = std::max(max_tokens, 0);
-    Draft d = use_tree_spec ? draft_tree(node, idx, max_tokens, min_token_prob)
-                            : draft_path(node, idx, max_tokens, min_token_prob);
-    if (d.score >= best.score) {
-      best = std::move(d);
-      best.match_len = (int)match_len;
+  uint32_t node;
+  int idx;
+  int64_t longest = 0, beyond = n;  // suffixes of length <= longest match; those of length >= beyond do not
+  while (beyond - longest > 1) {
+    const int64_t mid = longest + (beyond - longest) / 2;
+    if (match(context + (n - mid), mid, node, idx)) longest = mid; else beyond = mid;
+  }
+  if (longest == 0) return best;
+  std::vector<int> budget((size_t)longest + 1, 0), budget_below((size_t)longest + 1, 0);
+  for (int64_t m = 1; m <= longest; ++m) {
+    const int tokens =
+        std::min(max_spec_tokens, static_cast<int>((int)m * max_spec_factor + max_spec_offset + 1e-6));
+    budget[m] = std::max(tokens, 0);
+    budget_below[m] = std::max(budget_below[m - 1], budget[m - 1]);  // largest budget of any shorter match
+  }
+  bool have = false;
+  for (int64_t m = longest; m >= 1; --m) {
+    if (have && (float)budget[m] <= best.score) {
+      if ((float)budget_below[m] <= best.score) break;
+      continue;
     }
+    match(context + (n - m), m, node, idx);
+    Draft d = use_tree_spec ? draft_tree(node, idx, budget[m], min_token_prob)
+                            : draft_path(node, idx, budget[m], min_token_prob);
+    if (!have || d.score > best.score) {
+      best = std::move(d);
+      best.match_len = (int)m;
+      have = true;
+    }
+    if ((float)budget_below[m] <= best.score) break;
   }
   return best;
 }
@@ -698,6 +816,7 @@ Draft arctic_suffix_tree::speculate(const int32_t *context, int64_t n, int max_s
 std::string arctic_suffix_tree::check_integrity() {
   // 1. every node: links, order of children, labels, endpoints
   std::vector<uint32_t> order{root_};
+  size_t endpoint_records = 0;
   for (size_t at = 0; at < order.size(); ++at) {
     const uint32_t node = order[at];
     const Node &n = nodes_[node];
@@ -708,14 +827,13 @@ std::string arctic_suffix_tree::check_integrity() {
       const Bucket &k = buckets_[b];
       ARCTIC_EXPECT(k.prev == prev_bucket);
       ARCTIC_EXPECT(k.head != NIL && k.tail != NIL);
-      const int64_t count = nodes_[k.head].count;
-      ARCTIC_EXPECT(last_count < 0 || count < last_count);  // buckets in strictly decreasing count
-      last_count = count;
+      ARCTIC_EXPECT(last_count < 0 || k.count < last_count);  // buckets in strictly decreasing count
+      last_count = k.count;
       uint32_t prev = NIL;
       for (uint32_t c = k.head; c != NIL; c = nodes_[c].next) {
         const Node &ch = nodes_[c];
         ARCTIC_EXPECT(ch.bucket == b && ch.prev == prev && ch.parent == node);
-        ARCTIC_EXPECT(ch.count == count);
+        ARCTIC_EXPECT(ch.count == k.count);
         ARCTIC_EXPECT(child_of(node, ch.token) == c);
         ARCTIC_EXPECT(node == root_ || ch.count < n.count);  // else the two should be one node
         prev = c;
@@ -732,18 +850,18 @@ std::string arctic_suffix_tree::check_integrity() {
       continue;
     }
     ARCTIC_EXPECT(n.length > 0 && n.count > 0);
-    auto ref = seqs_.find(n.ref_seq);
-    ARCTIC_EXPECT(ref != seqs_.end());
-    ARCTIC_EXPECT(n.ref_idx >= 0 && (size_t)(n.ref_idx + n.length) <= ref->second.tokens.size());
-    ARCTIC_EXPECT(n.token == ref->second.tokens[n.ref_idx]);
+    ARCTIC_EXPECT(n.ref_seq >= 0 && (size_t)n.ref_seq < slots_.size() && slots_[n.ref_seq] != nullptr);
+    const std::vector<int32_t> &ref = slots_[n.ref_seq]->tokens;
+    ARCTIC_EXPECT(n.ref_idx >= 0 && (size_t)(n.ref_idx + n.length) <= ref.size());
+    ARCTIC_EXPECT(n.token == ref[n.ref_idx]);
     uint32_t listed = 0;
     for (uint32_t e = n.first_endpoint; e != NIL; e = endpoints_[e].next) {
       const Endpoint &r = endpoints_[e];
       ++listed;
-      ARCTIC_EXPECT(r.node == node && endpoint_of(node, r.seq) == e);
-      auto s = seqs_.find(r.seq);
-      ARCTIC_EXPECT(s != seqs_.end());
-      ARCTIC_EXPECT(r.end > 0 && (size_t)r.end <= s->second.tokens.size());
+      ARCTIC_EXPECT(r.node == node && find_endpoint(node, r.seq) == e);  // also: one record per sequence
+      ARCTIC_EXPECT(r.seq >= 0 && (size_t)r.seq < slots_.size() && slots_[r.seq] != nullptr);
+      const std::vector<int32_t> &s = slots_[r.seq]->tokens;
+      ARCTIC_EXPECT(r.end > 0 && (size_t)r.end <= s.size());
       // the tokens before the endpoint spell the path from the root to here
       int32_t idx = r.end;
       for (uint32_t up = node; up != root_; up = nodes_[up].parent) {
@@ -751,16 +869,19 @@ std::string arctic_suffix_tree::check_integrity() {
         ARCTIC_EXPECT(u.length <= idx);
         idx -= u.length;
         const int32_t *text = label(up);
-        for (int32_t i = 0; i < u.length; ++i) ARCTIC_EXPECT(s->second.tokens[idx + i] == text[i]);
+        for (int32_t i = 0; i < u.length; ++i) ARCTIC_EXPECT(s[idx + i] == text[i]);
       }
     }
     ARCTIC_EXPECT(listed == n.num_endpoints);
+    endpoint_records += listed;
   }
   ARCTIC_EXPECT(order.size() == nodes_.live());
+  ARCTIC_EXPECT(endpoint_records == endpoints_.live());
   // 2. every suffix of every sequence is in the tree, and the counts are the number of visits
   std::unordered_map<uint32_t, int64_t> visits;
-  for (const auto &entry : seqs_) {
-    const std::vector<int32_t> &seq = entry.second.tokens;
+  for (const auto &entry : slot_of_) {
+    ARCTIC_EXPECT(slots_[entry.second] != nullptr && slots_[entry.second]->id == entry.first);
+    const std::vector<int32_t> &seq = slots_[entry.second]->tokens;
     for (size_t start = 0; start < seq.size(); ++start) {
       size_t idx = start;
       uint32_t node = root_;
@@ -775,7 +896,11 @@ std::string arctic_suffix_tree::check_integrity() {
         for (int32_t i = 0; i < n.length; ++i) ARCTIC_EXPECT(seq[idx + i] == text[i]);
         idx += n.length;
       }
-      ARCTIC_EXPECT(endpoint_of(node, entry.first) != NIL);
+      ARCTIC_EXPECT(find_endpoint(node, entry.second) != NIL);
+    }
+    // the growing suffixes point at their own records
+    for (const Growing &g : slots_[entry.second]->active) {
+      ARCTIC_EXPECT(endpoints_[g.endpoint].node == g.node && endpoints_[g.endpoint].seq == entry.second);
     }
   }
   for (uint32_t node : order) ARCTIC_EXPECT(nodes_[node].count == visits[node]);
@@ -784,10 +909,10 @@ std::string arctic_suffix_tree::check_integrity() {
 
 size_t arctic_suffix_tree::estimate_memory() const {
   size_t total = sizeof(*this) + nodes_.bytes() + buckets_.bytes() + endpoints_.bytes() + children_.bytes() +
-                 endpoint_index_.bytes();
-  for (const auto &entry : seqs_)
-    total += sizeof(entry) + entry.second.tokens.capacity() * sizeof(int32_t) +
-             entry.second.active.size() * sizeof(uint32_t);
+                 endpoint_index_.bytes() + slots_.capacity() * sizeof(Sequence *) +
+                 slot_of_.size() * (sizeof(std::pair<int32_t, int32_t>) + 2 * sizeof(void *));
+  for (const Sequence *s : slots_)
+    if (s) total += sizeof(*s) + s->tokens.capacity() * sizeof(int32_t) + s->active.size() * sizeof(Growing);
   return total;
 }
 

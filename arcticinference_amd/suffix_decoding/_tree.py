@@ -97,6 +97,17 @@ class SuffixTree:
         self._handle = _lib.arctic_suffix_tree_create(int(max_depth))
         if not self._handle:
             raise ValueError("SuffixTree: max_depth must be a positive integer")
+        self._score, self._match_len = ctypes.c_float(0.0), ctypes.c_int(0)
+        self._score_ref, self._match_len_ref = ctypes.byref(self._score), ctypes.byref(self._match_len)
+        self._reserve(64)
+
+    def _reserve(self, capacity: int) -> None:
+        # output arrays of speculate, kept between calls
+        self._capacity = capacity
+        self._token_ids = np.empty(capacity, dtype=np.int32)
+        self._parents = np.empty(capacity, dtype=np.int32)
+        self._probs = np.empty(capacity, dtype=np.float32)
+        self._out = (self._token_ids.ctypes.data, self._parents.ctypes.data, self._probs.ctypes.data)
 
     def __del__(self):
         handle, self._handle = getattr(self, "_handle", None), None
@@ -125,16 +136,16 @@ class SuffixTree:
 
     def speculate_ndarray(self, context: np.ndarray, max_spec_tokens: int, max_spec_factor: float,
                           max_spec_offset: float, min_token_prob: float, use_tree_spec: bool) -> Draft:
-        cap = max(int(max_spec_tokens), 0)
-        token_ids = np.empty(cap, dtype=np.int32)
-        parents = np.empty(cap, dtype=np.int32)
-        probs = np.empty(cap, dtype=np.float32)
-        score, match_len = ctypes.c_float(0.0), ctypes.c_int(0)
-        n = _check(_lib.arctic_suffix_tree_speculate(
-            self._handle, context.ctypes.data, context.size, int(max_spec_tokens), max_spec_factor, max_spec_offset,
-            min_token_prob, 1 if use_tree_spec else 0, token_ids.ctypes.data, parents.ctypes.data, probs.ctypes.data,
-            ctypes.byref(score), ctypes.byref(match_len)), "speculate")
-        return Draft(token_ids[:n].tolist(), parents[:n].tolist(), probs[:n].tolist(), score.value, match_len.value)
+        max_spec_tokens = int(max_spec_tokens)
+        if max_spec_tokens > self._capacity:
+            self._reserve(max_spec_tokens)
+        n = _lib.arctic_suffix_tree_speculate(
+            self._handle, context.ctypes.data, context.size, max_spec_tokens, max_spec_factor, max_spec_offset,
+            min_token_prob, 1 if use_tree_spec else 0, *self._out, self._score_ref, self._match_len_ref)
+        if n < 0:
+            _check(n, "speculate")
+        return Draft(self._token_ids[:n].tolist(), self._parents[:n].tolist(), self._probs[:n].tolist(),
+                     self._score.value, self._match_len.value)
 
     def check_integrity(self) -> str:
         """Empty string if every invariant of the tree holds, else a description of the first broken one."""

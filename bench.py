@@ -362,6 +362,75 @@ def bench_row_gather(ops, dev, steps):
     return out
 
 
+def bench_suffix_decoding():
+    """Suffix-tree speculation on the host cores (no GPU): libarctic_suffix.so next to the reference's own
+    code (oracle/_ref, compiled from the reference's sources, when it is there), both driven through the
+    same raw ctypes calls with preallocated buffers.  One global tree of depth 64 over 256 responses of 1024
+    tokens made of recurring phrases (so contexts do match); then decoding steps of 32 requests: speculate
+    from the last 64 tokens (path and tree drafts), append token by token; then eviction of half the cache."""
+    import ctypes
+    import numpy as np
+    from arcticinference_amd.suffix_decoding import _tree
+    from oracle.suffix_ref import RefTree
+
+    rng = np.random.default_rng(11)
+    phrases = [rng.integers(0, 32000, int(rng.integers(8, 40))).astype(np.int32) for _ in range(400)]
+
+    def text(n):
+        out = []
+        while sum(len(p) for p in out) < n:
+            out.append(phrases[int(rng.zipf(1.3)) % len(phrases)] if rng.random() < 0.9
+                       else rng.integers(0, 32000, 5).astype(np.int32))
+        return np.ascontiguousarray(np.concatenate(out)[:n])
+
+    responses = [text(1024) for _ in range(256)]
+    decode = [text(64 + 128) for _ in range(32)]
+    tok, par = np.empty(64, np.int32), np.empty(64, np.int32)
+    prob = np.empty(64, np.float32)
+    score, mlen = ctypes.c_float(), ctypes.c_int()
+    outs = (tok.ctypes.data, par.ctypes.data, prob.ctypes.data, ctypes.byref(score), ctypes.byref(mlen))
+
+    def run(create, extend, speculate, remove):
+        h = create(64)
+        out = {}
+        t0 = time.perf_counter()
+        for i, r in enumerate(responses):
+            extend(h, i, r.ctypes.data, r.size)
+        out["extend_Mtokens_per_s"] = round(len(responses) * 1024 / (time.perf_counter() - t0) / 1e6, 3)
+        for mode, use_tree in (("speculate_path", 0), ("speculate_tree", 1)):
+            jobs = [(d.ctypes.data + 4 * (pos - 64)) for d in decode for pos in range(64, len(d), 4)]
+            t0, drafted = time.perf_counter(), 0
+            for ptr in jobs:
+                drafted += speculate(h, ptr, 64, 16, 2.0, 0.0, 0.1, use_tree, *outs)
+            dt = time.perf_counter() - t0
+            out[mode + "_kcalls_per_s"] = round(len(jobs) / dt / 1e3, 2)
+            out[mode + "_tokens_per_call"] = round(drafted / len(jobs), 2)
+        jobs = [(1000 + j, d.ctypes.data + 4 * pos) for j, d in enumerate(decode) for pos in range(64, len(d))]
+        t0 = time.perf_counter()
+        for sid, ptr in jobs:                                # token-by-token growth of live responses
+            extend(h, sid, ptr, 1)
+        out["append_Mtokens_per_s"] = round(len(jobs) / (time.perf_counter() - t0) / 1e6, 3)
+        t0 = time.perf_counter()
+        for i in range(0, len(responses), 2):
+            remove(h, i)
+        out["remove_sequences_per_s"] = round(len(responses) / 2 / (time.perf_counter() - t0), 1)
+        return out
+
+    lib = _tree._lib
+    mine = run(lib.arctic_suffix_tree_create, lib.arctic_suffix_tree_extend, lib.arctic_suffix_tree_speculate,
+               lib.arctic_suffix_tree_remove)
+    result = {"library": mine, "cores": 1}
+    if RefTree.available():
+        ref_lib = RefTree.lib()
+        ref = run(ref_lib.ref_suffix_tree_create, ref_lib.ref_suffix_tree_extend, ref_lib.ref_suffix_tree_speculate,
+                  ref_lib.ref_suffix_tree_remove)
+        result["reference"] = ref
+        result["speedup"] = {k: round(mine[k] / ref[k], 2) for k in mine if not k.endswith("tokens_per_call")}
+    else:
+        result["reference"] = "oracle/_ref/libsuffix_ref.so not present"
+    return result
+
+
 def box_reference(dev):
     """What plain library kernels reach on this very GPU (boxes of one pool differ by up to 20 %):
     a contiguous bf16 -> fp8 cast of 1.3 GB (the same 2:1 read:write mix as the bulk fp8 write, no
@@ -642,6 +711,7 @@ def main():
         extras["speculator"] = bench_speculator(ops, dev, args.steps, args.warmup)
         extras["decode_mix"] = bench_decode_mix(ops, dev, args.steps)
         extras["swiftkv_select_decode_70b"] = bench_row_gather(ops, dev, args.steps)
+        extras["suffix_decoding_cpu"] = bench_suffix_decoding()
         log(f"extras: {extras}")
 
     result = {

@@ -630,7 +630,8 @@ def main():
             fc()
         extras["bulk_fp8_70b_compact_pool"] = dict(
             kernel_stats(fc, args.steps, wc.bytes),
-            placement="source and 40 caches of 8192 blocks allocated alone on an empty GPU (13 GiB, one HBM region)")
+            placement="source and 40 caches of 8192 blocks allocated first in the process (13 GiB; inside one HBM "
+                      "region when the GPU was idle before)")
         log(f"compact placement: {extras['bulk_fp8_70b_compact_pool']}")
         del wc, fc
         torch.cuda.empty_cache()
@@ -702,7 +703,7 @@ def main():
         m = statistics.median(event_times_us(f2, args.steps))
         extras["bulk_fp8_8b_prefill"] = {"kernel_us": round(m, 2), "GBps": round(w2.bytes / m / 1e3, 1),
                                          "hbm_frac": round(w2.bytes / m / 1e3 / HBM_PEAK_GBS, 4),
-                                         "placement": "source and 16 caches of 8192 blocks allocated alone (one HBM region)"}
+                                         "placement": "source and 16 caches of 8192 blocks allocated together (2.4 GiB)"}
         del w2, f2
         torch.cuda.empty_cache()
         extras["box_reference"] = box_reference(dev)

@@ -75,7 +75,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         vp, vp, vp, vp,        # host tables: key caches, value caches, k scales, v scales
         vp, i64,               # slot_mapping, num_tokens
         i32, i32, i32, i32,    # num_layers, num_heads, head_size, block_size
-        i64, i32, i32, vp]     # block_stride, src_dtype, kv_cache_dtype, stream
+        i64, i64, i32, i32, vp]  # block_stride, num_blocks, src_dtype, kv_cache_dtype, stream
     lib.arctic_reshape_and_cache_flash_bulk.restype = i32
     lib.arctic_reshape_and_cache_flash_fp4.argtypes = [
         vp, vp, i64, i64, vp, vp, vp, vp, vp, i64, i32, i32, i32, i64, i64, i64, i32, vp]

@@ -23,6 +23,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdint>
 #include <cstdlib>
 #include <type_traits>
 
@@ -48,6 +49,7 @@ struct BulkParams {
   int64_t key_stride_bytes;
   int64_t value_stride_bytes;
   int64_t block_stride;  // elements
+  int64_t num_slots;     // slots at or beyond this move nothing
   int num_layers;        // layers in this launch
   int layers_per_group;  // consecutive layers owned by one workgroup
   int groups_per_token;
@@ -160,7 +162,7 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
   int c = threadIdx.x;
   uint4 cur[kUnroll];
   load_batch(c, cur);
-  if (slot < 0) return;  // padding token: uniform exit, before any barrier
+  if (slot < 0 || slot >= p.num_slots) return;  // padding (or a slot outside the cache): uniform exit, before any barrier
 
   int64_t blk, off;
   if (slot < 0x7fffffffLL) {
@@ -221,7 +223,7 @@ __global__ __launch_bounds__(kScalarThreads) void kv_write_bulk_scalar_kernel(
   const int layer0 = group * p.layers_per_group;
   const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
   const int64_t slot = p.slot_mapping[token];
-  if (slot < 0) return;
+  if (slot < 0 || slot >= p.num_slots) return;
   const int64_t blk = slot / p.block_size;
   const int64_t off = slot - blk * p.block_size;
   const int64_t row_elem = blk * p.block_stride + off * (int64_t)p.n;
@@ -308,8 +310,8 @@ extern "C" int arctic_reshape_and_cache_flash_bulk(
     const void *const *key_cache_ptrs, const void *const *value_cache_ptrs,
     const float *const *k_scale_ptrs, const float *const *v_scale_ptrs,
     const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads,
-    int head_size, int block_size, int64_t block_stride, int src_dtype, int kv_cache_dtype,
-    void *stream) {
+    int head_size, int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype,
+    int kv_cache_dtype, void *stream) {
   const char *fn = "reshape_and_cache_flash_bulk";
   if (num_layers == 0 || num_tokens == 0) return ARCTIC_OK;  // reference :87-89
   if (num_layers < 0 || num_layers > ARCTIC_MAX_LAYERS)
@@ -319,6 +321,7 @@ extern "C" int arctic_reshape_and_cache_flash_bulk(
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: num_tokens=%lld outside [0, 2^31)", fn, (long long)num_tokens);
   if (num_heads <= 0 || head_size <= 0 || block_size <= 0)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: num_heads, head_size and block_size must be positive", fn);
+  if (num_blocks < 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: negative num_blocks", fn);
   if (src_dtype != ARCTIC_DTYPE_F32 && src_dtype != ARCTIC_DTYPE_F16 && src_dtype != ARCTIC_DTYPE_BF16)
     return fail(ARCTIC_ERR_UNSUPPORTED, "%s: Unsupported input type of kv cache: %d", fn, src_dtype);
   if (kv_cache_dtype != ARCTIC_KV_AUTO && kv_cache_dtype != ARCTIC_KV_FP8_E4M3 &&
@@ -368,6 +371,7 @@ extern "C" int arctic_reshape_and_cache_flash_bulk(
     p.key_stride_bytes = key_stride * es;
     p.value_stride_bytes = value_stride * es;
     p.block_stride = block_stride;
+    p.num_slots = num_blocks > 0 ? num_blocks * (int64_t)block_size : INT64_MAX;
     p.num_layers = count;
     p.n = n;
     p.block_size = block_size;

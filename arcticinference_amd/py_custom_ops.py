@@ -203,7 +203,7 @@ def _reshape_and_cache_flash_bulk_impl(
             _ptr_table(key_caches), _ptr_table(value_caches),
             _ptr_table(k_scales), _ptr_table(v_scales),
             slot_mapping.data_ptr(), num_tokens, num_layers, int(num_heads), int(head_size),
-            int(block_size), int(block_stride), src_code, kv_code, _stream_of(keys))
+            int(block_size), int(block_stride), int(key_caches[0].size(0)), src_code, kv_code, _stream_of(keys))
     _native.check(rc)
 
 

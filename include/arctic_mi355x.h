@@ -85,6 +85,9 @@ const char *arctic_last_error(void);
  *   slot_mapping        device int64[num_tokens]
  *   block_stride        ELEMENTS between consecutive cache blocks (same for K and
  *                       V); inside a block the layout is [block_size][n] dense
+ *   num_blocks          blocks in every cache; a slot >= num_blocks * block_size
+ *                       moves nothing, like a negative one (the reference writes
+ *                       out of bounds there).  0 = unknown, slots are not checked.
  * Distinct valid slots are required for a deterministic result (as in the
  * reference).  num_layers == 0 or num_tokens == 0 is a successful no-op.
  */
@@ -94,8 +97,8 @@ int arctic_reshape_and_cache_flash_bulk(
     const void *const *value_cache_ptrs, const float *const *k_scale_ptrs,
     const float *const *v_scale_ptrs, const int64_t *slot_mapping,
     int64_t num_tokens, int num_layers, int num_heads, int head_size,
-    int block_size, int64_t block_stride, int src_dtype, int kv_cache_dtype,
-    void *stream);
+    int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype,
+    int kv_cache_dtype, void *stream);
 
 /*
  * NVFP4-style KV-cache write for ONE layer: e2m1 values, two per byte (first element

@@ -70,17 +70,17 @@ def test_argument_errors_return_codes_without_launching(lib):
     rc = lib.arctic_sum_lstm(*([None] * 9), 4, 64, 256, 256, 64, 64, 1.0, 1e-6, 1e-6, 0, _native.DTYPE_F32, None)
     assert rc == 2 and b"sum_lstm: only fp16 and bf16" in lib.arctic_last_error()
     rc = lib.arctic_reshape_and_cache_flash_bulk(None, None, 0, 0, None, None, None, None, None, 4, 2, 2, 64, 16, 0,
-                                                 _native.DTYPE_BF16, 7, None)
+                                                 0, _native.DTYPE_BF16, 7, None)
     assert rc == 2 and b"Unsupported data type of kv cache" in lib.arctic_last_error()
     rc = lib.arctic_reshape_and_cache_flash_bulk(None, None, 0, 0, None, None, None, None, None, 4, 2, 2, 64, 16, 0,
-                                                 9, _native.KV_AUTO, None)
+                                                 0, 9, _native.KV_AUTO, None)
     assert rc == 2 and b"Unsupported input type of kv cache" in lib.arctic_last_error()
     rc = lib.arctic_reshape_and_cache_flash_bulk(None, None, 0, 0, None, None, None, None, None, 4, 100000, 2, 64, 16,
-                                                 0, _native.DTYPE_BF16, _native.KV_AUTO, None)
+                                                 0, 0, _native.DTYPE_BF16, _native.KV_AUTO, None)
     assert rc == 1 and b"num_layers" in lib.arctic_last_error()
     # empty problems are successful no-ops (reference: reshape_and_cache_flash_bulk.cu:87-89)
     assert lib.arctic_reshape_and_cache_flash_bulk(None, None, 0, 0, None, None, None, None, None, 4, 0, 2, 64, 16, 0,
-                                                   _native.DTYPE_BF16, _native.KV_AUTO, None) == 0
+                                                   0, _native.DTYPE_BF16, _native.KV_AUTO, None) == 0
     assert lib.arctic_speculator_ln(None, None, None, None, 0, 128, 128, 1e-6, _native.DTYPE_BF16, None) == 0
 
 

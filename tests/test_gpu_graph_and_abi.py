@@ -144,7 +144,7 @@ def test_direct_c_abi_calls(ops):
     rc = lib.arctic_reshape_and_cache_flash_bulk(
         d["keys"].data_ptr(), d["values"].data_ptr(), d["keys"].stride(0), d["values"].stride(0),
         tab(d["key_caches"]), tab(d["value_caches"]), tab(d["k_scales"]), tab(d["v_scales"]),
-        d["slot_mapping"].data_ptr(), 20, L, 2, 64, 8, d["key_caches"][0].stride(0), _native.DTYPE_BF16,
+        d["slot_mapping"].data_ptr(), 20, L, 2, 64, 8, d["key_caches"][0].stride(0), 4, _native.DTYPE_BF16,
         _native.KV_FP8_E4M3, stream)
     assert rc == 0, lib.arctic_last_error()
     torch.cuda.synchronize()

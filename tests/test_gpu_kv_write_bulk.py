@@ -62,6 +62,21 @@ def test_all_padding_leaves_cache_untouched(ops):
     assert_bulk_equal(dcase["bufs"], before)
 
 
+def test_slots_outside_the_cache_move_nothing(ops):
+    """A slot at or beyond num_blocks * block_size is skipped like a padding slot (the reference would
+    write out of bounds); the other tokens are written as usual."""
+    case = make_bulk_case(T=24, L=3, H=2, D=64, bs=16, NB=4, kv_cache_dtype="fp8", seed=8, pad_fraction=0.1)
+    bad = [1, 7, 20]
+    for t, slot in zip(bad, (4 * 16, 4 * 16 + 5, 1 << 40)):
+        case["slot_mapping"][t] = slot
+    dcase = bulk_case_to(case, DEV)
+    ops.reshape_and_cache_flash_bulk(*bulk_args(dcase))
+    torch.cuda.synchronize()
+    case["slot_mapping"][bad] = -1           # what the oracle has to see to do the same
+    oracle.reshape_and_cache_flash_bulk(*bulk_args(case))
+    assert_bulk_equal(dcase["bufs"], case["bufs"])
+
+
 def test_empty_inputs(ops):
     case = make_bulk_case(T=4, L=2, H=2, D=64, bs=16, NB=2, seed=1)
     dcase = bulk_case_to(case, DEV)

@@ -78,7 +78,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         i64, i64, i32, i32, vp]  # block_stride, num_blocks, src_dtype, kv_cache_dtype, stream
     lib.arctic_reshape_and_cache_flash_bulk.restype = i32
     lib.arctic_reshape_and_cache_flash_fp4.argtypes = [
-        vp, vp, i64, i64, vp, vp, vp, vp, vp, i64, i32, i32, i32, i64, i64, i64, i32, vp]
+        vp, vp, i64, i64, vp, vp, vp, vp, vp, i64, i32, i32, i32, i64, i64, i64, i64, i32, vp]
     lib.arctic_reshape_and_cache_flash_fp4.restype = i32
     lib.arctic_speculator_ln.argtypes = [vp, vp, vp, vp, i64, i32, i64, f32, i32, vp]
     lib.arctic_speculator_ln.restype = i32

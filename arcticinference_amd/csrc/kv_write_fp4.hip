@@ -11,6 +11,8 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <cstdint>
+
 #include "common.hpp"
 
 namespace arctic {
@@ -29,6 +31,7 @@ struct Fp4Params {
   int64_t page_stride;
   int64_t head_stride;
   int64_t total_groups;  // num_tokens * 2 * num_heads * groups_per_head
+  int64_t num_slots;     // slots at or beyond this move nothing
   int num_heads;
   int groups_per_head;   // head_size / 16
   int block_size;
@@ -47,7 +50,7 @@ __global__ __launch_bounds__(256) void kv_write_fp4_kernel(const Fp4Params p) {
   const bool is_v = row & 1;
 
   const int64_t slot = p.slot_mapping[token];
-  if (slot < 0) return;  // padding token
+  if (slot < 0 || slot >= p.num_slots) return;  // padding token, or a slot outside the cache
   const int64_t blk = slot / p.block_size;
   const int64_t off = slot - blk * p.block_size;
 
@@ -101,7 +104,7 @@ extern "C" int arctic_reshape_and_cache_flash_fp4(
     const void *key, const void *value, int64_t key_stride, int64_t value_stride, void *key_cache,
     void *value_cache, void *key_scale_cache, void *value_scale_cache, const int64_t *slot_mapping,
     int64_t num_tokens, int num_heads, int head_size, int block_size, int64_t block_stride,
-    int64_t page_stride, int64_t head_stride, int dtype, void *stream) {
+    int64_t page_stride, int64_t head_stride, int64_t num_blocks, int dtype, void *stream) {
   const char *fn = "reshape_and_cache_flash_fp4";
   if (dtype != ARCTIC_DTYPE_F16 && dtype != ARCTIC_DTYPE_BF16)
     return fail(ARCTIC_ERR_UNSUPPORTED,
@@ -135,6 +138,7 @@ extern "C" int arctic_reshape_and_cache_flash_fp4(
   p.groups_per_head = head_size / 16;
   p.block_size = block_size;
   p.total_groups = num_tokens * 2 * num_heads * p.groups_per_head;
+  p.num_slots = num_blocks > 0 ? num_blocks * (int64_t)block_size : INT64_MAX;
   const int64_t grid = (p.total_groups + 255) / 256;
   if (grid > 0x7fffffffLL) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: too many tokens", fn);
   hipStream_t s = (hipStream_t)stream;

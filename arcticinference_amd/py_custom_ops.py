@@ -255,7 +255,7 @@ def _reshape_and_cache_flash_fp4_impl(
             key.data_ptr(), value.data_ptr(), key.stride(0), value.stride(0), key_cache.data_ptr(),
             value_cache.data_ptr(), key_scale_cache.data_ptr(), value_scale_cache.data_ptr(),
             slot_mapping.data_ptr(), num_tokens, num_heads, head_size, int(block_size), int(block_stride),
-            int(page_stride), int(head_stride), _HALF_DTYPES[key.dtype], _stream_of(key))
+            int(page_stride), int(head_stride), int(key_cache.size(0)), _HALF_DTYPES[key.dtype], _stream_of(key))
     _native.check(rc)
 
 

@@ -121,13 +121,16 @@ int arctic_reshape_and_cache_flash_bulk(
  *
  *   key, value   device; [num_tokens, num_heads*head_size] F16 or BF16, row strides in ELEMENTS,
  *                16-byte aligned rows; head_size % 16 == 0
+ *   num_blocks   blocks in each cache; a slot >= num_blocks * block_size moves nothing.
+ *                0 = unknown, slots are not checked.
  */
 int arctic_reshape_and_cache_flash_fp4(
     const void *key, const void *value, int64_t key_stride, int64_t value_stride,
     void *key_cache, void *value_cache, void *key_scale_cache,
     void *value_scale_cache, const int64_t *slot_mapping, int64_t num_tokens,
     int num_heads, int head_size, int block_size, int64_t block_stride,
-    int64_t page_stride, int64_t head_stride, int dtype, void *stream);
+    int64_t page_stride, int64_t head_stride, int64_t num_blocks, int dtype,
+    void *stream);
 
 /*
  * Speculator "LayerNorm" (an RMS norm with optional scale and shift).  Replaces

@@ -37,6 +37,20 @@ def test_random(ops, dtype, nhd, shape):
     run_both(ops, *make_case(T, H, D, bs, NB, dtype, nhd, seed=21))
 
 
+@pytest.mark.parametrize("nhd", [True, False])
+def test_slots_outside_the_cache_move_nothing(ops, nhd):
+    key, value, kc, vc, ksc, vsc, slots = make_case(20, 4, 64, 8, 3, torch.bfloat16, nhd, seed=23)
+    bad = [2, 11]
+    d = [t.to(DEV) for t in (key, value, kc, vc, ksc, vsc, slots)]
+    d[6][bad[0]], d[6][bad[1]] = 3 * 8, 1 << 35          # first slot past the end, and far past it
+    ops.reshape_and_cache_flash_fp4(d[0], d[1], d[2], d[3], d[4], d[5], d[6], "fp4", ZERO.to(DEV), ZERO.to(DEV))
+    torch.cuda.synchronize()
+    slots[bad] = -1                                       # what the oracle has to see to do the same
+    oracle.reshape_and_cache_flash_fp4(key, value, kc, vc, ksc, vsc, slots, "fp4", ZERO, ZERO)
+    for got, want in zip(d[2:6], (kc, vc, ksc, vsc)):
+        assert torch.equal(got.cpu(), want)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_every_finite_sixteen_bit_value(ops, dtype):
     """All 16-bit patterns as inputs (NaN patterns replaced by 0: the NaN nibble is unpinned),

@@ -117,6 +117,10 @@ __device__ __forceinline__ void store16_stream(void *p, const uint4 &v) {
   *(ARCTIC_GLOBAL u32x4 *)p = t;
 #endif
 }
+__device__ __forceinline__ void store16(void *p, const uint4 &v) {  // stays in the caches: read again soon
+  const u32x4 t = {v.x, v.y, v.z, v.w};
+  *(ARCTIC_GLOBAL u32x4 *)p = t;
+}
 __device__ __forceinline__ void store8_stream(void *p, const uint2 &v) {
   const u32x2 t = {v.x, v.y};
 #if ARCTIC_NT_STORE
@@ -146,6 +150,7 @@ struct Chunk<8> {
   __device__ static __forceinline__ Chunk load(const void *p) { return Chunk{load16(p)}; }
   __device__ static __forceinline__ Chunk load_stream(const void *p) { return Chunk{load16_stream(p)}; }
   __device__ __forceinline__ void store_stream(void *p) const { store16_stream(p, v); }
+  __device__ __forceinline__ void store(void *p) const { store16(p, v); }
   template <typename T>
   __device__ __forceinline__ void unpack(float (&f)[8]) const { unpack8<T>(v, f); }
   template <typename T>

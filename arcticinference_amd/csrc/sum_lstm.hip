@@ -97,7 +97,9 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
     zf[k] = kSharedZ ? zc[k] : C::load_stream(z_row + off[k]);
   }
 #pragma unroll
-  for (int k = 0; k < K; ++k) pc[k] = C::load_stream(pc_row + off[k]);
+  // the cell comes straight from the previous step's launch and both outputs are read by the next
+  // kernels of the step, so these three accesses stay in the caches; the gates are touched once and stream
+  for (int k = 0; k < K; ++k) pc[k] = C::load(pc_row + off[k]);
 #pragma unroll
   for (int k = 0; k < K; ++k) {
     si[k] = C::load_stream(s_row + gate_bytes + off[k]);
@@ -169,7 +171,7 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
       cell[k][j] = cnew;
     }
     const C packed = C::template pack<T>(cell[k]);
-    if (live[k]) packed.store_stream(oc_row + off[k]);
+    if (live[k]) packed.store(oc_row + off[k]);
     packed.template unpack<T>(cell[k]);
   }
   const float inv_cnew = rsqrtf(block_sum(ss, slots_cnew) * p.inv_D + p.eps_state);
@@ -193,7 +195,7 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
     zo[k].template unpack<T>(g);
 #pragma unroll
     for (int j = 0; j < E; ++j) st[j] *= sigmoid_f(fmaf(p.alpha, g[j], a[j]));
-    if (live[k]) C::template pack<T>(st).store_stream(os_row + off[k]);
+    if (live[k]) C::template pack<T>(st).store(os_row + off[k]);
   }
 }
 

@@ -162,6 +162,9 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
     pc[k].template unpack<T>(c);
 #pragma unroll
     for (int j = 0; j < E; ++j) cell[k][j] = sigmoid_f(fmaf(p.alpha, b[j], a[j])) * c[j];
+    // keep the forget-gate arithmetic ahead of the wait for the input gate: it then runs while that gate
+    // is still arriving instead of in the short stretch between the last two gates
+    __builtin_amdgcn_sched_barrier(0);
     si[k].template unpack<T>(a);
     zi[k].template unpack<T>(b);
 #pragma unroll

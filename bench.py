@@ -706,6 +706,22 @@ def main():
                                          "placement": "source and 16 caches of 8192 blocks allocated together (2.4 GiB)"}
         del w2, f2
         torch.cuda.empty_cache()
+        # the same shape on the memory map of an 8B serving process: 8 GiB of weights, then the pool of all 32
+        # layers sized like the 70B one, to fill 90 % of the HBM (229376 blocks = 7 GiB per layer); layers 16-31
+        # are written
+        try:
+            mem8 = ServingMemoryMap(dev, 8, 32, 16, 229376, 16, 8, 128, torch.uint8)
+            w3 = BulkWorkload("8B-prefill-serving", 8192, 16, 8, 128, 16, 229376, "fp8", 0.0, 1, 1.5, dev,
+                              bufs=mem8.written_layers())
+            f3 = lambda: ops.reshape_and_cache_flash_bulk(*w3.args())
+            for _ in range(5):
+                f3()
+            extras["bulk_fp8_8b_prefill_serving_map"] = dict(kernel_stats(f3, args.steps, w3.bytes),
+                                                             memory_map=mem8.describe())
+            del mem8, w3, f3
+        except torch.OutOfMemoryError:
+            extras["bulk_fp8_8b_prefill_serving_map"] = "not enough free device memory"
+        torch.cuda.empty_cache()
         extras["box_reference"] = box_reference(dev)
         extras["fp4_write_8b_layer"] = bench_fp4(ops, dev, args.steps)
         torch.cuda.empty_cache()

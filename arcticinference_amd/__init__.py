@@ -12,6 +12,7 @@ from .py_custom_ops import (  # noqa: F401
     reshape_and_cache_flash_bulk,
     scatter_rows,
     speculator_add_ln_gelu,
+    speculator_argmax,
     speculator_ln,
     speculator_ln_scaled,
     sum_lstm,

@@ -31,6 +31,7 @@ EXPORTED_SYMBOLS = (
     "arctic_sum_lstm",
     "arctic_sum_lstm_shared_z",
     "arctic_gather_rows",
+    "arctic_argmax_clamp",
 )
 
 _lib: Optional[ctypes.CDLL] = None
@@ -90,6 +91,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.arctic_sum_lstm_shared_z.restype = i32
     lib.arctic_gather_rows.argtypes = [i32, vp, vp, vp, vp, vp, vp, i32, i64, i64, i32, vp]
     lib.arctic_gather_rows.restype = i32
+    lib.arctic_argmax_clamp.argtypes = [vp, vp, i64, i32, i64, i64, i32, vp]
+    lib.arctic_argmax_clamp.restype = i32
 
 
 def load() -> ctypes.CDLL:

@@ -1,0 +1,189 @@
+// Row-wise argmax with clamping, gfx950.
+//
+// Stands for the token selection at the end of every speculator step,
+//   last_tokens = torch.argmax(logits, dim=-1); last_tokens.clamp_(0, vocab_size - 1)
+// (arctic_inference/vllm/spec_dec/arctic_speculator.py:846-848, 862), with torch's rules for the winner:
+// the largest value, the lowest index among equal values, and a NaN beats every number (the first NaN wins).
+//
+// One workgroup per row; a lane walks 16-byte chunks of the row with streaming loads and keeps its own
+// (value, index) winner; winners are merged inside the wave with lane exchanges and across the waves
+// through LDS.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+
+#include "common.hpp"
+
+namespace arctic {
+
+struct Winner {
+  float value;
+  int index;   // -1: nothing seen yet
+};
+
+// torch's GreaterOrNan with the index as tie break (aten/src/ATen/native/SharedReduceOps.h)
+__device__ __forceinline__ bool beats(float a, int ia, float b, int ib) {
+  if (ib < 0) return true;
+  if (ia < 0) return false;
+  const bool a_nan = a != a, b_nan = b != b;
+  if (a_nan) return b_nan ? ia < ib : true;
+  if (b_nan) return false;
+  return a == b ? ia < ib : a > b;
+}
+
+__device__ __forceinline__ void offer(Winner &w, float v, int i) {
+  if (beats(v, i, w.value, w.index)) {
+    w.value = v;
+    w.index = i;
+  }
+}
+
+__device__ __forceinline__ Winner wave_winner(Winner w) {
+#pragma unroll
+  for (int step = 32; step >= 1; step >>= 1) {
+    const float ov = __shfl_xor(w.value, step, 64);
+    const int oi = __shfl_xor(w.index, step, 64);
+    offer(w, ov, oi);
+  }
+  return w;
+}
+
+struct F32Elem {
+  static constexpr int kPerChunk = 4;
+  __device__ static __forceinline__ void unpack(const uint4 &v, float (&f)[8]) {
+    f[0] = __uint_as_float(v.x);
+    f[1] = __uint_as_float(v.y);
+    f[2] = __uint_as_float(v.z);
+    f[3] = __uint_as_float(v.w);
+  }
+  __device__ static __forceinline__ float one(const void *p, int64_t i) { return ((const float *)p)[i]; }
+};
+template <typename T>
+struct HalfElem {
+  static constexpr int kPerChunk = 8;
+  __device__ static __forceinline__ void unpack(const uint4 &v, float (&f)[8]) { unpack8<T>(v, f); }
+  __device__ static __forceinline__ float one(const void *p, int64_t i) {
+    return T::lo((uint32_t)((const uint16_t *)p)[i]);
+  }
+};
+
+// kVec: rows are 16-byte aligned, so the body of a row is read in 16-byte chunks; the elements behind
+// the last whole chunk (and everything when !kVec) are read one by one.
+template <typename Elem, bool kVec>
+__global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ out, const char *__restrict__ in,
+                                                          int64_t row_stride_bytes, int cols, int64_t max_index) {
+  __shared__ float wave_value[16];
+  __shared__ int wave_index[16];
+  const char *row = in + (int64_t)blockIdx.x * row_stride_bytes;
+  // Per lane: the largest number seen and where (a strict ">" keeps the earlier of equal values, the
+  // lane's indices only grow), and apart from that the first NaN.  A chunk's sum is NaN only if the
+  // chunk holds a NaN (or infinities of both signs), so the per-element NaN test runs almost never.
+  constexpr int P = Elem::kPerChunk;
+  const int chunks = kVec ? cols / P : 0;
+  // the lane's first element stands in for "nothing below -inf here": a row of -inf must answer 0
+  float best = -__builtin_inff();
+  int best_at = (int)threadIdx.x < chunks ? (int)threadIdx.x * P
+                                           : (chunks * P + (int)threadIdx.x < cols ? chunks * P + (int)threadIdx.x : -1);
+  int nan_at = 0x7fffffff;
+  auto number = [&](float v, int i) {
+    if (v > best) {
+      best = v;
+      best_at = i;
+    }
+  };
+  int done = 0;
+  if (kVec) {
+    constexpr int kUnroll = 4;
+    for (int c0 = threadIdx.x; c0 < chunks; c0 += kUnroll * blockDim.x) {
+      uint4 raw[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int c = c0 + u * blockDim.x;
+        if (c < chunks) raw[u] = load16_stream(row + (int64_t)c * 16);
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int c = c0 + u * blockDim.x;
+        if (c < chunks) {
+          float f[8];
+          Elem::unpack(raw[u], f);
+          float sum = 0.f;
+#pragma unroll
+          for (int j = 0; j < P; ++j) {
+            number(f[j], c * P + j);
+            sum += f[j];
+          }
+          if (sum != sum) {
+#pragma unroll
+            for (int j = 0; j < P; ++j)
+              if (f[j] != f[j]) nan_at = min(nan_at, c * P + j);
+          }
+        }
+      }
+    }
+    done = chunks * P;
+  }
+  for (int i = done + threadIdx.x; i < cols; i += blockDim.x) {
+    const float v = Elem::one(row, i);
+    number(v, i);
+    if (v != v) nan_at = min(nan_at, i);
+  }
+  Winner w = nan_at != 0x7fffffff ? Winner{__builtin_nanf(""), nan_at} : Winner{best, best_at};
+
+  w = wave_winner(w);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0) {
+    wave_value[wave] = w.value;
+    wave_index[wave] = w.index;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    const int waves = blockDim.x >> 6;
+    Winner x = {0.f, -1};
+    if (lane < waves) x = Winner{wave_value[lane], wave_index[lane]};
+    x = wave_winner(x);
+    if (lane == 0) {
+      int64_t idx = x.index < 0 ? 0 : x.index;
+      out[blockIdx.x] = idx > max_index ? max_index : idx;
+    }
+  }
+}
+
+}  // namespace arctic
+
+using namespace arctic;
+
+extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t rows, int cols, int64_t row_stride,
+                                   int64_t max_index, int dtype, void *stream) {
+  const char *fn = "argmax_clamp";
+  if (dtype != ARCTIC_DTYPE_F32 && dtype != ARCTIC_DTYPE_F16 && dtype != ARCTIC_DTYPE_BF16)
+    return fail(ARCTIC_ERR_UNSUPPORTED, "%s: logits must be fp32, fp16 or bf16", fn);
+  if (rows < 0 || rows > 0x7fffffffLL || cols <= 0 || max_index < 0 || row_stride < 0)
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: rows >= 0, cols > 0, max_index >= 0 and a non-negative pitch are required",
+                fn);
+  if (rows == 0) return ARCTIC_OK;
+  if (!out || !logits) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
+  const int es = dtype == ARCTIC_DTYPE_F32 ? 4 : 2;
+  const int64_t stride_bytes = row_stride * es;
+  const bool vec = ((uintptr_t)logits % 16 == 0) && (stride_bytes % 16 == 0 || rows == 1);
+  const int per_chunk = 16 / es;
+  int threads = (int)std::min<int64_t>(1024, std::max<int64_t>(64, ((cols / per_chunk / 4 + 63) / 64) * 64));
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)rows), block((unsigned)threads);
+#define ARCTIC_ARGMAX_LAUNCH(ELEM)                                                                          \
+  do {                                                                                                      \
+    if (vec)                                                                                                \
+      hipLaunchKernelGGL((row_argmax_kernel<ELEM, true>), grid, block, 0, s, out, (const char *)logits,     \
+                         stride_bytes, cols, max_index);                                                    \
+    else                                                                                                    \
+      hipLaunchKernelGGL((row_argmax_kernel<ELEM, false>), grid, block, 0, s, out, (const char *)logits,    \
+                         stride_bytes, cols, max_index);                                                    \
+  } while (0)
+  if (dtype == ARCTIC_DTYPE_F32) ARCTIC_ARGMAX_LAUNCH(F32Elem);
+  else if (dtype == ARCTIC_DTYPE_BF16) ARCTIC_ARGMAX_LAUNCH(HalfElem<BF16>);
+  else ARCTIC_ARGMAX_LAUNCH(HalfElem<F16>);
+#undef ARCTIC_ARGMAX_LAUNCH
+  return check_launch(fn);
+}

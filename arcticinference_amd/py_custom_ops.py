@@ -45,6 +45,7 @@ _SCHEMAS = {
         "float eps_state, bool use_fast_gelu) -> (Tensor, Tensor)",
     "gather_rows": "gather_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
     "scatter_rows": "scatter_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
+    "speculator_argmax_cuda": "speculator_argmax_cuda(Tensor logits, int max_index) -> Tensor",
     "speculator_add_ln_act_cuda":
         "speculator_add_ln_act_cuda(Tensor input, Tensor? z, Tensor? weight, Tensor? bias, float alpha, "
         "float eps, str activation, float out_scale) -> Tensor",
@@ -458,7 +459,30 @@ def _scatter_rows_impl(sources: List[torch.Tensor], indices: torch.Tensor, outs:
     _move_rows_impl("scatter_rows", sources, indices, outs, True)
 
 
+def _speculator_argmax_impl(logits: torch.Tensor, max_index: int) -> torch.Tensor:
+    """``torch.argmax(logits, dim=-1).clamp_(0, max_index)`` in one launch
+    (arctic_inference/vllm/spec_dec/arctic_speculator.py:846-848, 862)."""
+    lib = _lib()
+    _check(logits.is_cuda, "speculator_argmax: logits must be CUDA")
+    _check(logits.dtype in _SRC_DTYPES, "speculator_argmax: logits must be fp32, fp16 or bf16")
+    _check(logits.dim() >= 1 and logits.size(-1) > 0, "speculator_argmax: logits need a non-empty last dimension")
+    _check(logits.stride(-1) == 1, "speculator_argmax: last dimension must be contiguous")
+    _check(max_index >= 0, "speculator_argmax: max_index must not be negative")
+    cols = logits.size(-1)
+    in_2d = logits.view(-1, cols)
+    rows = in_2d.size(0)
+    out = torch.empty(logits.shape[:-1], dtype=torch.int64, device=logits.device)
+    if rows == 0:
+        return out
+    with _on_device_of(logits):
+        rc = lib.arctic_argmax_clamp(out.data_ptr(), in_2d.data_ptr(), rows, cols, in_2d.stride(0), int(max_index),
+                                     _SRC_DTYPES[logits.dtype], _stream_of(logits))
+    _native.check(rc)
+    return out
+
+
 _IMPLS = {
+    "speculator_argmax_cuda": _speculator_argmax_impl,
     "gather_rows": _gather_rows_impl,
     "scatter_rows": _scatter_rows_impl,
     "sum_lstm_shared_z_cuda": _sum_lstm_shared_z_impl,
@@ -668,3 +692,10 @@ def scatter_rows(sources: List[torch.Tensor], indices: torch.Tensor, outs: List[
     ``orig_hidden_states[logits_indices] = hidden_states[:batch_size]``
     (arctic_inference/vllm/swiftkv/llama_swiftkv.py:733-742)."""
     _call("scatter_rows", list(sources), indices, list(outs))
+
+
+def speculator_argmax(logits: torch.Tensor, vocab_size: int) -> torch.Tensor:
+    """``torch.argmax(logits, dim=-1)`` followed by ``.clamp_(0, vocab_size - 1)`` in one launch: the token
+    selection at the end of a speculator step (arctic_inference/vllm/spec_dec/arctic_speculator.py:846-848,
+    862).  Same winner as torch: lowest index among equal values, a NaN beats every number."""
+    return _call("speculator_argmax_cuda", logits, int(vocab_size) - 1)

@@ -431,6 +431,31 @@ def bench_suffix_decoding():
     return result
 
 
+def bench_argmax(ops, dev, steps):
+    """Token selection at the end of a speculator step (arctic_speculator.py:846-848, 862): argmax over a
+    128256-wide vocabulary for 512 rows of bf16 logits (131 MB), clamped; one launch against torch's
+    argmax + clamp_.  Three rotating sets keep the logits out of the last-level cache."""
+    T, V, sets = 512, 128256, 3
+    g = torch.Generator(device=dev).manual_seed(8)
+    logits = [torch.randn(T, V, generator=g, device=dev).to(torch.bfloat16) for _ in range(sets)]
+    nbytes = T * V * 2 + T * 8
+    out = {"bytes_per_call": nbytes}
+    for name, fn in (("speculator_argmax", lambda i: ops.speculator_argmax(logits[i % sets], V)),
+                     ("torch_argmax_clamp", lambda i: torch.argmax(logits[i % sets], dim=-1).clamp_(0, V - 1))):
+        for i in range(3):
+            fn(i)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(sets):
+                fn(i)
+        graph.replay()
+        torch.cuda.synchronize()
+        med = statistics.median(event_times_us(graph.replay, max(10, steps // 2))) / sets
+        out[name] = {"us_per_call_graph": round(med, 2), "GBps": round(nbytes / med / 1e3, 1),
+                     "hbm_frac": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
+    return out
+
+
 def box_reference(dev):
     """What plain library kernels reach on this very GPU (boxes of one pool differ by up to 20 %):
     a contiguous bf16 -> fp8 cast of 1.3 GB (the same 2:1 read:write mix as the bulk fp8 write, no
@@ -728,6 +753,7 @@ def main():
         extras["speculator"] = bench_speculator(ops, dev, args.steps, args.warmup)
         extras["decode_mix"] = bench_decode_mix(ops, dev, args.steps)
         extras["swiftkv_select_decode_70b"] = bench_row_gather(ops, dev, args.steps)
+        extras["speculator_argmax_512x128256"] = bench_argmax(ops, dev, args.steps)
         extras["suffix_decoding_cpu"] = bench_suffix_decoding()
         log(f"extras: {extras}")
 

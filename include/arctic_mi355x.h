@@ -252,6 +252,20 @@ int arctic_gather_rows(int num_tensors, const void *const *src, void *const *dst
                        int index_bytes, int64_t num_indices, int64_t num_indexed_rows,
                        int scatter, void *stream);
 
+/*
+ * Row-wise argmax with clamping.  No native function of the reference corresponds to it; it stands for the
+ * token selection that ends every speculator step,
+ *   last_tokens = torch.argmax(logits, dim=-1); last_tokens.clamp_(0, vocab_size - 1)
+ *        arctic_inference/vllm/spec_dec/arctic_speculator.py:846-848, 862
+ * with torch's rules: the largest value wins, the lowest index among equal values, and a NaN beats every
+ * number (the first NaN wins).
+ *
+ *   out         device int64[rows]: min(argmax_j logits[r][j], max_index)
+ *   logits      device; rows of `cols` elements (F32, F16 or BF16), row_stride ELEMENTS apart
+ */
+int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t rows, int cols,
+                        int64_t row_stride, int64_t max_index, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

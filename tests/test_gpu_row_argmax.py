@@ -1,0 +1,73 @@
+"""GPU parity of speculator_argmax (torch.argmax(logits, -1).clamp_(0, vocab_size - 1),
+arctic_speculator.py:846-848, 862) against torch itself: exact indices."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def reference(logits, vocab_size):
+    # the reference's expression, on the CPU in fp32 (every 16-bit value is exact in fp32, so the order and
+    # the ties are the same)
+    return torch.argmax(logits.float().cpu(), dim=-1).clamp_(0, vocab_size - 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(512, 128256), (64, 32000), (7, 513), (3, 5, 1000), (9, 1), (2, 7), (33, 4100)])
+def test_random_logits(ops, dtype, shape):
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn(*shape, generator=g).to(dtype)          # bf16 makes many exact ties
+    got = ops.speculator_argmax(logits.to(DEV), shape[-1])
+    assert got.dtype == torch.int64 and got.shape == logits.shape[:-1]
+    assert torch.equal(got.cpu(), reference(logits, shape[-1]))
+    # the GPU's own torch.argmax agrees as well
+    assert torch.equal(got, torch.argmax(logits.to(DEV), dim=-1))
+
+
+def test_ties_take_the_lowest_index(ops):
+    x = torch.zeros(6, 5000, dtype=torch.bfloat16)
+    x[1, 4097], x[1, 77], x[1, 4999] = 3.0, 3.0, 3.0
+    x[2] = -float("inf")                                            # a row of -inf answers 0
+    x[3, 100] = -0.0                                                 # -0 == +0: still index 0
+    x[4, 17], x[4, 2050] = float("inf"), float("inf")
+    x[5, 4999] = 1.0
+    got = ops.speculator_argmax(x.to(DEV), 5000).cpu()
+    assert got.tolist() == [0, 77, 0, 0, 17, 4999]
+    assert torch.equal(got, reference(x, 5000))
+
+
+def test_nan_beats_every_number_and_the_first_nan_wins(ops):
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(5, 9000, generator=g)
+    x[0, 8000] = float("nan")
+    x[1, 5], x[1, 8999] = float("nan"), float("nan")
+    x[2, 3000], x[2, 10] = float("nan"), float("inf")
+    x[3, 100], x[3, 101] = float("inf"), -float("inf")              # a chunk sum that is NaN without any NaN in it
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
+        xs = x.to(dtype)
+        got = ops.speculator_argmax(xs.to(DEV), 9000).cpu()
+        assert got[:4].tolist() == [8000, 5, 3000, 100]
+        assert torch.equal(got, reference(xs, 9000))
+
+
+def test_clamp_and_row_pitch(ops):
+    g = torch.Generator().manual_seed(7)
+    full = torch.randn(40, 1100, generator=g).to(torch.bfloat16).to(DEV)
+    for view in (full[:, :1000], full[:, 4:1003], full[::2, :999]):   # aligned pitch, odd start, skipped rows
+        got = ops.speculator_argmax(view, 1000)
+        assert torch.equal(got, torch.argmax(view.float(), dim=-1).clamp_(0, 999))
+    # logits wider than the vocabulary (padded head): indices beyond it are clamped
+    padded = torch.zeros(4, 1024, dtype=torch.float16, device=DEV)
+    padded[:, 1010] = 5.0
+    assert ops.speculator_argmax(padded, 1000).tolist() == [999] * 4
+
+
+def test_empty_and_errors(ops):
+    assert ops.speculator_argmax(torch.empty(0, 64, device=DEV), 64).shape == (0,)
+    with pytest.raises(RuntimeError, match="non-empty last dimension"):
+        ops.speculator_argmax(torch.empty(4, 0, device=DEV), 1)
+    with pytest.raises(RuntimeError, match="fp32, fp16 or bf16"):
+        ops.speculator_argmax(torch.zeros(4, 8, dtype=torch.float64, device=DEV), 8)
+    with pytest.raises(RuntimeError, match="last dimension must be contiguous"):
+        ops.speculator_argmax(torch.zeros(8, 4, device=DEV).t(), 8)

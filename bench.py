@@ -196,6 +196,28 @@ def cpu_baseline_bulk(w: BulkWorkload, target_seconds=10.0):
     }
 
 
+def cpu_baseline_speculator():
+    """The CPU oracle (C, OpenMP) on the speculator workload: sum_lstm and speculator_ln at 512 x 4096 bf16."""
+    import oracle
+    T, Hd = 512, 4096
+    g = torch.Generator().manual_seed(3)
+    rn = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16)
+    s4, z4, pc, x = rn(T, 4 * Hd), rn(T, 4 * Hd), rn(T, Hd), rn(T, Hd)
+    w, b = (1 + 0.02 * torch.randn(Hd, generator=g)).to(torch.bfloat16), (0.02 * torch.randn(Hd, generator=g)).to(torch.bfloat16)
+    out = {"cores": oracle.num_threads(), "kind": "port"}
+    for name, fn in (("sum_lstm", lambda: oracle.sum_lstm(s4, z4, pc, w, b, w, b, 23.07, 1e-6, 1e-6, False)),
+                     ("speculator_ln", lambda: oracle.speculator_ln(x, w, b, 1e-6))):
+        fn()
+        times = []
+        t_end = time.perf_counter() + 1.0
+        while time.perf_counter() < t_end or len(times) < 5:
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+        out[name + "_us_per_call"] = round(statistics.median(times) * 1e6, 1)
+    return out
+
+
 def load_floor_kernels():
     """bench_floor.so: bare kernels that move the same bytes as the library's and compute nothing
     (built by __graft_entry__.build()).  None when it has not been built."""
@@ -615,8 +637,8 @@ def placement_sweep(ops, dev, steps):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--weight-gib", type=int, default=66, help="resident-weights placeholder allocated before the KV pool")
     ap.add_argument("--pool-blocks", type=int, default=65536, help="blocks per layer of the 80-layer KV pool")
     ap.add_argument("--no-extras", action="store_true", help="skip the speculator / decode-mix measurements")
@@ -703,7 +725,9 @@ def main():
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "kernel": "kv_write_bulk_kernel<bf16, e4m3>", "kernel_us_mean": round(kernel_us, 2),
-                "kernel_us_median": round(statistics.median(us), 2), "algorithmic_bytes": w.bytes}
+                "kernel_us_median": round(statistics.median(us), 2),
+                "kernel_us_p10": round(sorted(us)[len(us) // 10], 2),
+                "kernel_us_p90": round(sorted(us)[(9 * len(us)) // 10], 2), "algorithmic_bytes": w.bytes}
     log(f"bulk fp8 70B shape: {ms_per_step:.3f} ms/step wall, kernel {kernel_us:.1f} us, {achieved:.0f} GB/s")
 
     cpu = None
@@ -751,6 +775,8 @@ def main():
         extras["fp4_write_8b_layer"] = bench_fp4(ops, dev, args.steps)
         torch.cuda.empty_cache()
         extras["speculator"] = bench_speculator(ops, dev, args.steps, args.warmup)
+        if not args.no_cpu:
+            extras["speculator"]["cpu_baseline"] = cpu_baseline_speculator()
         extras["decode_mix"] = bench_decode_mix(ops, dev, args.steps)
         extras["swiftkv_select_decode_70b"] = bench_row_gather(ops, dev, args.steps)
         extras["speculator_argmax_512x128256"] = bench_argmax(ops, dev, args.steps)

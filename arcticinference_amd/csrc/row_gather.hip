@@ -68,30 +68,32 @@ __device__ __forceinline__ void move_units(const char *src, char *dst, int64_t f
 
 template <typename Index>
 __global__ __launch_bounds__(kGatherThreads) void row_gather_kernel(GatherTable tab, const Index *__restrict__ indices,
-                                                                    int64_t num_indexed_rows, int scatter) {
-  const int64_t row = blockIdx.y;
-  const int64_t idx = (int64_t)indices[row];
-  if (idx < 0 || idx >= num_indexed_rows) return;   // uniform over the workgroup
-  const int64_t src_row = scatter ? row : idx;
-  const int64_t dst_row = scatter ? idx : row;
-
+                                                                    int64_t num_indices, int64_t num_indexed_rows,
+                                                                    int scatter) {
   // the 1024 units of this workgroup may straddle tensors; each tensor's share is moved in turn
   const int64_t begin = (int64_t)blockIdx.x * (kGatherThreads * kGatherUnroll);
   const int64_t end = begin + kGatherThreads * kGatherUnroll;
-  for (int t = 0; t < tab.count; ++t) {
-    const int64_t lo = std::max(begin, tab.first_unit[t]);
-    const int64_t hi = std::min(end, tab.first_unit[t + 1]);
-    if (lo >= hi) continue;
-    const char *src = tab.src[t] + src_row * tab.src_stride[t];
-    char *dst = tab.dst[t] + dst_row * tab.dst_stride[t];
-    const int64_t first = lo - tab.first_unit[t] + threadIdx.x;
-    const int64_t last = hi - tab.first_unit[t];
-    switch (tab.unit_shift[t]) {
-      case 4: move_units<16>(src, dst, first, last); break;
-      case 3: move_units<8>(src, dst, first, last); break;
-      case 2: move_units<4>(src, dst, first, last); break;
-      case 1: move_units<2>(src, dst, first, last); break;
-      default: move_units<1>(src, dst, first, last); break;
+  // the grid's second dimension holds at most 65535 rows; beyond that a workgroup takes several
+  for (int64_t row = blockIdx.y; row < num_indices; row += gridDim.y) {
+    const int64_t idx = (int64_t)indices[row];
+    if (idx < 0 || idx >= num_indexed_rows) continue;   // uniform over the workgroup
+    const int64_t src_row = scatter ? row : idx;
+    const int64_t dst_row = scatter ? idx : row;
+    for (int t = 0; t < tab.count; ++t) {
+      const int64_t lo = std::max(begin, tab.first_unit[t]);
+      const int64_t hi = std::min(end, tab.first_unit[t + 1]);
+      if (lo >= hi) continue;
+      const char *src = tab.src[t] + src_row * tab.src_stride[t];
+      char *dst = tab.dst[t] + dst_row * tab.dst_stride[t];
+      const int64_t first = lo - tab.first_unit[t] + threadIdx.x;
+      const int64_t last = hi - tab.first_unit[t];
+      switch (tab.unit_shift[t]) {
+        case 4: move_units<16>(src, dst, first, last); break;
+        case 3: move_units<8>(src, dst, first, last); break;
+        case 2: move_units<4>(src, dst, first, last); break;
+        case 1: move_units<2>(src, dst, first, last); break;
+        default: move_units<1>(src, dst, first, last); break;
+      }
     }
   }
 }
@@ -115,9 +117,7 @@ extern "C" int arctic_gather_rows(int num_tensors, const void *const *src, void 
                 num_tensors);
   if (index_bytes != 4 && index_bytes != 8)
     return fail(ARCTIC_ERR_UNSUPPORTED, "%s: indices must be int32 or int64", fn);
-  if (num_indices < 0 || num_indices > 65535)
-    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: between 0 and 65535 indices per call, got %lld", fn,
-                (long long)num_indices);
+  if (num_indices < 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: negative number of indices", fn);
   if (num_indexed_rows < 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: negative row count", fn);
   if (num_tensors == 0 || num_indices == 0) return ARCTIC_OK;
   if (!src || !dst || !row_bytes || !src_row_stride_bytes || !dst_row_stride_bytes || !indices)
@@ -150,13 +150,13 @@ extern "C" int arctic_gather_rows(int num_tensors, const void *const *src, void 
   const int64_t groups = (units + per_group - 1) / per_group;
   if (groups > 0x7fffffffLL) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: rows too long", fn);
 
-  const dim3 grid((unsigned)groups, (unsigned)num_indices);
+  const dim3 grid((unsigned)groups, (unsigned)std::min<int64_t>(num_indices, 65535));
   hipStream_t s = (hipStream_t)stream;
   if (index_bytes == 8)
     hipLaunchKernelGGL(row_gather_kernel<int64_t>, grid, dim3(kGatherThreads), 0, s, tab, (const int64_t *)indices,
-                       num_indexed_rows, scatter);
+                       num_indices, num_indexed_rows, scatter);
   else
     hipLaunchKernelGGL(row_gather_kernel<int32_t>, grid, dim3(kGatherThreads), 0, s, tab, (const int32_t *)indices,
-                       num_indexed_rows, scatter);
+                       num_indices, num_indexed_rows, scatter);
   return check_launch(fn);
 }

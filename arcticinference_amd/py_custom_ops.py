@@ -43,12 +43,6 @@ _SCHEMAS = {
         "sum_lstm_cuda(Tensor states_4d, Tensor z4_4d, Tensor prev_cell_d, Tensor? w_cell, "
         "Tensor? b_cell, Tensor? w_state, Tensor? b_state, float alpha, float eps_cell, "
         "float eps_state, bool use_fast_gelu) -> (Tensor, Tensor)",
-    "gather_rows": "gather_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
-    "scatter_rows": "scatter_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
-    "speculator_argmax_cuda": "speculator_argmax_cuda(Tensor logits, int max_index) -> Tensor",
-    "speculator_add_ln_act_cuda":
-        "speculator_add_ln_act_cuda(Tensor input, Tensor? z, Tensor? weight, Tensor? bias, float alpha, "
-        "float eps, str activation, float out_scale) -> Tensor",
 }
 
 # Operators that fuse a caller-side step into one of the above; the reference has no such schema.
@@ -57,11 +51,12 @@ _EXTRA_SCHEMAS = {
         "sum_lstm_shared_z_cuda(Tensor states_4d, Tensor z_d, Tensor prev_cell_d, Tensor? w_cell, "
         "Tensor? b_cell, Tensor? w_state, Tensor? b_state, float alpha, float eps_cell, "
         "float eps_state, bool use_fast_gelu) -> (Tensor, Tensor)",
-    "gather_rows": "gather_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
-    "scatter_rows": "scatter_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
     "speculator_add_ln_act_cuda":
         "speculator_add_ln_act_cuda(Tensor input, Tensor? z, Tensor? weight, Tensor? bias, float alpha, "
         "float eps, str activation, float out_scale) -> Tensor",
+    "speculator_argmax_cuda": "speculator_argmax_cuda(Tensor logits, int max_index) -> Tensor",
+    "gather_rows": "gather_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
+    "scatter_rows": "scatter_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
 }
 
 _SRC_DTYPES = {
@@ -494,6 +489,40 @@ _IMPLS = {
 }
 
 
+# Shape-only implementations for meta tensors (tracing under torch.compile): the same output shapes,
+# strides and dtypes as the launches above, no data.  The reference binds the CUDA key only
+# (torch_bindings.cpp:17,32,37,50), so its operators cannot be traced; these change nothing for real tensors.
+def _meta_like_input(input, *args):
+    return torch.empty_like(input)
+
+
+def _meta_sum_lstm(states_4d, z, prev_cell_d, *args):
+    p2 = prev_cell_d.view(-1, prev_cell_d.size(-1))
+    make = lambda: torch.empty_strided(p2.size(), p2.stride(), dtype=p2.dtype, device=p2.device).view(prev_cell_d.size())
+    return make(), make()
+
+
+def _meta_argmax(logits, max_index):
+    return torch.empty(logits.shape[:-1], dtype=torch.int64, device=logits.device)
+
+
+def _meta_nothing(*args):
+    return None
+
+
+_META_IMPLS = {
+    "speculator_ln_cuda": _meta_like_input,
+    "speculator_add_ln_act_cuda": _meta_like_input,
+    "sum_lstm_cuda": _meta_sum_lstm,
+    "sum_lstm_shared_z_cuda": _meta_sum_lstm,
+    "speculator_argmax_cuda": _meta_argmax,
+    "reshape_and_cache_flash_bulk": _meta_nothing,
+    "reshape_and_cache_flash_fp4": _meta_nothing,
+    "gather_rows": _meta_nothing,
+    "scatter_rows": _meta_nothing,
+}
+
+
 def _register_ops() -> None:
     """Define the four schemas and bind the CUDA key (the only key the reference
     binds, torch_bindings.cpp:17,32,37,50)."""
@@ -504,6 +533,7 @@ def _register_ops() -> None:
     for name, schema in {**_SCHEMAS, **_EXTRA_SCHEMAS}.items():
         lib.define(schema)
         lib.impl(name, _IMPLS[name], "CUDA")
+        lib.impl(name, _META_IMPLS[name], "Meta")
     _torch_lib = lib  # keep alive: dropping the Library object unregisters the ops
     _registered = True
 

@@ -243,7 +243,7 @@ int arctic_sum_lstm_shared_z(void *out_state, void *out_cell, const void *states
  *   row_bytes           HOST array: bytes per row of each tensor (0 skips the tensor)
  *   *_row_stride_bytes  HOST arrays: bytes between rows
  *   indices             device, num_indices entries of index_bytes (4 or 8) each, signed
- *   num_indices         at most 65535
+ *   num_indices         number of rows moved per tensor (any count; more than 65535 are walked by a loop in the kernel)
  *   num_indexed_rows    rows of the indexed side (sources of a gather, destinations of a scatter)
  */
 int arctic_gather_rows(int num_tensors, const void *const *src, void *const *dst,

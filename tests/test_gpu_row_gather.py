@@ -104,6 +104,22 @@ def test_scatter_back(ops):
     assert torch.equal(d.cpu().view(torch.int16), want.view(torch.int16))
 
 
+def test_more_indices_than_one_grid_dimension_holds(ops):
+    # 70000 indices: the grid's second dimension stops at 65535, the kernel walks the rest
+    g = torch.Generator().manual_seed(7)
+    tensors = [torch.randn(1000, 24, generator=g).to(torch.bfloat16), torch.randint(0, 1 << 30, (1000,), generator=g)]
+    idx = torch.randint(0, 1000, (70000,), generator=g)
+    idx[65535:65540] = torch.tensor([-1, 1000, 0, 999, 5])
+    check_gather(ops, tensors, idx, 70000)
+    perm = torch.randperm(70000, generator=g)
+    rows = torch.randn(70000, 6, generator=g)
+    want = torch.zeros(70000, 6)
+    want[perm] = rows
+    d = torch.zeros(70000, 6, device=DEV)
+    ops.scatter_rows([rows.to(DEV)], perm.to(DEV), [d])
+    assert torch.equal(d.cpu(), want)
+
+
 def test_empty_and_errors(ops):
     x = torch.randn(8, 64, device=DEV)
     empty = torch.empty(0, dtype=torch.int64, device=DEV)

@@ -53,6 +53,26 @@ def test_no_cpu_backend_and_no_fallback(loaded):
         ops.reshape_and_cache_flash_bulk(x, x, [x], [x], torch.zeros(4, dtype=torch.int64), "auto", [x], [x], 1, 64)
 
 
+def test_meta_tensors_trace_shapes_without_data(loaded):
+    # shape-only implementations: output shapes, strides and dtypes of the real launches
+    x = torch.empty(3, 5, 64, dtype=torch.bfloat16, device="meta")
+    y = ops.speculator_ln(x, None, None, 1e-6)
+    assert y.is_meta and y.shape == x.shape and y.dtype == x.dtype and y.is_contiguous()
+    y = ops.speculator_add_ln_gelu(x, x, None, None, 0.5, 1e-6)
+    assert y.is_meta and y.shape == x.shape
+    pc = torch.empty(7, 100, dtype=torch.float16, device="meta")[:, :64]     # pitched rows
+    s4 = torch.empty(7, 256, dtype=torch.float16, device="meta")
+    state, cell = ops.sum_lstm(s4, s4, pc, None, None, None, None, 1.0, 1e-6, 1e-6, False)
+    assert state.shape == cell.shape == (7, 64) and state.stride() == cell.stride() == (100, 1)
+    state, cell = ops.sum_lstm_shared_z(s4, pc, pc, None, None, None, None, 1.0, 1e-6, 1e-6, False)
+    assert state.shape == (7, 64) and state.dtype == torch.float16
+    logits = torch.empty(4, 2, 1000, device="meta")
+    t = ops.speculator_argmax(logits, 999)
+    assert t.is_meta and t.shape == (4, 2) and t.dtype == torch.int64
+    i = torch.empty(4, dtype=torch.int64, device="meta")
+    assert ops.reshape_and_cache_flash_bulk(x, x, [x], [x], i, "auto", [x], [x], 1, 64) is None
+
+
 def test_argument_checks_mirror_the_reference(loaded):
     # the shims run the reference's TORCH_CHECKs before touching the device, so the
     # ones that precede the device check can be exercised with CPU tensors

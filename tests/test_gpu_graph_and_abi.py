@@ -177,3 +177,40 @@ def test_side_stream(ops):
         y = ops.speculator_ln(dx, None, None, 1e-6)
     s.synchronize()
     assert_close(y, oracle.speculator_ln(x, None, None, 1e-6), what="ln on a side stream")
+
+
+@pytest.mark.parametrize("backend", ["eager", "aot_eager"])
+def test_operators_trace_under_torch_compile(ops, backend):
+    """Traced as opaque nodes (the Meta key gives the shapes), the operators compute what they compute eagerly,
+    the one that writes into its arguments included."""
+    g = torch.Generator().manual_seed(16)
+    rn = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(DEV)
+    x, w, s4, z4 = rn(64, 1024), rn(1024), rn(64, 4096), rn(64, 4096)
+
+    def step(x, s4, z4, w):
+        y = ops.speculator_ln(x, w, None, 1e-6)
+        state, cell = ops.sum_lstm(s4, z4, y, w, w, w, w, 0.5, 1e-6, 1e-6, False)
+        return state + 1, cell, ops.speculator_argmax(state.float(), 1000)
+
+    want = step(x, s4, z4, w)
+    got = torch.compile(step, backend=backend, fullgraph=True)(x, s4, z4, w)
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+
+    layers = 3
+    k, v = rn(16, layers * 128), rn(16, layers * 128)
+    slots = torch.randperm(64, generator=g)[:16].to(DEV)
+    scales = [torch.tensor([0.5], device=DEV) for _ in range(layers)]
+    caches = lambda: [torch.zeros(4, 16, 2, 64, dtype=torch.uint8, device=DEV) for _ in range(2 * layers)]
+
+    def write(k, v, kc, vc, slots, ks, vs):
+        ops.reshape_and_cache_flash_bulk(k, v, kc, vc, slots, "fp8", ks, vs, 2, 64)
+        return k * 2
+
+    eager, traced = caches(), caches()
+    write(k, v, eager[:layers], eager[layers:], slots, scales, scales)
+    out = torch.compile(write, backend=backend, fullgraph=True)(k, v, traced[:layers], traced[layers:], slots,
+                                                                scales, scales)
+    assert torch.equal(out, k * 2)
+    for a, b in zip(traced, eager):
+        assert torch.equal(a, b) and a.any()

@@ -10,12 +10,16 @@ from . import py_custom_ops  # noqa: F401
 from .py_custom_ops import (  # noqa: F401
     gather_rows,
     reshape_and_cache_flash_bulk,
+    reshape_and_cache_flash_fp4,
     scatter_rows,
     speculator_add_ln_gelu,
     speculator_argmax,
+    speculator_embed_add_ln_gelu,
     speculator_ln,
     speculator_ln_scaled,
     sum_lstm,
+    sum_lstm_embedded,
+    sum_lstm_shared_z,
     try_load_jit_library,
     try_load_torch_library,
 )

@@ -28,8 +28,10 @@ EXPORTED_SYMBOLS = (
     "arctic_reshape_and_cache_flash_fp4",
     "arctic_speculator_ln",
     "arctic_speculator_add_ln_act",
+    "arctic_speculator_embed_add_ln_act",
     "arctic_sum_lstm",
     "arctic_sum_lstm_shared_z",
+    "arctic_sum_lstm_embedded",
     "arctic_gather_rows",
     "arctic_argmax_clamp",
 )
@@ -89,6 +91,11 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.arctic_sum_lstm.restype = i32
     lib.arctic_sum_lstm_shared_z.argtypes = lib.arctic_sum_lstm.argtypes
     lib.arctic_sum_lstm_shared_z.restype = i32
+    lib.arctic_sum_lstm_embedded.argtypes = [vp] * 10 + [i64, i32, i64, i64, i64, i64, i64, f32, f32, f32, i32, i32, vp]
+    lib.arctic_sum_lstm_embedded.restype = i32
+    lib.arctic_speculator_embed_add_ln_act.argtypes = [vp, vp, vp, vp, vp, vp, i64, i32, i64, i64, i64, f32, f32, i32,
+                                                       f32, i32, vp]
+    lib.arctic_speculator_embed_add_ln_act.restype = i32
     lib.arctic_gather_rows.argtypes = [i32, vp, vp, vp, vp, vp, vp, i32, i64, i64, i32, vp]
     lib.arctic_gather_rows.restype = i32
     lib.arctic_argmax_clamp.argtypes = [vp, vp, i64, i32, i64, i64, i32, vp]

@@ -29,6 +29,8 @@ namespace arctic {
 struct LnGlue {
   const char *z;            // nullptr: no add
   int64_t z_row_stride_bytes;
+  const int64_t *z_index;   // row of z to add to each row (an embedding lookup); nullptr = the row itself
+  int64_t z_rows;           // rows of z when z_index is given; an index is clamped into [0, z_rows)
   float alpha;
   int activation;           // ARCTIC_ACT_*
   float out_scale;          // applied when != 1
@@ -71,7 +73,9 @@ __global__ __launch_bounds__(1024) void spec_ln_vec_kernel(
     if (c < chunks) raw[k] = load16_stream(row_in + (int64_t)c * 16);
   }
   if (kGlue && glue.z) {
-    const char *row_z = glue.z + (int64_t)blockIdx.x * glue.z_row_stride_bytes;
+    int64_t z_at = blockIdx.x;
+    if (glue.z_index) z_at = min(max(glue.z_index[blockIdx.x], (int64_t)0), glue.z_rows - 1);
+    const char *row_z = glue.z + z_at * glue.z_row_stride_bytes;
     uint4 zr[kChunksPerThread];
 #pragma unroll
     for (int k = 0; k < kChunksPerThread; ++k) {
@@ -135,8 +139,9 @@ __global__ __launch_bounds__(256) void spec_ln_scalar_kernel(
     LnGlue glue) {
   __shared__ float slots[16];
   const uint16_t *row_in = in + (int64_t)blockIdx.x * in_row_stride;
-  const uint16_t *row_z =
-      glue.z ? (const uint16_t *)(glue.z + (int64_t)blockIdx.x * glue.z_row_stride_bytes) : nullptr;
+  int64_t z_at = blockIdx.x;
+  if (glue.z && glue.z_index) z_at = min(max(glue.z_index[blockIdx.x], (int64_t)0), glue.z_rows - 1);
+  const uint16_t *row_z = glue.z ? (const uint16_t *)(glue.z + z_at * glue.z_row_stride_bytes) : nullptr;
   uint16_t *row_out = out + (int64_t)blockIdx.x * hidden;
   auto element = [&](int j) {
     float x = T::lo(row_in[j]);
@@ -167,7 +172,7 @@ static void launch_ln(void *out, const void *in, const void *w, const void *b, i
   const float inv_hidden = 1.0f / (float)hidden;
   const bool vec = (hidden % 8 == 0) && (in_row_stride % 8 == 0 || rows == 1) && aligned16(in) &&
                    aligned16(out) && (!w || aligned16(w)) && (!b || aligned16(b)) && chunks <= 8 * 1024 &&
-                   (!glue.z || (aligned16(glue.z) && (glue.z_row_stride_bytes % 16 == 0 || rows == 1)));
+                   (!glue.z || (aligned16(glue.z) && (glue.z_row_stride_bytes % 16 == 0 || (rows == 1 && !glue.z_index))));
   const bool plain = !glue.z && glue.activation == ARCTIC_ACT_NONE && glue.out_scale == 1.0f;
   const dim3 grid((unsigned)rows);
   if (vec) {
@@ -228,7 +233,7 @@ static int ln_entry(const char *fn, void *out, const void *in, const void *weigh
 extern "C" int arctic_speculator_ln(void *out, const void *in, const void *weight, const void *bias,
                                     int64_t rows, int hidden, int64_t in_row_stride, float eps, int dtype,
                                     void *stream) {
-  const LnGlue none = {nullptr, 0, 0.0f, ARCTIC_ACT_NONE, 1.0f};
+  const LnGlue none = {nullptr, 0, nullptr, 0, 0.0f, ARCTIC_ACT_NONE, 1.0f};
   return ln_entry("speculator_ln", out, in, weight, bias, rows, hidden, in_row_stride, eps, none, dtype, stream);
 }
 
@@ -236,7 +241,19 @@ extern "C" int arctic_speculator_add_ln_act(void *out, const void *in, const voi
                                             const void *bias, int64_t rows, int hidden, int64_t in_row_stride,
                                             int64_t z_row_stride, float alpha, float eps, int activation,
                                             float out_scale, int dtype, void *stream) {
-  const LnGlue glue = {(const char *)z, z_row_stride * 2, alpha, activation, out_scale};
+  const LnGlue glue = {(const char *)z, z_row_stride * 2, nullptr, 0, alpha, activation, out_scale};
   return ln_entry("speculator_add_ln_act", out, in, weight, bias, rows, hidden, in_row_stride, eps, glue, dtype,
                   stream);
+}
+
+extern "C" int arctic_speculator_embed_add_ln_act(void *out, const void *in, const void *emb_table,
+                                                  const int64_t *token_ids, const void *weight, const void *bias,
+                                                  int64_t rows, int hidden, int64_t in_row_stride, int64_t emb_row_stride,
+                                                  int64_t num_embeddings, float alpha, float eps, int activation,
+                                                  float out_scale, int dtype, void *stream) {
+  const char *fn = "speculator_embed_add_ln_act";
+  if (rows > 0 && (!emb_table || !token_ids)) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null embedding table or token ids", fn);
+  if (rows > 0 && num_embeddings <= 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: the embedding table has no rows", fn);
+  const LnGlue glue = {(const char *)emb_table, emb_row_stride * 2, token_ids, num_embeddings, alpha, activation, out_scale};
+  return ln_entry(fn, out, in, weight, bias, rows, hidden, in_row_stride, eps, glue, dtype, stream);
 }

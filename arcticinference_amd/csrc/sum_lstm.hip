@@ -30,6 +30,8 @@ struct LstmParams {
   const char *b_cell;
   const char *w_state;
   const char *b_state;
+  const int64_t *z_index;  // shared-z only: row of z4 to use for each row (an embedding lookup); nullptr = the row itself
+  int64_t z_rows;          // rows of z4 when z_index is given; an index is clamped into [0, z_rows)
   int64_t s_stride;   // all strides in elements
   int64_t z_stride;
   int64_t pc_stride;
@@ -61,7 +63,9 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
   const int64_t row = blockIdx.x;
   const int64_t gate_bytes = (int64_t)D * 2;
   const char *s_row = p.states + row * p.s_stride * 2;
-  const char *z_row = p.z4 + row * p.z_stride * 2;
+  int64_t zr = row;
+  if (kSharedZ && p.z_index) zr = min(max(p.z_index[row], (int64_t)0), p.z_rows - 1);
+  const char *z_row = p.z4 + zr * p.z_stride * 2;
   const char *pc_row = p.prev_cell + row * p.pc_stride * 2;
   char *oc_row = p.out_cell + row * p.out_stride * 2;
   char *os_row = p.out_state + row * p.out_stride * 2;
@@ -211,7 +215,9 @@ __global__ __launch_bounds__(256) void sum_lstm_scalar_kernel(const LstmParams p
   const int D = p.D;
   const int64_t row = blockIdx.x;
   const uint16_t *s = (const uint16_t *)p.states + row * p.s_stride;
-  const uint16_t *z = (const uint16_t *)p.z4 + row * p.z_stride;
+  int64_t zr = row;
+  if (p.z_index) zr = min(max(p.z_index[row], (int64_t)0), p.z_rows - 1);
+  const uint16_t *z = (const uint16_t *)p.z4 + zr * p.z_stride;
   const uint16_t *pc = (const uint16_t *)p.prev_cell + row * p.pc_stride;
   uint16_t *oc = (uint16_t *)p.out_cell + row * p.out_stride;
   uint16_t *os = (uint16_t *)p.out_state + row * p.out_stride;
@@ -258,6 +264,7 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
   const bool vec = (p.D % 8 == 0) && chunks <= 2 * 1024 &&
                    (!multi || (p.s_stride % 8 == 0 && p.z_stride % 8 == 0 && p.pc_stride % 8 == 0 &&
                                p.out_stride % 8 == 0)) &&
+                   (!p.z_index || p.z_stride % 8 == 0) &&
                    aligned16(p.states) && aligned16(p.z4) && aligned16(p.prev_cell) &&
                    aligned16(p.out_state) && aligned16(p.out_cell) && aligned16(p.w_cell) &&
                    aligned16(p.b_cell) && aligned16(p.w_state) && aligned16(p.b_state);
@@ -283,7 +290,7 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
 using namespace arctic;
 
 static int sum_lstm_entry(const char *fn, bool shared_z, void *out_state, void *out_cell, const void *states,
-                          const void *z, const void *prev_cell, const void *w_cell, const void *b_cell,
+                          const void *z, const int64_t *z_index, int64_t z_rows, const void *prev_cell, const void *w_cell, const void *b_cell,
                           const void *w_state, const void *b_state, int64_t rows, int D, int64_t s_stride,
                           int64_t z_stride, int64_t pc_stride, int64_t out_stride, float alpha, float eps_cell,
                           float eps_state, int fast_gelu, int dtype, void *stream) {
@@ -294,7 +301,10 @@ static int sum_lstm_entry(const char *fn, bool shared_z, void *out_state, void *
   if (rows == 0) return ARCTIC_OK;
   if (!out_state || !out_cell || !states || !z || !prev_cell)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
+  if (z_index && z_rows <= 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: the embedding table has no rows", fn);
   LstmParams p;
+  p.z_index = z_index;
+  p.z_rows = z_rows;
   p.out_state = (char *)out_state;
   p.out_cell = (char *)out_cell;
   p.states = (const char *)states;
@@ -336,7 +346,7 @@ extern "C" int arctic_sum_lstm(void *out_state, void *out_cell, const void *stat
                                int64_t s_stride, int64_t z_stride, int64_t pc_stride, int64_t out_stride,
                                float alpha, float eps_cell, float eps_state, int fast_gelu, int dtype,
                                void *stream) {
-  return sum_lstm_entry("sum_lstm", false, out_state, out_cell, states, z4, prev_cell, w_cell, b_cell, w_state,
+  return sum_lstm_entry("sum_lstm", false, out_state, out_cell, states, z4, nullptr, 0, prev_cell, w_cell, b_cell, w_state,
                         b_state, rows, D, s_stride, z_stride, pc_stride, out_stride, alpha, eps_cell, eps_state,
                         fast_gelu, dtype, stream);
 }
@@ -347,7 +357,20 @@ extern "C" int arctic_sum_lstm_shared_z(void *out_state, void *out_cell, const v
                                         int64_t s_stride, int64_t z_stride, int64_t pc_stride,
                                         int64_t out_stride, float alpha, float eps_cell, float eps_state,
                                         int fast_gelu, int dtype, void *stream) {
-  return sum_lstm_entry("sum_lstm_shared_z", true, out_state, out_cell, states, z, prev_cell, w_cell, b_cell,
+  return sum_lstm_entry("sum_lstm_shared_z", true, out_state, out_cell, states, z, nullptr, 0, prev_cell, w_cell, b_cell,
                         w_state, b_state, rows, D, s_stride, z_stride, pc_stride, out_stride, alpha, eps_cell,
+                        eps_state, fast_gelu, dtype, stream);
+}
+
+extern "C" int arctic_sum_lstm_embedded(void *out_state, void *out_cell, const void *states, const void *emb_table,
+                                        const int64_t *token_ids, const void *prev_cell, const void *w_cell,
+                                        const void *b_cell, const void *w_state, const void *b_state, int64_t rows,
+                                        int D, int64_t s_stride, int64_t emb_stride, int64_t pc_stride,
+                                        int64_t out_stride, int64_t num_embeddings, float alpha, float eps_cell,
+                                        float eps_state, int fast_gelu, int dtype, void *stream) {
+  const char *fn = "sum_lstm_embedded";
+  if (rows > 0 && !token_ids) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null token ids", fn);
+  return sum_lstm_entry(fn, true, out_state, out_cell, states, emb_table, token_ids, num_embeddings, prev_cell, w_cell,
+                        b_cell, w_state, b_state, rows, D, s_stride, emb_stride, pc_stride, out_stride, alpha, eps_cell,
                         eps_state, fast_gelu, dtype, stream);
 }

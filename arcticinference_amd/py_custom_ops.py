@@ -54,6 +54,13 @@ _EXTRA_SCHEMAS = {
     "speculator_add_ln_act_cuda":
         "speculator_add_ln_act_cuda(Tensor input, Tensor? z, Tensor? weight, Tensor? bias, float alpha, "
         "float eps, str activation, float out_scale) -> Tensor",
+    "sum_lstm_embedded_cuda":
+        "sum_lstm_embedded_cuda(Tensor states_4d, Tensor emb_weight, Tensor token_ids, Tensor prev_cell_d, "
+        "Tensor? w_cell, Tensor? b_cell, Tensor? w_state, Tensor? b_state, float alpha, float eps_cell, "
+        "float eps_state, bool use_fast_gelu) -> (Tensor, Tensor)",
+    "speculator_embed_add_ln_act_cuda":
+        "speculator_embed_add_ln_act_cuda(Tensor input, Tensor emb_weight, Tensor token_ids, Tensor? weight, "
+        "Tensor? bias, float alpha, float eps, str activation, float out_scale) -> Tensor",
     "speculator_argmax_cuda": "speculator_argmax_cuda(Tensor logits, int max_index) -> Tensor",
     "gather_rows": "gather_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
     "scatter_rows": "scatter_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
@@ -258,9 +265,23 @@ def _reshape_and_cache_flash_fp4_impl(
 _ACTIVATIONS = {"none": 0, "gelu": 1, "gelu_tanh": 2}
 
 
+def _check_embedding(fn: str, emb_weight: torch.Tensor, token_ids: torch.Tensor, like: torch.Tensor, width: int,
+                     rows: int) -> None:
+    """An embedding table [V, width] in the activations' type and one int64 token id per row."""
+    _check(emb_weight.is_cuda and token_ids.is_cuda and emb_weight.device == like.device
+           and token_ids.device == like.device, f"{fn}: embedding table and token ids must be on the input's device")
+    _check(emb_weight.dtype == like.dtype, f"{fn}: embedding table dtype must match input dtype")
+    _check(emb_weight.dim() == 2 and emb_weight.size(1) == width and emb_weight.stride(1) == 1,
+           f"{fn}: embedding table must be [num_embeddings, {width}] with contiguous rows")
+    _check(emb_weight.size(0) > 0, f"{fn}: the embedding table has no rows")
+    _check(token_ids.dtype == torch.int64, f"{fn}: token ids must be int64")
+    _check(token_ids.numel() == rows and token_ids.is_contiguous(),
+           f"{fn}: one contiguous token id per row is needed ({token_ids.numel()} ids, {rows} rows)")
+
+
 def _ln_common(fn: str, input: torch.Tensor, z: Optional[torch.Tensor], weight: Optional[torch.Tensor],
                bias: Optional[torch.Tensor], alpha: float, eps: float, activation: str,
-               out_scale: float) -> torch.Tensor:
+               out_scale: float, token_ids: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Argument checks and launch shared by speculator_ln_cuda and speculator_add_ln_act_cuda
     (the checks are those of csrc/custom_ops/speculator_ln.cu:152-201)."""
     lib = _lib()
@@ -287,7 +308,9 @@ def _ln_common(fn: str, input: torch.Tensor, z: Optional[torch.Tensor], weight: 
     rows = in_2d.size(0)
     row_stride = in_2d.stride(0)
     z_2d = None
-    if z is not None:
+    if token_ids is not None:
+        _check_embedding(fn, z, token_ids, input, hidden, rows)
+    elif z is not None:
         _check(z.is_cuda and z.device == input.device, "z must be CUDA, on the input's device")
         _check(z.dtype == dtype, "z dtype must match input dtype")
         _check(z.shape == input.shape, "z must have the input's shape")
@@ -301,7 +324,12 @@ def _ln_common(fn: str, input: torch.Tensor, z: Optional[torch.Tensor], weight: 
     w_ptr = weight.data_ptr() if weight is not None else None
     b_ptr = bias.data_ptr() if bias is not None else None
     with _on_device_of(input):
-        if z is None and activation == "none" and out_scale == 1.0:
+        if token_ids is not None:
+            rc = lib.arctic_speculator_embed_add_ln_act(
+                out_2d.data_ptr(), in_2d.data_ptr(), z.data_ptr(), token_ids.data_ptr(), w_ptr, b_ptr, rows, hidden,
+                row_stride, z.stride(0), z.size(0), float(alpha), float(eps), _ACTIVATIONS[activation],
+                float(out_scale), _HALF_DTYPES[dtype], _stream_of(input))
+        elif z is None and activation == "none" and out_scale == 1.0:
             rc = lib.arctic_speculator_ln(out_2d.data_ptr(), in_2d.data_ptr(), w_ptr, b_ptr, rows, hidden,
                                           row_stride, float(eps), _HALF_DTYPES[dtype], _stream_of(input))
         else:
@@ -327,6 +355,15 @@ def _speculator_add_ln_act_impl(input: torch.Tensor, z: Optional[torch.Tensor], 
     return _ln_common("speculator_add_ln_act", input, z, weight, bias, alpha, eps, activation, out_scale)
 
 
+def _speculator_embed_add_ln_act_impl(input: torch.Tensor, emb_weight: torch.Tensor, token_ids: torch.Tensor,
+                                      weight: Optional[torch.Tensor], bias: Optional[torch.Tensor], alpha: float,
+                                      eps: float, activation: str, out_scale: float) -> torch.Tensor:
+    """speculator_add_ln_act with z = emb_weight[clamp(token_ids)] looked up inside the launch
+    (arctic_inference/vllm/spec_dec/arctic_speculator.py:301-309, 845, 862)."""
+    return _ln_common("speculator_embed_add_ln_act", input, emb_weight, weight, bias, alpha, eps, activation,
+                      out_scale, token_ids=token_ids)
+
+
 def _sum_lstm_impl(
     states_4d: torch.Tensor,
     z4_4d: torch.Tensor,
@@ -340,6 +377,7 @@ def _sum_lstm_impl(
     eps_state: float,
     use_fast_gelu: bool,
     _shared_z: bool = False,
+    _token_ids: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """Host side of sum_lstm_cuda (csrc/custom_ops/sum_lstm.cu:293-473).  With _shared_z the
     second argument is the un-repeated [..., D] embedding row (see sum_lstm_shared_z)."""
@@ -373,7 +411,11 @@ def _sum_lstm_impl(
     z2 = z4_4d.view(-1, d_gate if _shared_z else hidden4)
     p2 = prev_cell_d.view(-1, d_cell)
     rows = s2.size(0)
-    _check(z2.size(0) == rows and p2.size(0) == rows, "sum_lstm: row counts of the inputs differ")
+    if _token_ids is not None:
+        _check(p2.size(0) == rows, "sum_lstm: row counts of the inputs differ")
+        _check_embedding("sum_lstm_embedded", z4_4d, _token_ids, states_4d, d_gate, rows)
+    else:
+        _check(z2.size(0) == rows and p2.size(0) == rows, "sum_lstm: row counts of the inputs differ")
     # outputs inherit prev_cell's row pitch (reference :356-365)
     out_cell = torch.empty_strided(p2.size(), p2.stride(), dtype=dtype, device=p2.device)
     out_state = torch.empty_strided(p2.size(), p2.stride(), dtype=dtype, device=p2.device)
@@ -388,12 +430,20 @@ def _sum_lstm_impl(
 
     entry = lib.arctic_sum_lstm_shared_z if _shared_z else lib.arctic_sum_lstm
     with _on_device_of(states_4d):
-        rc = entry(
-            out_state.data_ptr(), out_cell.data_ptr(), s2.data_ptr(), z2.data_ptr(), p2.data_ptr(),
-            ptr(w_cell), ptr(b_cell), ptr(w_state), ptr(b_state),
-            rows, d_gate, s2.stride(0), z2.stride(0), p2.stride(0), out_cell.stride(0),
-            float(alpha), float(eps_cell), float(eps_state), int(bool(use_fast_gelu)),
-            _HALF_DTYPES[dtype], _stream_of(states_4d))
+        if _token_ids is not None:
+            rc = lib.arctic_sum_lstm_embedded(
+                out_state.data_ptr(), out_cell.data_ptr(), s2.data_ptr(), z4_4d.data_ptr(), _token_ids.data_ptr(),
+                p2.data_ptr(), ptr(w_cell), ptr(b_cell), ptr(w_state), ptr(b_state),
+                rows, d_gate, s2.stride(0), z4_4d.stride(0), p2.stride(0), out_cell.stride(0), z4_4d.size(0),
+                float(alpha), float(eps_cell), float(eps_state), int(bool(use_fast_gelu)),
+                _HALF_DTYPES[dtype], _stream_of(states_4d))
+        else:
+            rc = entry(
+                out_state.data_ptr(), out_cell.data_ptr(), s2.data_ptr(), z2.data_ptr(), p2.data_ptr(),
+                ptr(w_cell), ptr(b_cell), ptr(w_state), ptr(b_state),
+                rows, d_gate, s2.stride(0), z2.stride(0), p2.stride(0), out_cell.stride(0),
+                float(alpha), float(eps_cell), float(eps_state), int(bool(use_fast_gelu)),
+                _HALF_DTYPES[dtype], _stream_of(states_4d))
     _native.check(rc)
     return out_state_orig, out_cell_orig
 
@@ -402,6 +452,14 @@ def _sum_lstm_shared_z_impl(states_4d, z_d, prev_cell_d, w_cell, b_cell, w_state
                             eps_state, use_fast_gelu):
     return _sum_lstm_impl(states_4d, z_d, prev_cell_d, w_cell, b_cell, w_state, b_state, alpha, eps_cell,
                           eps_state, use_fast_gelu, _shared_z=True)
+
+
+def _sum_lstm_embedded_impl(states_4d, emb_weight, token_ids, prev_cell_d, w_cell, b_cell, w_state, b_state, alpha,
+                            eps_cell, eps_state, use_fast_gelu):
+    """sum_lstm_shared_z with z = emb_weight[clamp(token_ids)] looked up inside the launch
+    (arctic_inference/vllm/spec_dec/arctic_speculator.py:744, 845, 862)."""
+    return _sum_lstm_impl(states_4d, emb_weight, prev_cell_d, w_cell, b_cell, w_state, b_state, alpha, eps_cell,
+                          eps_state, use_fast_gelu, _shared_z=True, _token_ids=token_ids)
 
 
 def _move_rows_impl(fn: str, sources: List[torch.Tensor], indices: torch.Tensor, outs: List[torch.Tensor],
@@ -481,7 +539,9 @@ _IMPLS = {
     "gather_rows": _gather_rows_impl,
     "scatter_rows": _scatter_rows_impl,
     "sum_lstm_shared_z_cuda": _sum_lstm_shared_z_impl,
+    "sum_lstm_embedded_cuda": _sum_lstm_embedded_impl,
     "speculator_add_ln_act_cuda": _speculator_add_ln_act_impl,
+    "speculator_embed_add_ln_act_cuda": _speculator_embed_add_ln_act_impl,
     "reshape_and_cache_flash_bulk": _reshape_and_cache_flash_bulk_impl,
     "reshape_and_cache_flash_fp4": _reshape_and_cache_flash_fp4_impl,
     "speculator_ln_cuda": _speculator_ln_impl,
@@ -494,6 +554,10 @@ _IMPLS = {
 # (torch_bindings.cpp:17,32,37,50), so its operators cannot be traced; these change nothing for real tensors.
 def _meta_like_input(input, *args):
     return torch.empty_like(input)
+
+
+def _meta_sum_lstm_embedded(states_4d, emb_weight, token_ids, prev_cell_d, *args):
+    return _meta_sum_lstm(states_4d, emb_weight, prev_cell_d)
 
 
 def _meta_sum_lstm(states_4d, z, prev_cell_d, *args):
@@ -515,6 +579,8 @@ _META_IMPLS = {
     "speculator_add_ln_act_cuda": _meta_like_input,
     "sum_lstm_cuda": _meta_sum_lstm,
     "sum_lstm_shared_z_cuda": _meta_sum_lstm,
+    "sum_lstm_embedded_cuda": _meta_sum_lstm_embedded,
+    "speculator_embed_add_ln_act_cuda": _meta_like_input,
     "speculator_argmax_cuda": _meta_argmax,
     "reshape_and_cache_flash_bulk": _meta_nothing,
     "reshape_and_cache_flash_fp4": _meta_nothing,
@@ -672,6 +738,44 @@ def sum_lstm_shared_z(
     Bit-identical to the two-step form; reads 6*D fewer bytes per row."""
     return _call("sum_lstm_shared_z_cuda", states_4d, z_d, prev_cell_d, w_cell, b_cell, w_state, b_state,
                                          alpha, eps_cell, eps_state, use_fast_gelu)
+
+
+def sum_lstm_embedded(
+    states_4d: torch.Tensor,
+    emb_weight: torch.Tensor,
+    token_ids: torch.Tensor,
+    prev_cell_d: torch.Tensor,
+    w_cell: Optional[torch.Tensor],
+    b_cell: Optional[torch.Tensor],
+    w_state: Optional[torch.Tensor],
+    b_state: Optional[torch.Tensor],
+    alpha: float,
+    eps_cell: float,
+    eps_state: float,
+    use_fast_gelu: bool,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``sum_lstm_shared_z(states_4d, emb_weight[token_ids.clamp(0, V - 1)], ...)`` without the lookup as a
+    launch of its own: the speculator's ``forget_emb[i](last_tokens)`` with the clamp of ``last_tokens``
+    (arctic_inference/vllm/spec_dec/arctic_speculator.py:744, 845, 862) folded into the operator.
+    Bit-identical to the two-step form."""
+    return _call("sum_lstm_embedded_cuda", states_4d, emb_weight, token_ids, prev_cell_d, w_cell, b_cell, w_state,
+                 b_state, alpha, eps_cell, eps_state, use_fast_gelu)
+
+
+def speculator_embed_add_ln_gelu(
+    states: torch.Tensor,
+    emb_weight: torch.Tensor,
+    token_ids: torch.Tensor,
+    weight: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor],
+    alpha: float,
+    eps: float,
+) -> torch.Tensor:
+    """``speculator_add_ln_gelu(states, emb_weight[token_ids.clamp(0, V - 1)], ...)`` in one launch: the MLP
+    speculator's ``z = emb[i](last_tokens); states.add_(z, alpha=...); activation(ln(states))``
+    (arctic_inference/vllm/spec_dec/arctic_speculator.py:301-309).  ``states`` is left unchanged."""
+    return _call("speculator_embed_add_ln_act_cuda", states, emb_weight, token_ids, weight, bias, alpha, eps, "gelu",
+                 1.0)
 
 
 def speculator_add_ln_gelu(

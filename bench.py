@@ -261,6 +261,24 @@ def bench_speculator(ops, dev, steps, warmup):
             _, cell = ops.sum_lstm_shared_z(S[i % sets][k], Z[i % sets][k][:, :Hd], cell, w_cell, b_cell, w_state,
                                             b_state, alpha, 1e-6, 1e-6, False)
 
+    # the embedding lookup in front of every step: forget_emb(last_tokens) of a 32000 x 4096 table
+    table = rn(32000, Hd)
+    IDS = [torch.randint(0, 32000, (T, 1), generator=g, device=dev) for _ in range(sets)]
+
+    def lstm3_lookup_repeat(i):
+        # as the reference's caller runs it: lookup, repeat(1, 1, 4), sum_lstm
+        cell = C0[i % sets]
+        for k in range(3):
+            z4 = torch.nn.functional.embedding(IDS[(i + k) % sets], table).repeat(1, 1, 4)
+            _, cell = ops.sum_lstm(S[i % sets][k], z4.flatten(0, 1), cell, w_cell, b_cell, w_state, b_state,
+                                   alpha, 1e-6, 1e-6, False)
+
+    def lstm3_embedded(i):
+        cell = C0[i % sets]
+        for k in range(3):
+            _, cell = ops.sum_lstm_embedded(S[i % sets][k], table, IDS[(i + k) % sets], cell, w_cell, b_cell, w_state,
+                                            b_state, alpha, 1e-6, 1e-6, False)
+
     def ln(i):
         ops.speculator_ln(X[i % sets], w_cell, b_cell, 1e-6)
 
@@ -285,6 +303,8 @@ def bench_speculator(ops, dev, steps, warmup):
 
     cases = [("sum_lstm", lstm3, 22 * Hd * T, 3),
              ("sum_lstm_shared_z", lstm3_shared_z, 16 * Hd * T, 3),
+             ("lookup_repeat_sum_lstm_as_three_ops", lstm3_lookup_repeat, 16 * Hd * T, 3),
+             ("sum_lstm_embedded", lstm3_embedded, 16 * Hd * T, 3),
              ("speculator_ln", ln, 4 * Hd * T, 1),
              ("speculator_add_ln_gelu", add_ln_gelu, 6 * Hd * T, 1),
              ("add_ln_gelu_as_three_ops", add_ln_gelu_separate, 6 * Hd * T, 1)]

@@ -176,6 +176,24 @@ int arctic_speculator_add_ln_act(void *out, const void *in, const void *z,
                                  void *stream);
 
 /*
+ * arctic_speculator_add_ln_act with z looked up in an embedding table: row r adds
+ * emb_table[clamp(token_ids[r], 0, num_embeddings - 1)], which is
+ *   z = self.emb[i](last_tokens); states.add_(z, alpha=...); activation(ln(states))
+ *        arctic_inference/vllm/spec_dec/arctic_speculator.py:301-309
+ * with the clamp the caller applies to last_tokens (:845, :862) in the same launch, and no z tensor.
+ *
+ *   emb_table    device; num_embeddings rows of `hidden` elements, emb_row_stride ELEMENTS apart
+ *   token_ids    device, int64 [rows]
+ */
+int arctic_speculator_embed_add_ln_act(void *out, const void *in, const void *emb_table,
+                                       const int64_t *token_ids, const void *weight,
+                                       const void *bias, int64_t rows, int hidden,
+                                       int64_t in_row_stride, int64_t emb_row_stride,
+                                       int64_t num_embeddings, float alpha, float eps,
+                                       int activation, float out_scale, int dtype,
+                                       void *stream);
+
+/*
  * Fused LSTM-style gate / cell / state update.  Replaces
  *   sum_lstm_cuda()                           csrc/custom_ops/sum_lstm.cu:293-473
  *   sum_lstm_vec_kernel<> / sum_lstm_scalar_kernel<>   csrc/custom_ops/sum_lstm.cu:28-291
@@ -222,6 +240,25 @@ int arctic_sum_lstm_shared_z(void *out_state, void *out_cell, const void *states
                              int64_t z_stride, int64_t pc_stride, int64_t out_stride,
                              float alpha, float eps_cell, float eps_state, int fast_gelu,
                              int dtype, void *stream);
+
+/*
+ * arctic_sum_lstm_shared_z with the embedding lookup folded in: row r uses
+ * emb_table[clamp(token_ids[r], 0, num_embeddings - 1)] as its z, which is
+ *   z4 = self.forget_emb[i](last_tokens).repeat(1, 1, 4)
+ *        arctic_inference/vllm/spec_dec/arctic_speculator.py:744
+ * and the clamp of last_tokens (:845, :862) inside the operator: no z and no z4 tensor, one launch less.
+ *
+ *   emb_table    device; num_embeddings rows of D elements, emb_stride ELEMENTS apart
+ *   token_ids    device, int64 [rows]
+ */
+int arctic_sum_lstm_embedded(void *out_state, void *out_cell, const void *states,
+                             const void *emb_table, const int64_t *token_ids,
+                             const void *prev_cell, const void *w_cell, const void *b_cell,
+                             const void *w_state, const void *b_state, int64_t rows, int D,
+                             int64_t s_stride, int64_t emb_stride, int64_t pc_stride,
+                             int64_t out_stride, int64_t num_embeddings, float alpha,
+                             float eps_cell, float eps_state, int fast_gelu, int dtype,
+                             void *stream);
 
 /*
  * Row gather / scatter over up to 8 tensors in one launch.  No native function of

@@ -132,6 +132,33 @@ def test_add_ln_gelu_against_the_three_separate_gpu_ops(ops):
     assert same_fraction(fused, separate) > 0.99
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,hidden,vocab,table_pad", [(512, 4096, 32000, 0), (33, 1024, 50, 8), (5, 260, 7, 3),
+                                                         (1, 12288, 2, 0)])
+def test_embed_add_ln_gelu_equals_lookup_then_add_ln_gelu(ops, dtype, rows, hidden, vocab, table_pad):
+    """z = emb(last_tokens) looked up inside the launch (arctic_speculator.py:301-309) with the caller's
+    clamp of last_tokens (:845, :862): the very bits of the lookup followed by speculator_add_ln_gelu."""
+    x, _, w, b = glue_inputs(rows, hidden, dtype, 31)
+    g = torch.Generator().manual_seed(32)
+    table = torch.randn(vocab, hidden + table_pad, generator=g).to(dtype)[:, :hidden]
+    ids = torch.randint(0, vocab, (rows,), generator=g)
+    ids[0] = -1
+    ids[-1] = vocab
+    z = torch.nn.functional.embedding(ids.clamp(0, vocab - 1), table)
+    alpha = 2.3716
+    xd, wd, bd = x.to(DEV), w.to(DEV), b.to(DEV)
+    dtable = to_device_pitched(table, DEV)
+    fused = ops.speculator_embed_add_ln_gelu(xd, dtable, ids.to(DEV), wd, bd, alpha, 1e-6)
+    two_step = ops.speculator_add_ln_gelu(xd, z.to(DEV), wd, bd, alpha, 1e-6)
+    assert torch.equal(fused, two_step)
+    assert_close(fused, oracle.speculator_add_ln_act(x, z, w, b, alpha, 1e-6, "gelu", 1.0), RTOL, ATOL, "embedded z")
+    with pytest.raises(RuntimeError, match="one contiguous token id per row"):
+        ops.speculator_embed_add_ln_gelu(xd, dtable, ids.to(DEV)[: rows - 1] if rows > 1 else ids.to(DEV).repeat(2),
+                                         wd, bd, alpha, 1e-6)
+    with pytest.raises(RuntimeError, match="embedding table must be"):
+        ops.speculator_embed_add_ln_gelu(xd, dtable[:, : hidden - 4], ids.to(DEV), wd, bd, alpha, 1e-6)
+
+
 @pytest.mark.parametrize("affine", [False, True])
 def test_ln_scaled_is_ln_then_scale(ops, affine):
     # ln0(x) / SQRT2 of the speculator (arctic_speculator.py:296-297): no affine terms there

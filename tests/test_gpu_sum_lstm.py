@@ -94,6 +94,59 @@ def test_shared_z_equals_repeated_z(ops, cfg, dtype):
     assert_close(st_s, want_s, RTOL, ATOL, "state (shared z)")
 
 
+@pytest.mark.parametrize("cfg", [dict(rows=512, D=4096, pad4=0, padD=0, vocab=32000, table_pad=0),
+                                 dict(rows=33, D=512, pad4=16, padD=8, vocab=100, table_pad=8),
+                                 dict(rows=5, D=100, pad4=0, padD=0, vocab=7, table_pad=3),     # element-wise kernel
+                                 dict(rows=1, D=8200, pad4=0, padD=0, vocab=3, table_pad=0)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_embedded_equals_lookup_then_shared_z(ops, cfg, dtype):
+    """sum_lstm_embedded(states, table, ids) must give the very bits of
+    sum_lstm_shared_z(states, table[ids.clamp(0, V - 1)]): forget_emb(last_tokens) with the caller's clamp
+    (arctic_speculator.py:744, 845, 862); ids outside the table included."""
+    cfg = dict(cfg)
+    vocab, table_pad = cfg.pop("vocab"), cfg.pop("table_pad")
+    c = make_lstm_case(dtype=dtype, seed=123, **cfg)
+    D, rows = cfg["D"], cfg["rows"]
+    g = torch.Generator().manual_seed(5)
+    table = torch.randn(vocab, D + table_pad, generator=g).to(dtype)[:, :D]
+    ids = torch.randint(0, vocab, (rows, 1), generator=g)
+    ids[0, 0] = -3
+    ids[-1, 0] = vocab + 5
+    z = torch.nn.functional.embedding(ids.clamp(0, vocab - 1), table).flatten(0, 1)
+    alpha = speculator_alpha(3, D)
+    args = [dev(c[k]) for k in ("prev_cell", "w_cell", "b_cell", "w_state", "b_state")]
+    dtable = to_device_pitched(table, DEV)
+    assert dtable.stride(0) == D + table_pad
+    st_e, ce_e = ops.sum_lstm_embedded(dev(c["states"]), dtable, ids.to(DEV), *args, alpha, 1e-6, 1e-6, False)
+    st_s, ce_s = ops.sum_lstm_shared_z(dev(c["states"]), z.to(DEV), *args, alpha, 1e-6, 1e-6, False)
+    torch.cuda.synchronize()
+    assert st_e.stride() == c["prev_cell"].stride()
+    assert torch.equal(st_e, st_s) and torch.equal(ce_e, ce_s)
+    want_s, want_c = oracle.sum_lstm(c["states"], z.repeat(1, 4), c["prev_cell"], c["w_cell"], c["b_cell"],
+                                     c["w_state"], c["b_state"], alpha, 1e-6, 1e-6, False)
+    assert_close(ce_e, want_c, RTOL, ATOL, "cell (embedded z)")
+    assert_close(st_e, want_s, RTOL, ATOL, "state (embedded z)")
+
+
+def test_embedded_errors(ops):
+    bf = dict(dtype=torch.bfloat16, device=DEV)
+    s, pc, table = torch.randn(4, 256, **bf), torch.randn(4, 64, **bf), torch.randn(10, 64, **bf)
+    ids = torch.arange(4, device=DEV)
+    tail = (pc, None, None, None, None, 1.0, 1e-6, 1e-6, False)
+    st, _ = ops.sum_lstm_embedded(s.view(4, 1, 256), table, ids.view(4, 1), pc.view(4, 1, 64), *tail[1:])
+    assert st.shape == (4, 1, 64)
+    with pytest.raises(RuntimeError, match="token ids must be int64"):
+        ops.sum_lstm_embedded(s, table, ids.int(), *tail)
+    with pytest.raises(RuntimeError, match="one contiguous token id per row"):
+        ops.sum_lstm_embedded(s, table, ids[:3], *tail)
+    with pytest.raises(RuntimeError, match="z must have last dim D_gate"):
+        ops.sum_lstm_embedded(s, torch.randn(10, 32, **bf), ids, *tail)
+    with pytest.raises(RuntimeError, match="all input dtypes must match"):
+        ops.sum_lstm_embedded(s, table.half(), ids, *tail)
+    with pytest.raises(RuntimeError, match="no rows"):
+        ops.sum_lstm_embedded(s, table[:0], ids, *tail)
+
+
 def test_rank3_inputs(ops):
     c = make_lstm_case(rows=6, D=256, seed=8)
     for k in ("states", "z4", "prev_cell"):

@@ -76,7 +76,8 @@ def test_decode_step_in_one_graph(ops):
 
 def test_next_row_operators_in_one_graph(ops):
     """gather_rows, the bulk write, ln0 / sqrt2, add + norm + GELU, sum_lstm with the shared embedding row
-    and scatter_rows captured as one graph; every replay must equal the eager run bit for bit."""
+    scatter_rows, argmax + clamp and the operators with the embedding lookup captured as one graph; every
+    replay must equal the eager run bit for bit."""
     T, D, n_sel = 96, 1024, 40
     g = torch.Generator().manual_seed(77)
     case = make_bulk_case(T=T, L=4, H=8, D=128, bs=16, NB=16, kv_cache_dtype="fp8", seed=5, std=1.5)
@@ -90,6 +91,7 @@ def test_next_row_operators_in_one_graph(ops):
     z, w, b = rn(64, D), rn(D), rn(D)
     s4, pc = rn(64, 4 * D), rn(64, D)
     orig = rn(T, D)
+    table = rn(500, D)
     alpha = speculator_alpha(3, D)
 
     def step():
@@ -100,7 +102,11 @@ def test_next_row_operators_in_one_graph(ops):
         st, cell = ops.sum_lstm_shared_z(s4, act, pc, w, b, w, b, alpha, 1e-6, 1e-6, False)
         out = orig.clone()
         ops.scatter_rows([st], idx, [out])
-        return x0, act, st, cell, out, p
+        # the next head: tokens from the argmax of (stand-in) logits, looked up inside the operators
+        tokens = ops.speculator_argmax(st[:, :600], 499)
+        st2, cell2 = ops.sum_lstm_embedded(s4, table, tokens, cell, w, b, w, b, alpha, 1e-6, 1e-6, False)
+        act2 = ops.speculator_embed_add_ln_gelu(x0, table, tokens, w, b, alpha, 1e-6)
+        return x0, act, st, cell, out, p, tokens, st2, cell2, act2
 
     eager = [t.clone() for t in step()]
     torch.cuda.synchronize()

@@ -218,6 +218,36 @@ def cpu_baseline_speculator():
     return out
 
 
+def bench_decode_sizes(ops, dev, mem, steps):
+    """The bulk write at decode batch sizes on the same memory map (40 layers, fp8, no padding): 640 MB of
+    source sets rotated inside one HIP graph so that the K/V rows come from HBM, not from the last-level cache."""
+    out = {}
+    for T in (64, 256, 512, 2048):
+        source_bytes = 2 * T * 40 * 1024 * 2
+        sets = min(64, max(4, -(-640 * 2 ** 20 // source_bytes)))   # 640 MB of K/V rows in rotation
+        ws = [BulkWorkload(f"decode-{T}", T, 40, 8, 128, 16, mem.NB, "fp8", 0.0, 20 + k, 1.5, dev,
+                           bufs=mem.written_layers()) for k in range(sets)]
+        rounds = max(1, (8192 // T) // sets)   # enough launches per replay that the replay's own start-up does not show
+
+        def run():
+            for _ in range(rounds):
+                for w in ws:
+                    ops.reshape_and_cache_flash_bulk(*w.args())
+        run()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            run()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        us = statistics.median(event_times_us(graph.replay, max(10, steps // 2))) / (len(ws) * rounds)
+        out[f"{T}_tokens"] = {"us_per_call_graph": round(us, 2), "GBps": round(ws[0].bytes / us / 1e3, 1),
+                              "hbm_frac": round(ws[0].bytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        del ws, graph
+    return out
+
+
 def load_floor_kernels():
     """bench_floor.so: bare kernels that move the same bytes as the library's and compute nothing
     (built by __graft_entry__.build()).  None when it has not been built."""
@@ -734,6 +764,8 @@ def main():
     us = event_times_us(fn, args.steps)
     kernel_us = statistics.mean(us)
     achieved = w.bytes / kernel_us / 1e3
+    if not args.no_extras:
+        extras["bulk_fp8_70b_decode_sizes_serving_map"] = bench_decode_sizes(ops, dev, mem, args.steps)
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)

@@ -10,6 +10,7 @@ from . import py_custom_ops  # noqa: F401
 from .py_custom_ops import (  # noqa: F401
     gather_rows,
     reshape_and_cache_flash_bulk,
+    reshape_and_cache_flash_bulk_select,
     reshape_and_cache_flash_fp4,
     scatter_rows,
     speculator_add_ln_gelu,

@@ -25,6 +25,8 @@ EXPORTED_SYMBOLS = (
     "arctic_abi_version",
     "arctic_last_error",
     "arctic_reshape_and_cache_flash_bulk",
+    "arctic_reshape_and_cache_flash_bulk_select",
+    "arctic_build_row_map",
     "arctic_reshape_and_cache_flash_fp4",
     "arctic_speculator_ln",
     "arctic_speculator_add_ln_act",
@@ -80,6 +82,11 @@ def _declare(lib: ctypes.CDLL) -> None:
         i32, i32, i32, i32,    # num_layers, num_heads, head_size, block_size
         i64, i64, i32, i32, vp]  # block_stride, num_blocks, src_dtype, kv_cache_dtype, stream
     lib.arctic_reshape_and_cache_flash_bulk.restype = i32
+    lib.arctic_reshape_and_cache_flash_bulk_select.argtypes = lib.arctic_reshape_and_cache_flash_bulk.argtypes[:-1] + [
+        vp, vp, vp, i64, i64, i64, vp]   # row_map, keys_out, values_out, their row strides, num_out_rows, stream
+    lib.arctic_reshape_and_cache_flash_bulk_select.restype = i32
+    lib.arctic_build_row_map.argtypes = [vp, i64, vp, i32, i64, vp]
+    lib.arctic_build_row_map.restype = i32
     lib.arctic_reshape_and_cache_flash_fp4.argtypes = [
         vp, vp, i64, i64, vp, vp, vp, vp, vp, i64, i32, i32, i32, i64, i64, i64, i64, i32, vp]
     lib.arctic_reshape_and_cache_flash_fp4.restype = i32

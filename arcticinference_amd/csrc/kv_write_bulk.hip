@@ -57,6 +57,14 @@ struct BulkParams {
   int block_size;
   int chunks_per_row;    // 16-byte source chunks per (token, layer) row
   int chunk_shift;       // log2(chunks_per_row) or -1
+  // select variant: token t's source rows are also copied, unconverted, to row row_map[t] of keys_out /
+  // values_out (already offset to the first layer of this launch); a negative row or one >= num_out_rows = none
+  const int64_t *row_map;
+  char *keys_out;
+  char *values_out;
+  int64_t out_key_stride_bytes;
+  int64_t out_value_stride_bytes;
+  int64_t num_out_rows;
 };
 
 struct __align__(16) RowDesc {
@@ -113,7 +121,7 @@ __device__ __forceinline__ void emit_chunk(const uint4 &v, const RowDesc &d, int
 // kBulkThreads x kUnroll 16-byte chunks form one batch of a workgroup.  Two shapes
 // are built: 512 x 2 (a workgroup moves two batches or more) and 256 x 4 (decode:
 // few tokens, a single batch per workgroup).
-template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll>
+template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll, bool kSelect>
 __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
     const BulkParams p, const LayerTables tab) {
   constexpr bool kCopy = std::is_same<Dst, Copy>::value;
@@ -159,37 +167,51 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
   // while the row descriptors below are being built.  (A padding token throws
   // its first batch away.)
   const int64_t slot = p.slot_mapping[token];
+  int64_t out_row = -1;
+  if constexpr (kSelect) out_row = p.row_map[token];
   int c = threadIdx.x;
   uint4 cur[kUnroll];
   load_batch(c, cur);
-  if (slot < 0 || slot >= p.num_slots) return;  // padding (or a slot outside the cache): uniform exit, before any barrier
+  // padding (or a slot outside the cache) writes no cache row; both tests are uniform over the workgroup
+  const bool to_cache = slot >= 0 && slot < p.num_slots;
+  const bool to_out = kSelect && out_row >= 0 && out_row < p.num_out_rows;
+  if (!to_cache && !to_out) return;  // before any barrier
 
-  int64_t blk, off;
-  if (slot < 0x7fffffffLL) {
-    const uint32_t s32 = (uint32_t)slot, bs = (uint32_t)p.block_size;
-    blk = s32 / bs;
-    off = s32 - (uint32_t)blk * bs;
-  } else {
-    blk = slot / p.block_size;
-    off = slot - blk * p.block_size;
-  }
-  const int64_t row_elem = blk * p.block_stride + off * (int64_t)p.n;
-
-  // one lane per (layer, K|V) row of this token
-  for (int r = threadIdx.x; r < 2 * nlayers; r += kBulkThreads) {
-    const int layer = layer0 + (r >> 1);
-    const bool is_v = r & 1;
-    const void *base = is_v ? tab.value_cache[layer] : tab.key_cache[layer];
-    RowDesc d;
-    d.dst = (char *)base + row_elem * kDstElemBytes;
-    d.inv = 0.0;
-    if constexpr (!kCopy) {
-      const float *sp = is_v ? tab.v_scale[layer] : tab.k_scale[layer];
-      d.inv = 1.0 / (double)(*sp);
+  if (to_cache) {
+    int64_t blk, off;
+    if (slot < 0x7fffffffLL) {
+      const uint32_t s32 = (uint32_t)slot, bs = (uint32_t)p.block_size;
+      blk = s32 / bs;
+      off = s32 - (uint32_t)blk * bs;
+    } else {
+      blk = slot / p.block_size;
+      off = slot - blk * p.block_size;
     }
-    rows[r] = d;
+    const int64_t row_elem = blk * p.block_stride + off * (int64_t)p.n;
+
+    // one lane per (layer, K|V) row of this token
+    for (int r = threadIdx.x; r < 2 * nlayers; r += kBulkThreads) {
+      const int layer = layer0 + (r >> 1);
+      const bool is_v = r & 1;
+      const void *base = is_v ? tab.value_cache[layer] : tab.key_cache[layer];
+      RowDesc d;
+      d.dst = (char *)base + row_elem * kDstElemBytes;
+      d.inv = 0.0;
+      if constexpr (!kCopy) {
+        const float *sp = is_v ? tab.v_scale[layer] : tab.k_scale[layer];
+        d.inv = 1.0 / (double)(*sp);
+      }
+      rows[r] = d;
+    }
+    __syncthreads();
   }
-  __syncthreads();
+  char *kout = nullptr, *vout = nullptr;
+  if constexpr (kSelect) {
+    if (to_out) {
+      kout = p.keys_out + out_row * p.out_key_stride_bytes + (int64_t)layer0 * p.n * Src::kBytes;
+      vout = p.values_out + out_row * p.out_value_stride_bytes + (int64_t)layer0 * p.n * Src::kBytes;
+    }
+  }
 
   // software-pipelined main loop: the next batch is in flight while this one
   // is converted and stored
@@ -203,7 +225,10 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
       if (cu < total) {
         int r, col;
         locate(cu, r, col);
-        emit_chunk<Src, Dst>(cur[u], rows[r], col);
+        if (!kSelect || to_cache) emit_chunk<Src, Dst>(cur[u], rows[r], col);
+        if constexpr (kSelect) {
+          if (to_out) store16_stream(((r & 1) ? vout : kout) + ((int64_t)(r >> 1) * cpr + col) * 16, cur[u]);
+        }
       }
     }
 #pragma unroll
@@ -223,12 +248,24 @@ __global__ __launch_bounds__(kScalarThreads) void kv_write_bulk_scalar_kernel(
   const int layer0 = group * p.layers_per_group;
   const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
   const int64_t slot = p.slot_mapping[token];
-  if (slot < 0 || slot >= p.num_slots) return;
+  const int64_t out_row = p.row_map ? p.row_map[token] : -1;
+  const bool to_cache = slot >= 0 && slot < p.num_slots;
+  const bool to_out = out_row >= 0 && out_row < p.num_out_rows;
+  if (!to_cache && !to_out) return;
+  const SrcElem *ks = reinterpret_cast<const SrcElem *>(p.keys + token * p.key_stride_bytes);
+  const SrcElem *vs = reinterpret_cast<const SrcElem *>(p.values + token * p.value_stride_bytes);
+  if (to_out) {
+    SrcElem *ko = reinterpret_cast<SrcElem *>(p.keys_out + out_row * p.out_key_stride_bytes);
+    SrcElem *vo = reinterpret_cast<SrcElem *>(p.values_out + out_row * p.out_value_stride_bytes);
+    for (int64_t i = (int64_t)layer0 * p.n + threadIdx.x; i < (int64_t)(layer0 + nlayers) * p.n; i += kScalarThreads) {
+      ko[i] = ks[i];
+      vo[i] = vs[i];
+    }
+  }
+  if (!to_cache) return;
   const int64_t blk = slot / p.block_size;
   const int64_t off = slot - blk * p.block_size;
   const int64_t row_elem = blk * p.block_stride + off * (int64_t)p.n;
-  const SrcElem *ks = reinterpret_cast<const SrcElem *>(p.keys + token * p.key_stride_bytes);
-  const SrcElem *vs = reinterpret_cast<const SrcElem *>(p.values + token * p.value_stride_bytes);
 
   for (int l = layer0; l < layer0 + nlayers; ++l) {
     double kinv = 0.0, vinv = 0.0;
@@ -263,17 +300,22 @@ __global__ __launch_bounds__(kScalarThreads) void kv_write_bulk_scalar_kernel(
   }
 }
 
-template <typename Src, typename Dst>
-static void launch_vec(const BulkParams &p, const LayerTables &tab, int64_t grid, bool wide, hipStream_t s) {
+template <typename Src, typename Dst, bool kSelect>
+static void launch_vec_shape(const BulkParams &p, const LayerTables &tab, int64_t grid, bool wide, hipStream_t s) {
   const dim3 g((unsigned)grid);
   if (p.chunk_shift >= 0) {
     if (wide)
-      hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 512, 2>), g, dim3(512), 0, s, p, tab);
+      hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 512, 2, kSelect>), g, dim3(512), 0, s, p, tab);
     else
-      hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 256, 4>), g, dim3(256), 0, s, p, tab);
+      hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 256, 4, kSelect>), g, dim3(256), 0, s, p, tab);
   } else {
-    hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, false, 256, 4>), g, dim3(256), 0, s, p, tab);
+    hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, false, 256, 4, kSelect>), g, dim3(256), 0, s, p, tab);
   }
+}
+template <typename Src, typename Dst>
+static void launch_vec(const BulkParams &p, const LayerTables &tab, int64_t grid, bool wide, hipStream_t s) {
+  if (p.row_map) launch_vec_shape<Src, Dst, true>(p, tab, grid, wide, s);
+  else launch_vec_shape<Src, Dst, false>(p, tab, grid, wide, s);
 }
 template <typename SrcElem, typename Dst>
 static void launch_scalar(const BulkParams &p, const LayerTables &tab, int64_t grid, int src_dtype,
@@ -299,20 +341,41 @@ static void dispatch_src(bool vec, bool wide, int src_dtype, const BulkParams &p
   }
 }
 
+// row_map[t] = j where indices[j] == t, -1 where no j is: one workgroup, so that the fill is complete
+// (barrier) before the rows are entered.  Tens of thousands of tokens at most: a few microseconds.
+template <typename Index>
+__global__ __launch_bounds__(1024) void build_row_map_kernel(int64_t *__restrict__ row_map, int64_t num_tokens,
+                                                             const Index *__restrict__ indices, int64_t num_indices) {
+  for (int64_t t = threadIdx.x; t < num_tokens; t += blockDim.x) row_map[t] = -1;
+  __syncthreads();
+  for (int64_t j = threadIdx.x; j < num_indices; j += blockDim.x) {
+    const int64_t t = (int64_t)indices[j];
+    if (t >= 0 && t < num_tokens) row_map[t] = j;
+  }
+}
+
 static inline bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p % a) == 0; }
 
 }  // namespace arctic
 
 using namespace arctic;
 
-extern "C" int arctic_reshape_and_cache_flash_bulk(
-    const void *keys, const void *values, int64_t key_stride, int64_t value_stride,
-    const void *const *key_cache_ptrs, const void *const *value_cache_ptrs,
-    const float *const *k_scale_ptrs, const float *const *v_scale_ptrs,
-    const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads,
-    int head_size, int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype,
-    int kv_cache_dtype, void *stream) {
-  const char *fn = "reshape_and_cache_flash_bulk";
+// The rows a launch may also copy out (the select variant); row_map == nullptr: none.
+struct SelectArgs {
+  const int64_t *row_map;
+  void *keys_out;
+  void *values_out;
+  int64_t out_key_stride;    // elements
+  int64_t out_value_stride;
+  int64_t num_out_rows;
+};
+
+static int bulk_entry(const char *fn, const void *keys, const void *values, int64_t key_stride, int64_t value_stride,
+                      const void *const *key_cache_ptrs, const void *const *value_cache_ptrs,
+                      const float *const *k_scale_ptrs, const float *const *v_scale_ptrs,
+                      const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads, int head_size,
+                      int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype, int kv_cache_dtype,
+                      const SelectArgs &sel, void *stream) {
   if (num_layers == 0 || num_tokens == 0) return ARCTIC_OK;  // reference :87-89
   if (num_layers < 0 || num_layers > ARCTIC_MAX_LAYERS)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: num_layers=%d outside [0, %d]", fn, num_layers,
@@ -329,6 +392,9 @@ extern "C" int arctic_reshape_and_cache_flash_bulk(
     return fail(ARCTIC_ERR_UNSUPPORTED, "%s: Unsupported data type of kv cache: %d", fn, kv_cache_dtype);
   if (!keys || !values || !slot_mapping || !key_cache_ptrs || !value_cache_ptrs)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
+  if (sel.row_map && (!sel.keys_out || !sel.values_out || sel.num_out_rows < 0 || sel.out_key_stride < 0 ||
+                      sel.out_value_stride < 0))
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: the selected rows need keys_out, values_out and non-negative sizes", fn);
   const bool quant = kv_cache_dtype != ARCTIC_KV_AUTO;
   if (quant && (!k_scale_ptrs || !v_scale_ptrs))
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: fp8 cache needs k_scales and v_scales", fn);
@@ -352,6 +418,10 @@ extern "C" int arctic_reshape_and_cache_flash_bulk(
              ((value_stride * es) % 16 == 0 || num_tokens == 1) && ((block_stride * des) % store_bytes == 0);
   for (int l = 0; vec && l < num_layers; ++l)
     vec = aligned(key_cache_ptrs[l], store_bytes) && aligned(value_cache_ptrs[l], store_bytes);
+  if (vec && sel.row_map)
+    vec = aligned(sel.keys_out, 16) && aligned(sel.values_out, 16) &&
+          ((sel.out_key_stride * es) % 16 == 0 || sel.num_out_rows <= 1) &&
+          ((sel.out_value_stride * es) % 16 == 0 || sel.num_out_rows <= 1);
 
   hipStream_t s = (hipStream_t)stream;
   for (int first = 0; first < num_layers; first += kLayersPerLaunch) {
@@ -368,6 +438,12 @@ extern "C" int arctic_reshape_and_cache_flash_bulk(
     p.keys = (const char *)keys + (int64_t)first * n * es;
     p.values = (const char *)values + (int64_t)first * n * es;
     p.slot_mapping = slot_mapping;
+    p.row_map = sel.row_map;
+    p.keys_out = sel.row_map ? (char *)sel.keys_out + (int64_t)first * n * es : nullptr;
+    p.values_out = sel.row_map ? (char *)sel.values_out + (int64_t)first * n * es : nullptr;
+    p.out_key_stride_bytes = sel.out_key_stride * es;
+    p.out_value_stride_bytes = sel.out_value_stride * es;
+    p.num_out_rows = sel.row_map ? sel.num_out_rows : 0;
     p.key_stride_bytes = key_stride * es;
     p.value_stride_bytes = value_stride * es;
     p.block_stride = block_stride;
@@ -420,4 +496,50 @@ extern "C" int arctic_reshape_and_cache_flash_bulk(
     if (rc) return rc;
   }
   return ARCTIC_OK;
+}
+
+extern "C" int arctic_reshape_and_cache_flash_bulk(
+    const void *keys, const void *values, int64_t key_stride, int64_t value_stride,
+    const void *const *key_cache_ptrs, const void *const *value_cache_ptrs,
+    const float *const *k_scale_ptrs, const float *const *v_scale_ptrs,
+    const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads,
+    int head_size, int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype,
+    int kv_cache_dtype, void *stream) {
+  const SelectArgs none = {nullptr, nullptr, nullptr, 0, 0, 0};
+  return bulk_entry("reshape_and_cache_flash_bulk", keys, values, key_stride, value_stride, key_cache_ptrs,
+                    value_cache_ptrs, k_scale_ptrs, v_scale_ptrs, slot_mapping, num_tokens, num_layers, num_heads,
+                    head_size, block_size, block_stride, num_blocks, src_dtype, kv_cache_dtype, none, stream);
+}
+
+extern "C" int arctic_reshape_and_cache_flash_bulk_select(
+    const void *keys, const void *values, int64_t key_stride, int64_t value_stride,
+    const void *const *key_cache_ptrs, const void *const *value_cache_ptrs,
+    const float *const *k_scale_ptrs, const float *const *v_scale_ptrs,
+    const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads,
+    int head_size, int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype,
+    int kv_cache_dtype, const int64_t *row_map, void *keys_out, void *values_out,
+    int64_t out_key_stride, int64_t out_value_stride, int64_t num_out_rows, void *stream) {
+  const char *fn = "reshape_and_cache_flash_bulk_select";
+  if (num_layers != 0 && num_tokens != 0 && !row_map) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null row map", fn);
+  const SelectArgs sel = {row_map, keys_out, values_out, out_key_stride, out_value_stride, num_out_rows};
+  return bulk_entry(fn, keys, values, key_stride, value_stride, key_cache_ptrs, value_cache_ptrs, k_scale_ptrs,
+                    v_scale_ptrs, slot_mapping, num_tokens, num_layers, num_heads, head_size, block_size, block_stride,
+                    num_blocks, src_dtype, kv_cache_dtype, sel, stream);
+}
+
+extern "C" int arctic_build_row_map(int64_t *row_map, int64_t num_tokens, const void *indices, int index_bytes,
+                                    int64_t num_indices, void *stream) {
+  const char *fn = "build_row_map";
+  if (index_bytes != 4 && index_bytes != 8) return fail(ARCTIC_ERR_UNSUPPORTED, "%s: indices must be int32 or int64", fn);
+  if (num_tokens < 0 || num_indices < 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: negative size", fn);
+  if (num_tokens == 0) return ARCTIC_OK;
+  if (!row_map || (num_indices > 0 && !indices)) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  hipStream_t s = (hipStream_t)stream;
+  if (index_bytes == 8)
+    hipLaunchKernelGGL(build_row_map_kernel<int64_t>, dim3(1), dim3(1024), 0, s, row_map, num_tokens,
+                       (const int64_t *)indices, num_indices);
+  else
+    hipLaunchKernelGGL(build_row_map_kernel<int32_t>, dim3(1), dim3(1024), 0, s, row_map, num_tokens,
+                       (const int32_t *)indices, num_indices);
+  return check_launch(fn);
 }

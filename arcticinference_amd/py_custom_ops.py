@@ -62,6 +62,11 @@ _EXTRA_SCHEMAS = {
         "speculator_embed_add_ln_act_cuda(Tensor input, Tensor emb_weight, Tensor token_ids, Tensor? weight, "
         "Tensor? bias, float alpha, float eps, str activation, float out_scale) -> Tensor",
     "speculator_argmax_cuda": "speculator_argmax_cuda(Tensor logits, int max_index) -> Tensor",
+    "reshape_and_cache_flash_bulk_select":
+        "reshape_and_cache_flash_bulk_select(Tensor keys, Tensor values, Tensor(c!)[] key_caches, "
+        "Tensor(d!)[] value_caches, Tensor slot_mapping, str kv_cache_dtype, Tensor(e)[] k_scales, "
+        "Tensor(f)[] v_scales, int num_heads, int head_size, Tensor logits_indices, Tensor(g!) k_out, "
+        "Tensor(h!) v_out) -> ()",
     "gather_rows": "gather_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
     "scatter_rows": "scatter_rows(Tensor[] sources, Tensor indices, Tensor(a!)[] outs) -> ()",
 }
@@ -157,6 +162,7 @@ def _reshape_and_cache_flash_bulk_impl(
     v_scales: List[torch.Tensor],
     num_heads: int,
     head_size: int,
+    _select: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor, int]] = None,
 ) -> None:
     """Host side of the bulk KV write; follows the reference's launcher
     (csrc/custom_ops/reshape_and_cache_flash_bulk.cu:77-144) up to the point
@@ -200,14 +206,70 @@ def _reshape_and_cache_flash_bulk_impl(
     devices.update((values.device, slot_mapping.device, keys.device))
     _check(len(devices) == 1, "reshape_and_cache_flash_bulk: all tensors must be on the same device")
 
+    common = (keys.data_ptr(), values.data_ptr(), key_stride, value_stride,
+              _ptr_table(key_caches), _ptr_table(value_caches),
+              _ptr_table(k_scales), _ptr_table(v_scales),
+              slot_mapping.data_ptr(), num_tokens, num_layers, int(num_heads), int(head_size),
+              int(block_size), int(block_stride), int(key_caches[0].size(0)), src_code, kv_code)
     with _on_device_of(keys):
-        rc = lib.arctic_reshape_and_cache_flash_bulk(
-            keys.data_ptr(), values.data_ptr(), key_stride, value_stride,
-            _ptr_table(key_caches), _ptr_table(value_caches),
-            _ptr_table(k_scales), _ptr_table(v_scales),
-            slot_mapping.data_ptr(), num_tokens, num_layers, int(num_heads), int(head_size),
-            int(block_size), int(block_stride), int(key_caches[0].size(0)), src_code, kv_code, _stream_of(keys))
+        if _select is None:
+            rc = lib.arctic_reshape_and_cache_flash_bulk(*common, _stream_of(keys))
+        else:
+            row_map, k_out, v_out, out_rows = _select
+            rc = lib.arctic_reshape_and_cache_flash_bulk_select(
+                *common, row_map.data_ptr(), k_out.data_ptr(), v_out.data_ptr(), k_out.stride(0), v_out.stride(0),
+                out_rows, _stream_of(keys))
     _native.check(rc)
+
+
+def _reshape_and_cache_flash_bulk_select_impl(
+    keys: torch.Tensor,
+    values: torch.Tensor,
+    key_caches: List[torch.Tensor],
+    value_caches: List[torch.Tensor],
+    slot_mapping: torch.Tensor,
+    kv_cache_dtype: str,
+    k_scales: List[torch.Tensor],
+    v_scales: List[torch.Tensor],
+    num_heads: int,
+    head_size: int,
+    logits_indices: torch.Tensor,
+    k_out: torch.Tensor,
+    v_out: torch.Tensor,
+) -> None:
+    """The bulk KV write and, in the same pass over keys / values, ``k_out[j] = keys[logits_indices[j]]`` and
+    ``v_out[j] = values[logits_indices[j]]``: the two largest index_select calls of swiftkv_select
+    (arctic_inference/vllm/swiftkv/llama_swiftkv.py:663-679) without a second read of k_states / v_states.
+    ``logits_indices`` must not repeat an index (SwiftKV's never do: one per request)."""
+    fn = "reshape_and_cache_flash_bulk_select"
+    num_layers = len(key_caches)
+    n_sel = logits_indices.numel()
+    _check(logits_indices.is_cuda and logits_indices.dim() == 1 and logits_indices.dtype in (torch.int32, torch.int64),
+           f"{fn}: logits_indices must be a 1-D int32 or int64 CUDA tensor")
+    for name, src, out in (("k_out", keys, k_out), ("v_out", values, v_out)):
+        _check(out.is_cuda and out.device == src.device and out.dtype == src.dtype,
+               f"{fn}: {name} must be on the device of keys / values and of their type")
+        _check(out.dim() == 2 and out.size(0) >= n_sel, f"{fn}: {name} must be 2-D with at least {n_sel} rows")
+        _check(out.stride(1) == 1, f"{fn}: rows of {name} must be contiguous")
+    if num_layers == 0 or slot_mapping.size(0) == 0:
+        # nothing is written to a cache, but the selected rows are still wanted
+        if n_sel:
+            torch.index_select(keys, 0, logits_indices, out=k_out[:n_sel])
+            torch.index_select(values, 0, logits_indices, out=v_out[:n_sel])
+        return
+    width = num_layers * int(num_heads) * int(head_size)
+    _check(k_out.size(1) == width and v_out.size(1) == width and keys.size(1) >= width and values.size(1) >= width,
+           f"{fn}: k_out and v_out must have {width} columns (layers x heads x head_size)")
+    # the inverse of logits_indices: which output row, if any, a token goes to
+    num_tokens = slot_mapping.size(0)
+    row_map = torch.empty(num_tokens, dtype=torch.int64, device=keys.device)
+    idx = logits_indices if logits_indices.is_contiguous() else logits_indices.contiguous()
+    with _on_device_of(keys):
+        rc = _lib().arctic_build_row_map(row_map.data_ptr(), num_tokens, idx.data_ptr(), idx.element_size(), n_sel,
+                                         _stream_of(keys))
+    _native.check(rc)
+    _reshape_and_cache_flash_bulk_impl(keys, values, key_caches, value_caches, slot_mapping, kv_cache_dtype, k_scales,
+                                       v_scales, num_heads, head_size, _select=(row_map, k_out, v_out, n_sel))
 
 
 def _reshape_and_cache_flash_fp4_impl(
@@ -543,6 +605,7 @@ _IMPLS = {
     "speculator_add_ln_act_cuda": _speculator_add_ln_act_impl,
     "speculator_embed_add_ln_act_cuda": _speculator_embed_add_ln_act_impl,
     "reshape_and_cache_flash_bulk": _reshape_and_cache_flash_bulk_impl,
+    "reshape_and_cache_flash_bulk_select": _reshape_and_cache_flash_bulk_select_impl,
     "reshape_and_cache_flash_fp4": _reshape_and_cache_flash_fp4_impl,
     "speculator_ln_cuda": _speculator_ln_impl,
     "sum_lstm_cuda": _sum_lstm_impl,
@@ -583,6 +646,7 @@ _META_IMPLS = {
     "speculator_embed_add_ln_act_cuda": _meta_like_input,
     "speculator_argmax_cuda": _meta_argmax,
     "reshape_and_cache_flash_bulk": _meta_nothing,
+    "reshape_and_cache_flash_bulk_select": _meta_nothing,
     "reshape_and_cache_flash_fp4": _meta_nothing,
     "gather_rows": _meta_nothing,
     "scatter_rows": _meta_nothing,
@@ -674,6 +738,31 @@ def reshape_and_cache_flash_bulk(
 ) -> None:
     _call("reshape_and_cache_flash_bulk", keys, values, key_caches, value_caches, slot_mapping,
                                         kv_cache_dtype, k_scales, v_scales, num_heads, head_size)
+
+
+def reshape_and_cache_flash_bulk_select(
+    keys: torch.Tensor,
+    values: torch.Tensor,
+    key_caches: List[torch.Tensor],
+    value_caches: List[torch.Tensor],
+    slot_mapping: torch.Tensor,
+    kv_cache_dtype: str,
+    k_scales: List[torch.Tensor],
+    v_scales: List[torch.Tensor],
+    num_heads: int,
+    head_size: int,
+    logits_indices: torch.Tensor,
+    k_out: torch.Tensor,
+    v_out: torch.Tensor,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``reshape_and_cache_flash_bulk(...)`` followed by ``torch.index_select(keys, 0, logits_indices,
+    out=k_out[:n])`` and the same for values (arctic_inference/vllm/swiftkv/llama_swiftkv.py:617-622, 663-679),
+    with keys / values read once for both.  Returns ``(k_out[:n], v_out[:n])``.  ``logits_indices`` must not
+    repeat an index."""
+    _call("reshape_and_cache_flash_bulk_select", keys, values, key_caches, value_caches, slot_mapping, kv_cache_dtype,
+          k_scales, v_scales, num_heads, head_size, logits_indices, k_out, v_out)
+    n = logits_indices.numel()
+    return k_out[:n], v_out[:n]
 
 
 def reshape_and_cache_flash_fp4(

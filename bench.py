@@ -434,6 +434,57 @@ def bench_row_gather(ops, dev, steps):
     return out
 
 
+def bench_bulk_select(ops, dev, steps):
+    """The bulk write and swiftkv_select of a decode-only batch together (llama_swiftkv.py:617-622, 663-679):
+    512 tokens, 40 layers x 8 x 128, fp8 cache of 8192 blocks per layer; hidden_states and residual 8192 bf16.
+    As the reference's caller runs them (bulk write + five index_select), with gather_rows for the five, and
+    with the K/V selection folded into the bulk write (k_states / v_states read once).  Four rotating sets."""
+    T, L, H, D, bs, NB, hidden, sets = 512, 40, 8, 128, 16, 8192, 8192, 4
+    n = H * D
+    g = torch.Generator(device=dev).manual_seed(8)
+    rn = lambda *s: torch.randn(*s, generator=g, device=dev).to(torch.bfloat16)
+    bufs = [torch.zeros(2, NB, bs, H, D, dtype=torch.uint8, device=dev) for _ in range(L)]
+    kc, vc = [b[0] for b in bufs], [b[1] for b in bufs]
+    sc = [torch.tensor([0.02], device=dev) for _ in range(L)]
+    K, V = [rn(T, L * n) for _ in range(sets)], [rn(T, L * n) for _ in range(sets)]
+    Hs, Rs = [rn(T, hidden) for _ in range(sets)], [rn(T, hidden) for _ in range(sets)]
+    P = torch.arange(T, device=dev)
+    S = [torch.randperm(NB * bs, generator=g, device=dev)[:T] for _ in range(sets)]
+    idx = torch.arange(T, device=dev)
+    ob = [torch.empty(T, hidden, dtype=torch.bfloat16, device=dev), torch.empty(T, hidden, dtype=torch.bfloat16, device=dev),
+          torch.empty(T, dtype=torch.int64, device=dev), torch.empty(T, L * n, dtype=torch.bfloat16, device=dev),
+          torch.empty(T, L * n, dtype=torch.bfloat16, device=dev)]
+
+    def reference_sequence(i):
+        ops.reshape_and_cache_flash_bulk(K[i], V[i], kc, vc, S[i], "fp8", sc, sc, H, D)
+        for src, o in zip([Hs[i], Rs[i], P, K[i], V[i]], ob):
+            torch.index_select(src, 0, idx, out=o)
+
+    def with_gather_rows(i):
+        ops.reshape_and_cache_flash_bulk(K[i], V[i], kc, vc, S[i], "fp8", sc, sc, H, D)
+        ops.gather_rows([Hs[i], Rs[i], P, K[i], V[i]], idx, ob)
+
+    def with_bulk_select(i):
+        ops.reshape_and_cache_flash_bulk_select(K[i], V[i], kc, vc, S[i], "fp8", sc, sc, H, D, idx, ob[3], ob[4])
+        ops.gather_rows([Hs[i], Rs[i], P], idx, ob[:3])
+
+    out = {}
+    for name, fn in (("bulk_write_then_five_index_select", reference_sequence),
+                     ("bulk_write_then_gather_rows", with_gather_rows),
+                     ("bulk_select_then_gather_rows_of_three", with_bulk_select)):
+        for i in range(sets):
+            fn(i)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(sets):
+                fn(i)
+        graph.replay()
+        torch.cuda.synchronize()
+        out[name] = {"us_per_step_graph": round(statistics.median(event_times_us(graph.replay, max(10, steps // 2))) / sets, 2)}
+    return out
+
+
 def bench_suffix_decoding():
     """Suffix-tree speculation on the host cores (no GPU): libarctic_suffix.so next to the reference's own
     code (oracle/_ref, compiled from the reference's sources, when it is there), both driven through the
@@ -831,6 +882,8 @@ def main():
             extras["speculator"]["cpu_baseline"] = cpu_baseline_speculator()
         extras["decode_mix"] = bench_decode_mix(ops, dev, args.steps)
         extras["swiftkv_select_decode_70b"] = bench_row_gather(ops, dev, args.steps)
+        extras["bulk_write_and_select_decode_70b"] = bench_bulk_select(ops, dev, args.steps)
+        torch.cuda.empty_cache()
         extras["speculator_argmax_512x128256"] = bench_argmax(ops, dev, args.steps)
         extras["suffix_decoding_cpu"] = bench_suffix_decoding()
         log(f"extras: {extras}")

@@ -101,6 +101,40 @@ int arctic_reshape_and_cache_flash_bulk(
     int kv_cache_dtype, void *stream);
 
 /*
+ * Helper of arctic_reshape_and_cache_flash_bulk_select: the inverse of an index list.
+ *   row_map[t] = j where indices[j] == t, -1 for every other t < num_tokens
+ * in one launch (indices outside [0, num_tokens) are ignored; of repeated indices one wins).  No counterpart in
+ * the reference, whose index_select calls take logits_indices as it is (llama_swiftkv.py:663-679).
+ *   row_map    device int64[num_tokens], written
+ *   indices    device, num_indices entries of index_bytes (4 or 8) each, signed
+ */
+int arctic_build_row_map(int64_t *row_map, int64_t num_tokens, const void *indices, int index_bytes,
+                         int64_t num_indices, void *stream);
+
+/*
+ * The bulk KV-cache write with the row selection that follows it in the caller folded in.  Everything
+ * arctic_reshape_and_cache_flash_bulk does, and in the same pass over the source: token t's rows are also
+ * copied, unconverted, to row row_map[t] of keys_out / values_out, which is
+ *   index_fn("k_states", k_states, logits_indices), index_fn("v_states", v_states, logits_indices)
+ *        arctic_inference/vllm/swiftkv/llama_swiftkv.py:663-679
+ * with row_map the inverse of logits_indices (row_map[logits_indices[j]] = j, -1 elsewhere), so k_states and
+ * v_states are read once for both steps.  No single function of the reference corresponds to it.
+ *
+ *   row_map            device int64[num_tokens]; negative or >= num_out_rows: the token is not copied.
+ *                      A token is copied whether or not its slot is padding.
+ *   keys_out, values_out   device; rows of num_layers*n elements of src_dtype, out_*_stride ELEMENTS apart
+ *   other arguments as arctic_reshape_and_cache_flash_bulk
+ */
+int arctic_reshape_and_cache_flash_bulk_select(
+    const void *keys, const void *values, int64_t key_stride, int64_t value_stride,
+    const void *const *key_cache_ptrs, const void *const *value_cache_ptrs,
+    const float *const *k_scale_ptrs, const float *const *v_scale_ptrs,
+    const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads,
+    int head_size, int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype,
+    int kv_cache_dtype, const int64_t *row_map, void *keys_out, void *values_out,
+    int64_t out_key_stride, int64_t out_value_stride, int64_t num_out_rows, void *stream);
+
+/*
  * NVFP4-style KV-cache write for ONE layer: e2m1 values, two per byte (first element
  * in the low nibble), plus one e4m3 scale byte per 16 elements.  Replaces
  *   reshape_and_cache_flash_fp4()             csrc/custom_ops/reshape_and_cache_flash_fp4.cu:256-337

@@ -94,9 +94,11 @@ def test_next_row_operators_in_one_graph(ops):
     table = rn(500, D)
     alpha = speculator_alpha(3, D)
 
+    kv_bufs = [torch.zeros(64, 4 * 1024, dtype=torch.bfloat16, device=DEV) for _ in range(2)]
+
     def step():
         h, r, p = ops.gather_rows([hidden, residual, positions], idx, bufs)
-        ops.reshape_and_cache_flash_bulk(*bulk_args(dcase))
+        k_sel, v_sel = ops.reshape_and_cache_flash_bulk_select(*bulk_args(dcase), idx, *kv_bufs)
         x0 = ops.speculator_ln_scaled(h, None, None, 1e-6, 0.70710678)
         act = ops.speculator_add_ln_gelu(x0, z, w, b, alpha, 1e-6)
         st, cell = ops.sum_lstm_shared_z(s4, act, pc, w, b, w, b, alpha, 1e-6, 1e-6, False)
@@ -106,7 +108,7 @@ def test_next_row_operators_in_one_graph(ops):
         tokens = ops.speculator_argmax(st[:, :600], 499)
         st2, cell2 = ops.sum_lstm_embedded(s4, table, tokens, cell, w, b, w, b, alpha, 1e-6, 1e-6, False)
         act2 = ops.speculator_embed_add_ln_gelu(x0, table, tokens, w, b, alpha, 1e-6)
-        return x0, act, st, cell, out, p, tokens, st2, cell2, act2
+        return x0, act, st, cell, out, p, tokens, st2, cell2, act2, k_sel, v_sel
 
     eager = [t.clone() for t in step()]
     torch.cuda.synchronize()
@@ -114,17 +116,25 @@ def test_next_row_operators_in_one_graph(ops):
     want[idx] = eager[2][:n_sel]
     assert torch.equal(eager[4], want)
     assert torch.equal(eager[5][:n_sel], positions[idx])
+    assert torch.equal(eager[10], dcase["keys"][idx]) and torch.equal(eager[11], dcase["values"][idx])
+    oracle.reshape_and_cache_flash_bulk(*bulk_args(case))
+    assert_bulk_equal(dcase["bufs"], case["bufs"])
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         outs = step()
     for replay in range(3):
-        for t in bufs:
+        for t in bufs + kv_bufs + dcase["bufs"]:
             t.zero_()                          # eager work between replays
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
         for a, e in zip(outs, eager):
             assert torch.equal(a, e), f"replay {replay} differs from the eager run"
+        # the caches were cleared before the replay: every written row is back, the rest stays zero
+        want = [torch.zeros_like(b) for b in case["bufs"]]
+        zcase = dict(case, bufs=want, key_caches=[b[0] for b in want], value_caches=[b[1] for b in want])
+        oracle.reshape_and_cache_flash_bulk(*bulk_args(zcase))
+        assert_bulk_equal(dcase["bufs"], want)
 
 
 def test_direct_c_abi_calls(ops):

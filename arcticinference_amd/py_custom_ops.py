@@ -254,8 +254,7 @@ def _reshape_and_cache_flash_bulk_select_impl(
     if num_layers == 0 or slot_mapping.size(0) == 0:
         # nothing is written to a cache, but the selected rows are still wanted
         if n_sel:
-            torch.index_select(keys, 0, logits_indices, out=k_out[:n_sel])
-            torch.index_select(values, 0, logits_indices, out=v_out[:n_sel])
+            _move_rows_impl("gather_rows", [keys, values], logits_indices, [k_out, v_out], False)
         return
     width = num_layers * int(num_heads) * int(head_size)
     _check(k_out.size(1) == width and v_out.size(1) == width and keys.size(1) >= width and values.size(1) >= width,

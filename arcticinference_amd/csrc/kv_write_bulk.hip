@@ -375,7 +375,7 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
                       const float *const *k_scale_ptrs, const float *const *v_scale_ptrs,
                       const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads, int head_size,
                       int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype, int kv_cache_dtype,
-                      const SelectArgs &sel, void *stream) {
+                      const SelectArgs &sel_in, void *stream) {
   if (num_layers == 0 || num_tokens == 0) return ARCTIC_OK;  // reference :87-89
   if (num_layers < 0 || num_layers > ARCTIC_MAX_LAYERS)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: num_layers=%d outside [0, %d]", fn, num_layers,
@@ -392,9 +392,12 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
     return fail(ARCTIC_ERR_UNSUPPORTED, "%s: Unsupported data type of kv cache: %d", fn, kv_cache_dtype);
   if (!keys || !values || !slot_mapping || !key_cache_ptrs || !value_cache_ptrs)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
-  if (sel.row_map && (!sel.keys_out || !sel.values_out || sel.num_out_rows < 0 || sel.out_key_stride < 0 ||
-                      sel.out_value_stride < 0))
-    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: the selected rows need keys_out, values_out and non-negative sizes", fn);
+  SelectArgs sel = sel_in;
+  if (sel.row_map && (sel.num_out_rows < 0 || sel.out_key_stride < 0 || sel.out_value_stride < 0))
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: negative number of output rows or row pitch", fn);
+  if (sel.row_map && sel.num_out_rows == 0) sel.row_map = nullptr;   // no row to copy to: the plain write
+  if (sel.row_map && (!sel.keys_out || !sel.values_out))
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null keys_out or values_out", fn);
   const bool quant = kv_cache_dtype != ARCTIC_KV_AUTO;
   if (quant && (!k_scale_ptrs || !v_scale_ptrs))
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: fp8 cache needs k_scales and v_scales", fn);

@@ -81,6 +81,34 @@ def test_rows_that_force_the_element_wise_kernel(ops, kv):
     run_select(ops, case, idx, 9, out_pad=1)
 
 
+def test_random_configurations(ops):
+    """Seeded sweep over shapes, dtypes, layouts, pitches, padding and selections (none, few, all, shuffled)."""
+    import random
+    rnd = random.Random(77)
+    for it in range(30):
+        H = rnd.choice([1, 2, 3, 8])
+        D = rnd.choice([16, 64, 80, 128, 20])
+        cfg = dict(T=rnd.choice([1, 2, 7, 33, 130, 600]), L=rnd.choice([1, 2, 5, 16, 33, 65]), H=H, D=D,
+                   bs=rnd.choice([1, 4, 16, 32]), NB=0,
+                   src_dtype=rnd.choice([torch.bfloat16, torch.float16, torch.float32]),
+                   kv_cache_dtype=rnd.choice(["auto", "fp8", "fp8_e5m2"]), seed=3000 + it, std=rnd.choice([0.1, 1.5, 30.0]),
+                   pad_fraction=rnd.choice([0.0, 0.1, 0.5]), layout=rnd.choice(["flash", "flashinfer"]),
+                   key_pad=rnd.choice([0, 0, 8, 3]))
+        cfg["NB"] = (cfg["T"] + cfg["bs"] - 1) // cfg["bs"] + rnd.choice([0, 1, 5])
+        if cfg["T"] * cfg["L"] * H * D > 20_000_000:
+            cfg["L"] = max(1, 20_000_000 // (cfg["T"] * H * D))
+        T = cfg["T"]
+        g = torch.Generator().manual_seed(it)
+        n_sel = rnd.choice([0, 1, max(1, T // 3), T])
+        idx = torch.randperm(T, generator=g)[:n_sel]
+        if rnd.random() < 0.6:
+            idx = torch.sort(idx).values
+        try:
+            run_select(ops, make_bulk_case(**cfg), idx, n_sel + rnd.choice([0, 3]), out_pad=rnd.choice([0, 8, 1]))
+        except AssertionError as e:
+            raise AssertionError(f"configuration {it}: {cfg}, {n_sel} selected: {e}") from None
+
+
 def test_empty_selection_and_no_layers(ops):
     case = make_bulk_case(T=64, L=4, H=8, D=128, bs=16, NB=8, kv_cache_dtype="fp8", seed=46)
     run_select(ops, case, torch.empty(0, dtype=torch.int64), 4)

@@ -71,3 +71,28 @@ def test_empty_and_errors(ops):
         ops.speculator_argmax(torch.zeros(4, 8, dtype=torch.float64, device=DEV), 8)
     with pytest.raises(RuntimeError, match="last dimension must be contiguous"):
         ops.speculator_argmax(torch.zeros(8, 4, device=DEV).t(), 8)
+
+
+def test_random_configurations(ops):
+    """Seeded sweep over types, row counts, row lengths around the chunk and workgroup sizes, row pitches, start
+    offsets (unaligned rows take the element-wise path), value ranges with many ties, and sprinkled NaN / inf."""
+    import random
+    rnd = random.Random(13)
+    for it in range(60):
+        g = torch.Generator().manual_seed(700 + it)
+        dtype = rnd.choice([torch.bfloat16, torch.float16, torch.float32])
+        rows = rnd.choice([1, 2, 17, 130])
+        cols = rnd.choice([1, 2, 7, 8, 9, 63, 64, 65, 255, 256, 257, 1023, 1025, 4096, 8200, 33000])
+        pad, off = rnd.choice([0, 0, 1, 8, 24]), rnd.choice([0, 0, 1, 3, 8])
+        levels = rnd.choice([2, 5, 1000])                 # few distinct values: ties everywhere
+        base = torch.randint(0, levels, (rows, off + cols + pad), generator=g).float() - levels / 2
+        for special in (float("nan"), float("inf"), -float("inf")):
+            if rnd.random() < 0.3:
+                r, c = rnd.randrange(rows), rnd.randrange(off + cols + pad)
+                base[r, c] = special
+        base = base.to(dtype)
+        logits = base[:, off:off + cols]
+        vocab = rnd.choice([cols, max(1, cols - 3), cols + 5])
+        got = ops.speculator_argmax(base.to(DEV)[:, off:off + cols], vocab)
+        want = torch.argmax(logits.float(), dim=-1).clamp_(0, vocab - 1)
+        assert torch.equal(got.cpu(), want), f"configuration {it}: {dtype}, {rows} x {cols}, pad {pad}, offset {off}"

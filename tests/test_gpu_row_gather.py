@@ -155,3 +155,41 @@ def test_c_abi_directly(ops):
     assert lib.arctic_gather_rows(1, vp(src.data_ptr()), vp(dst.data_ptr()), i64(40), i64(40), i64(40), idx.data_ptr(),
                                   2, 3, 6, 0, None) == 2
     assert b"int32 or int64" in lib.arctic_last_error()
+
+
+def test_random_configurations(ops):
+    """Seeded sweep over tensor counts, element types, row lengths, pitches, start offsets (so that every unit
+    size from 1 to 16 bytes is used) and index lists, gather and scatter."""
+    import random
+    rnd = random.Random(11)
+    dtypes = [torch.uint8, torch.int16, torch.bfloat16, torch.float32, torch.int64]
+    for it in range(40):
+        g = torch.Generator().manual_seed(500 + it)
+        rows = rnd.choice([1, 3, 40, 257])
+        n_idx = rnd.choice([0, 1, 5, rows, rows + 7])
+        tensors, dsrc = [], []
+        for _ in range(rnd.choice([1, 2, 5, 8])):
+            dt = rnd.choice(dtypes)
+            cols, pad, off = rnd.choice([1, 3, 8, 33, 256, 1000]), rnd.choice([0, 0, 1, 8]), rnd.choice([0, 0, 1, 4])
+            base = torch.randint(0, 127, (rows, off + cols + pad), generator=g).to(dt)
+            tensors.append(base[:, off:off + cols])
+            dsrc.append(base.to(DEV)[:, off:off + cols])
+        idx = torch.randint(-1, rows + 1, (n_idx,), generator=g)         # a few out of range on both sides
+        try:
+            bufs = [sentinel_like(t, n_idx + 2) for t in tensors]
+            want = oracle.gather_rows(tensors, idx, [b.clone() for b in bufs])
+            got = ops.gather_rows(dsrc, idx.to(DEV), [b.to(DEV) for b in bufs])
+            for k, (gk, wk) in enumerate(zip(got, want)):
+                assert torch.equal(gk.cpu().view(torch.uint8), wk.view(torch.uint8)), f"gather: tensor {k} differs"
+            # scatter the first rows of each tensor to distinct places of a sentinel-filled destination
+            n_sc = min(rows, 6)
+            perm = torch.randperm(rows + 3, generator=g)[:n_sc]
+            dst = [sentinel_like(t, rows + 3) for t in tensors]
+            ddst = [d.to(DEV) for d in dst]
+            oracle.scatter_rows(tensors, perm, dst)
+            ops.scatter_rows(dsrc, perm.to(DEV), ddst)
+            for k, (gk, wk) in enumerate(zip(ddst, dst)):
+                assert torch.equal(gk.cpu().view(torch.uint8), wk.view(torch.uint8)), f"scatter: tensor {k} differs"
+        except AssertionError as e:
+            raise AssertionError(f"configuration {it}: {[(t.dtype, tuple(t.shape), t.stride(0)) for t in tensors]}, "
+                                 f"{n_idx} indices: {e}") from None

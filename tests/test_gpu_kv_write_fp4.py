@@ -94,3 +94,20 @@ def test_errors(ops):
         ops.reshape_and_cache_flash_fp4(key, value, kc[0], vc[0], ksc, vsc, slots, "fp4", z, z)
     with pytest.raises(RuntimeError, match="block_stride mismatch"):
         ops.reshape_and_cache_flash_fp4(key, value, kc, torch.cat([vc, vc], dim=1), ksc, vsc, slots, "fp4", z, z)
+
+
+def test_random_configurations(ops):
+    """Seeded sweep over token counts, head counts, head sizes (powers of two and not), block sizes, both layouts,
+    both types and value ranges from denormal-sized to overflowing."""
+    import random
+    rnd = random.Random(17)
+    for it in range(40):
+        T, H = rnd.choice([1, 2, 7, 33, 130, 600]), rnd.choice([1, 2, 3, 8])
+        D, bs = rnd.choice([16, 32, 48, 64, 80, 128]), rnd.choice([1, 4, 16, 32])
+        NB = (T + bs - 1) // bs + rnd.choice([0, 1, 5])
+        dtype, nhd = rnd.choice([torch.float16, torch.bfloat16]), rnd.choice([True, False])
+        std = rnd.choice([1e-6, 0.01, 0.5, 30.0, 3000.0])
+        try:
+            run_both(ops, *make_case(T, H, D, bs, NB, dtype, nhd, seed=900 + it, std=std, pad=rnd.choice([0.0, 0.2, 0.6])))
+        except AssertionError as e:
+            raise AssertionError(f"configuration {it}: T={T} H={H} D={D} bs={bs} NB={NB} {dtype} nhd={nhd} std={std}: {e}") from None

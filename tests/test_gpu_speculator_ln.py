@@ -193,3 +193,42 @@ def test_add_ln_act_degenerate_and_errors(ops):
         op(xd, zd.half(), wd, bd, 1.0, 1e-6, "gelu", 1.0)
     with pytest.raises(RuntimeError, match="only fp16 and bf16"):
         op(xd.float(), None, None, None, 1.0, 1e-6, "gelu", 1.0)
+
+
+def test_random_configurations(ops):
+    """Seeded sweep over shapes (vector kernel with 1-8 chunks per lane, element-wise kernel), pitches, optional
+    vectors, activations and output scales, with z passed directly and by token id."""
+    import random
+    rnd = random.Random(23)
+    for it in range(40):
+        rows = rnd.choice([1, 2, 9, 70, 300])
+        hidden = rnd.choice([8, 64, 260, 513, 2880, 4096, 8200, 16384, 40000])
+        dtype = rnd.choice([torch.float16, torch.bfloat16])
+        pad = rnd.choice([0, 0, 8, 3])
+        x, z, w, b = glue_inputs(rows, hidden, dtype, 1500 + it, pad)
+        w, b = (w if rnd.random() < 0.7 else None), (b if rnd.random() < 0.7 else None)
+        use_z = rnd.random() < 0.7
+        act, scale = rnd.choice(["none", "gelu", "gelu_tanh"]), rnd.choice([1.0, 0.70710678, 3.0])
+        alpha, eps = rnd.choice([0.0, 0.35, 2.3716]), rnd.choice([1e-6, 1e-3])
+        d = lambda t: None if t is None else to_device_pitched(t, DEV)
+        try:
+            want = oracle.speculator_add_ln_act(x, z if use_z else None, w, b, alpha, eps, act, scale)
+            got = torch.ops.arctic_inference.speculator_add_ln_act_cuda(d(x), d(z) if use_z else None, d(w), d(b), alpha,
+                                                                       eps, act, scale)
+            assert got.shape == x.shape and got.is_contiguous()
+            assert_close(got, want, RTOL, ATOL, "add_ln_act")
+            if use_z:
+                g = torch.Generator().manual_seed(it)
+                perm = torch.randperm(rows + 2, generator=g)
+                table = torch.zeros(rows + 2, hidden, dtype=dtype)
+                table[perm[:rows]] = z
+                emb = torch.ops.arctic_inference.speculator_embed_add_ln_act_cuda(d(x), table.to(DEV), perm[:rows].to(DEV),
+                                                                                  d(w), d(b), alpha, eps, act, scale)
+                assert torch.equal(emb, got), "z by token id differs from z passed directly"
+            else:
+                plain = ops.speculator_ln(d(x), d(w), d(b), eps)
+                if act == "none" and scale == 1.0:
+                    assert torch.equal(plain, got), "the glue kernel without glue differs from speculator_ln"
+        except AssertionError as e:
+            raise AssertionError(f"configuration {it}: {rows} x {hidden} {dtype} pad={pad} z={use_z} act={act} "
+                                 f"scale={scale} alpha={alpha}: {e}") from None

@@ -82,6 +82,25 @@ def test_argument_errors_return_codes_without_launching(lib):
     assert lib.arctic_reshape_and_cache_flash_bulk(None, None, 0, 0, None, None, None, None, None, 4, 0, 2, 64, 16, 0,
                                                    0, _native.DTYPE_BF16, _native.KV_AUTO, None) == 0
     assert lib.arctic_speculator_ln(None, None, None, None, 0, 128, 128, 1e-6, _native.DTYPE_BF16, None) == 0
+    # the entry points of the "next" rows validate the same way
+    bulk = (None, None, 0, 0, None, None, None, None, None, 4, 2, 2, 64, 16, 0, 0, _native.DTYPE_BF16, _native.KV_AUTO)
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select(*bulk, None, None, None, 0, 0, 4, None)
+    assert rc == 1 and b"null row map" in lib.arctic_last_error()
+    assert lib.arctic_reshape_and_cache_flash_bulk_select(*bulk[:10], 0, *bulk[11:], None, None, None, 0, 0, 4, None) == 0
+    rc = lib.arctic_build_row_map(None, 8, None, 2, 0, None)
+    assert rc == 2 and b"int32 or int64" in lib.arctic_last_error()
+    rc = lib.arctic_build_row_map(None, 8, None, 8, 0, None)
+    assert rc == 1 and b"null" in lib.arctic_last_error()
+    assert lib.arctic_build_row_map(None, 0, None, 8, 0, None) == 0
+    rc = lib.arctic_sum_lstm_embedded(*([None] * 10), 4, 64, 256, 64, 64, 64, 100, 1.0, 1e-6, 1e-6, 0, _native.DTYPE_BF16, None)
+    assert rc == 1 and b"null token ids" in lib.arctic_last_error()
+    rc = lib.arctic_speculator_embed_add_ln_act(None, None, None, None, None, None, 4, 128, 128, 128, 10, 1.0, 1e-6, 1, 1.0,
+                                                _native.DTYPE_BF16, None)
+    assert rc == 1 and b"null embedding table or token ids" in lib.arctic_last_error()
+    rc = lib.arctic_argmax_clamp(None, None, 4, 0, 0, 0, _native.DTYPE_BF16, None)
+    assert rc == 1 and b"cols > 0" in lib.arctic_last_error()
+    rc = lib.arctic_gather_rows(9, None, None, None, None, None, None, 8, 1, 1, 0, None)
+    assert rc == 1 and b"between 0 and 8 tensors" in lib.arctic_last_error()
 
 
 def test_product_never_touches_the_oracle():

@@ -641,6 +641,66 @@ def bench_decode_mix(ops, dev, steps):
             "GBps": round(nbytes / med / 1e3, 1), "hbm_frac": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
 
 
+def bench_speculator_round_glue(ops, dev, steps):
+    """Everything but the matrix products of one proposal round of the LSTM speculator (three heads, 512 rows,
+    width 4096, 128256-entry vocabulary; arctic_speculator.py:733-862): ln0 / sqrt 2, then per head the embedding
+    lookup, the gate update and the token selection.  Once as the reference's caller issues it with its own two
+    operators (speculator_ln + division; embedding + repeat + sum_lstm; argmax + clamp_), once with the fused
+    operators (speculator_ln_scaled; sum_lstm_embedded; speculator_argmax).  The projections and the LM head sit
+    between these steps in the real loop; their outputs are stand-ins here.  One HIP graph each, two rotating sets."""
+    T, Hd, V, heads, sets = 512, 4096, 128256, 3, 2
+    g = torch.Generator(device=dev).manual_seed(9)
+    rn = lambda *s: torch.randn(*s, generator=g, device=dev).to(torch.bfloat16)
+    X = [rn(T, 1, Hd) for _ in range(sets)]
+    S = [[rn(T, 1, 4 * Hd) for _ in range(heads)] for _ in range(sets)]          # projection outputs
+    LOG = [[rn(T, V) for _ in range(heads)] for _ in range(sets)]                # LM-head outputs
+    table = rn(V, Hd)
+    tokens0 = torch.randint(0, V, (T, 1), generator=g, device=dev)
+    cell0 = rn(T, 1, Hd)
+    vec = lambda m: (m + 0.02 * torch.randn(Hd, generator=g, device=dev)).to(torch.bfloat16)
+    w_cell, b_cell, w_state, b_state = vec(1.0), vec(0.0), vec(1.0), vec(0.0)
+    sw = 0.5 ** (0.5 / 3)
+    alpha = ((1 - sw * sw) * (Hd / 2)) ** 0.5 / sw
+    sqrt2 = 2 ** 0.5
+
+    def as_the_caller(i):
+        prev = ops.speculator_ln(X[i], None, None, 1e-6) / sqrt2
+        tokens, cell = tokens0.clamp(0, V - 1), cell0
+        for k in range(heads):
+            z4 = torch.nn.functional.embedding(tokens, table).repeat(1, 1, 4)
+            state, cell = ops.sum_lstm(S[i][k].flatten(0, 1).contiguous(), z4.flatten(0, 1).contiguous(),
+                                       cell.flatten(0, 1).contiguous(), w_cell, b_cell, w_state, b_state, alpha, 1e-6,
+                                       1e-6, False)
+            state, cell = state.reshape(T, 1, Hd), cell.reshape(T, 1, Hd)
+            tokens = torch.argmax(LOG[i][k], dim=-1).reshape(T, -1)
+            tokens.clamp_(0, V - 1)
+        return prev, state, tokens
+
+    def fused(i):
+        prev = ops.speculator_ln_scaled(X[i], None, None, 1e-6, 1.0 / sqrt2)
+        tokens, cell = tokens0, cell0
+        for k in range(heads):
+            state, cell = ops.sum_lstm_embedded(S[i][k], table, tokens, cell, w_cell, b_cell, w_state, b_state, alpha,
+                                                1e-6, 1e-6, False)
+            tokens = ops.speculator_argmax(LOG[i][k], V).reshape(T, -1)
+        return prev, state, tokens
+
+    a, b = as_the_caller(0), fused(0)
+    torch.cuda.synchronize()
+    same = bool(torch.equal(a[2], b[2]) and torch.equal(a[1], b[1]))
+    out = {"outputs_identical": same}
+    for name, fn in (("as_the_reference_caller", as_the_caller), ("fused_operators", fused)):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(sets):
+                fn(i)
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        out[name] = {"us_per_round_graph": round(statistics.median(event_times_us(graph.replay, max(10, steps // 2))) / sets, 2)}
+    return out
+
+
 def placement_sweep(ops, dev, steps):
     """Where the caches sit in HBM against how fast the same launch runs.  The GPU's memory is taken in 32
     chunks of 8 GiB (allocation order follows physical order on an otherwise empty GPU); the 70B-shape
@@ -885,6 +945,9 @@ def main():
         extras["bulk_write_and_select_decode_70b"] = bench_bulk_select(ops, dev, args.steps)
         torch.cuda.empty_cache()
         extras["speculator_argmax_512x128256"] = bench_argmax(ops, dev, args.steps)
+        torch.cuda.empty_cache()
+        extras["speculator_round_without_matrix_products"] = bench_speculator_round_glue(ops, dev, args.steps)
+        torch.cuda.empty_cache()
         extras["suffix_decoding_cpu"] = bench_suffix_decoding()
         log(f"extras: {extras}")
 

@@ -83,7 +83,9 @@ _registered = False
 
 
 def _check(cond: bool, msg: str) -> None:
-    # TORCH_CHECK raises c10::Error, which Python sees as RuntimeError.
+    # TORCH_CHECK raises c10::Error, which Python sees as RuntimeError.  Checks whose message has to be
+    # formatted are written out as `if not (...): raise RuntimeError(f"...")` instead, so that the call
+    # path that succeeds formats nothing: these shims run once per operator call.
     if not cond:
         raise RuntimeError(msg)
 
@@ -105,6 +107,13 @@ def _stream_of(t: torch.Tensor) -> int:
     if _raw_stream is not None:
         return _raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _rows_of(t: torch.Tensor, cols: int) -> torch.Tensor:
+    """``t.view(-1, cols)``; a tensor that is 2-D already is passed through (a view costs a microsecond of
+    host time, and the speculator hands over 2-D tensors).  A single row still goes through view(), which
+    sets its row stride to ``cols`` as the reference's view() does."""
+    return t if t.dim() == 2 and t.size(0) != 1 else t.view(-1, cols)
 
 
 class _on_device_of:
@@ -184,8 +193,8 @@ def _reshape_and_cache_flash_bulk_impl(
     block_stride = key_caches[0].stride(0)
     _check(block_stride == value_caches[0].stride(0),
            "Expected block_stride == value_caches[0].stride(0) to be true")
-    _check(slot_mapping.dtype == torch.int64,
-           f"expected scalar type Long but found {slot_mapping.dtype}")
+    if not (slot_mapping.dtype == torch.int64):
+        raise RuntimeError(f"expected scalar type Long but found {slot_mapping.dtype}")
     # Not checked by the reference (it reinterprets the pointers); a mismatch
     # there corrupts memory, here it is an error.
     _check(values.dtype == keys.dtype, "reshape_and_cache_flash_bulk: keys and values dtype differ")
@@ -195,9 +204,9 @@ def _reshape_and_cache_flash_bulk_impl(
            "reshape_and_cache_flash_bulk: slot_mapping must be 1-D and contiguous")
     cache_elem = key_caches[0].element_size()
     want_elem = keys.element_size() if kv_code == _native.KV_AUTO else 1
-    _check(cache_elem == want_elem and value_caches[0].element_size() == want_elem,
-           f"reshape_and_cache_flash_bulk: cache element size {cache_elem} does not match "
-           f"kv_cache_dtype '{kv_cache_dtype}' (expected {want_elem})")
+    if not (cache_elem == want_elem and value_caches[0].element_size() == want_elem):
+        raise RuntimeError(f"reshape_and_cache_flash_bulk: cache element size {cache_elem} does not match "
+                           f"kv_cache_dtype '{kv_cache_dtype}' (expected {want_elem})")
     if kv_code != _native.KV_AUTO:
         _check({s.dtype for s in k_scales} == {torch.float32} and {s.dtype for s in v_scales} == {torch.float32},
                "reshape_and_cache_flash_bulk: k_scales / v_scales must be float32")
@@ -244,21 +253,25 @@ def _reshape_and_cache_flash_bulk_select_impl(
     fn = "reshape_and_cache_flash_bulk_select"
     num_layers = len(key_caches)
     n_sel = logits_indices.numel()
-    _check(logits_indices.is_cuda and logits_indices.dim() == 1 and logits_indices.dtype in (torch.int32, torch.int64),
-           f"{fn}: logits_indices must be a 1-D int32 or int64 CUDA tensor")
+    if not (
+            logits_indices.is_cuda and logits_indices.dim() == 1 and logits_indices.dtype in (torch.int32, torch.int64)
+    ):
+        raise RuntimeError(f"{fn}: logits_indices must be a 1-D int32 or int64 CUDA tensor")
     for name, src, out in (("k_out", keys, k_out), ("v_out", values, v_out)):
-        _check(out.is_cuda and out.device == src.device and out.dtype == src.dtype,
-               f"{fn}: {name} must be on the device of keys / values and of their type")
-        _check(out.dim() == 2 and out.size(0) >= n_sel, f"{fn}: {name} must be 2-D with at least {n_sel} rows")
-        _check(out.stride(1) == 1, f"{fn}: rows of {name} must be contiguous")
+        if not (out.is_cuda and out.device == src.device and out.dtype == src.dtype):
+            raise RuntimeError(f"{fn}: {name} must be on the device of keys / values and of their type")
+        if not (out.dim() == 2 and out.size(0) >= n_sel):
+            raise RuntimeError(f"{fn}: {name} must be 2-D with at least {n_sel} rows")
+        if not (out.stride(1) == 1):
+            raise RuntimeError(f"{fn}: rows of {name} must be contiguous")
     if num_layers == 0 or slot_mapping.size(0) == 0:
         # nothing is written to a cache, but the selected rows are still wanted
         if n_sel:
             _move_rows_impl("gather_rows", [keys, values], logits_indices, [k_out, v_out], False)
         return
     width = num_layers * int(num_heads) * int(head_size)
-    _check(k_out.size(1) == width and v_out.size(1) == width and keys.size(1) >= width and values.size(1) >= width,
-           f"{fn}: k_out and v_out must have {width} columns (layers x heads x head_size)")
+    if not (k_out.size(1) == width and v_out.size(1) == width and keys.size(1) >= width and values.size(1) >= width):
+        raise RuntimeError(f"{fn}: k_out and v_out must have {width} columns (layers x heads x head_size)")
     # the inverse of logits_indices: which output row, if any, a token goes to
     num_tokens = slot_mapping.size(0)
     row_map = torch.empty(num_tokens, dtype=torch.int64, device=keys.device)
@@ -307,7 +320,8 @@ def _reshape_and_cache_flash_fp4_impl(
     _check(value.dtype == key.dtype and value.shape == key.shape, "reshape_and_cache_flash_fp4: key/value mismatch")
     _check(key.stride(2) == 1 and key.stride(1) == head_size and value.stride(2) == 1 and
            value.stride(1) == head_size, "reshape_and_cache_flash_fp4: heads of a token must be dense")
-    _check(slot_mapping.dtype == torch.int64, f"expected scalar type Long but found {slot_mapping.dtype}")
+    if not (slot_mapping.dtype == torch.int64):
+        raise RuntimeError(f"expected scalar type Long but found {slot_mapping.dtype}")
     _check(all(t.element_size() == 1 for t in (key_cache, value_cache, key_scale_cache, value_scale_cache)),
            "reshape_and_cache_flash_fp4: caches and scale caches must be byte tensors")
     _check(key_cache.size(3) * 2 == head_size and key_cache.stride(3) == 1,
@@ -329,15 +343,21 @@ _ACTIVATIONS = {"none": 0, "gelu": 1, "gelu_tanh": 2}
 def _check_embedding(fn: str, emb_weight: torch.Tensor, token_ids: torch.Tensor, like: torch.Tensor, width: int,
                      rows: int) -> None:
     """An embedding table [V, width] in the activations' type and one int64 token id per row."""
-    _check(emb_weight.is_cuda and token_ids.is_cuda and emb_weight.device == like.device
-           and token_ids.device == like.device, f"{fn}: embedding table and token ids must be on the input's device")
-    _check(emb_weight.dtype == like.dtype, f"{fn}: embedding table dtype must match input dtype")
-    _check(emb_weight.dim() == 2 and emb_weight.size(1) == width and emb_weight.stride(1) == 1,
-           f"{fn}: embedding table must be [num_embeddings, {width}] with contiguous rows")
-    _check(emb_weight.size(0) > 0, f"{fn}: the embedding table has no rows")
-    _check(token_ids.dtype == torch.int64, f"{fn}: token ids must be int64")
-    _check(token_ids.numel() == rows and token_ids.is_contiguous(),
-           f"{fn}: one contiguous token id per row is needed ({token_ids.numel()} ids, {rows} rows)")
+    if not (
+            emb_weight.is_cuda and token_ids.is_cuda and emb_weight.device == like.device
+            and token_ids.device == like.device
+    ):
+        raise RuntimeError(f"{fn}: embedding table and token ids must be on the input's device")
+    if not (emb_weight.dtype == like.dtype):
+        raise RuntimeError(f"{fn}: embedding table dtype must match input dtype")
+    if not (emb_weight.dim() == 2 and emb_weight.size(1) == width and emb_weight.stride(1) == 1):
+        raise RuntimeError(f"{fn}: embedding table must be [num_embeddings, {width}] with contiguous rows")
+    if not (emb_weight.size(0) > 0):
+        raise RuntimeError(f"{fn}: the embedding table has no rows")
+    if not (token_ids.dtype == torch.int64):
+        raise RuntimeError(f"{fn}: token ids must be int64")
+    if not (token_ids.numel() == rows and token_ids.is_contiguous()):
+        raise RuntimeError(f"{fn}: one contiguous token id per row is needed ({token_ids.numel()} ids, {rows} rows)")
 
 
 def _ln_common(fn: str, input: torch.Tensor, z: Optional[torch.Tensor], weight: Optional[torch.Tensor],
@@ -346,13 +366,16 @@ def _ln_common(fn: str, input: torch.Tensor, z: Optional[torch.Tensor], weight: 
     """Argument checks and launch shared by speculator_ln_cuda and speculator_add_ln_act_cuda
     (the checks are those of csrc/custom_ops/speculator_ln.cu:152-201)."""
     lib = _lib()
-    _check(input.dtype in _HALF_DTYPES, f"{fn}: only fp16 and bf16 are supported.")
-    _check(input.is_cuda, f"{fn}: input must be CUDA")
+    if not (input.dtype in _HALF_DTYPES):
+        raise RuntimeError(f"{fn}: only fp16 and bf16 are supported.")
+    if not (input.is_cuda):
+        raise RuntimeError(f"{fn}: input must be CUDA")
     dtype = input.dtype
     hidden = input.size(-1)
-    _check(hidden > 0, f"{fn}: hidden size must be > 0")
-    _check(input.stride(-1) == 1,
-           f"{fn}: last dimension must be contiguous (stride -1 == 1)")
+    if not (hidden > 0):
+        raise RuntimeError(f"{fn}: hidden size must be > 0")
+    if not (input.stride(-1) == 1):
+        raise RuntimeError(f"{fn}: last dimension must be contiguous (stride -1 == 1)")
     if weight is not None:
         _check(weight.is_cuda, "weight must be CUDA")
         _check(weight.dtype == dtype, "weight dtype must match input dtype")
@@ -363,9 +386,10 @@ def _ln_common(fn: str, input: torch.Tensor, z: Optional[torch.Tensor], weight: 
         _check(bias.dtype == dtype, "bias dtype must match input dtype")
         _check(bias.dim() == 1 and bias.numel() == hidden, "bias must be 1D of size hidden")
         _check(bias.is_contiguous(), "bias must be contiguous")
-    _check(activation in _ACTIVATIONS, f"{fn}: activation must be one of {sorted(_ACTIVATIONS)}")
+    if not (activation in _ACTIVATIONS):
+        raise RuntimeError(f"{fn}: activation must be one of {sorted(_ACTIVATIONS)}")
 
-    in_2d = input.view(-1, hidden)
+    in_2d = _rows_of(input, hidden)
     rows = in_2d.size(0)
     row_stride = in_2d.stride(0)
     z_2d = None
@@ -375,13 +399,15 @@ def _ln_common(fn: str, input: torch.Tensor, z: Optional[torch.Tensor], weight: 
         _check(z.is_cuda and z.device == input.device, "z must be CUDA, on the input's device")
         _check(z.dtype == dtype, "z dtype must match input dtype")
         _check(z.shape == input.shape, "z must have the input's shape")
-        _check(z.stride(-1) == 1, f"{fn}: last dimension of z must be contiguous")
-        z_2d = z.view(-1, hidden)
+        if not (z.stride(-1) == 1):
+            raise RuntimeError(f"{fn}: last dimension of z must be contiguous")
+        z_2d = _rows_of(z, hidden)
     out = torch.empty_like(input)
-    out_2d = out.view(-1, hidden)  # rows are written dense, `hidden` apart
+    out_2d = _rows_of(out, hidden)  # rows are written dense, `hidden` apart
     if rows == 0:
         return out
-    _check(out_2d.stride(0) == hidden or rows == 1, f"{fn}: internal - output rows must be dense")
+    if not (out_2d.stride(0) == hidden or rows == 1):
+        raise RuntimeError(f"{fn}: internal - output rows must be dense")
     w_ptr = weight.data_ptr() if weight is not None else None
     b_ptr = bias.data_ptr() if bias is not None else None
     with _on_device_of(input):
@@ -457,20 +483,24 @@ def _sum_lstm_impl(
     else:
         _check(z4_4d.size(-1) == hidden4, "sum_lstm: z4 must have last dim 4*D_gate")
     d_cell = prev_cell_d.size(-1)
-    _check(d_cell == d_gate,
-           f"sum_lstm: prev_cell last dim must equal D_gate. Got {d_cell} vs expected {d_gate}.")
+    if not (d_cell == d_gate):
+        raise RuntimeError(f"sum_lstm: prev_cell last dim must equal D_gate. Got {d_cell} vs expected {d_gate}.")
     _check(states_4d.stride(-1) == 1 and z4_4d.stride(-1) == 1 and prev_cell_d.stride(-1) == 1,
            "sum_lstm: last dimension must be contiguous (stride -1 == 1)")
     for t, name in ((w_cell, "w_cell"), (b_cell, "b_cell"), (w_state, "w_state"), (b_state, "b_state")):
         if t is not None:
-            _check(t.is_cuda, f"sum_lstm: {name} must be CUDA")
-            _check(t.dtype == dtype, f"sum_lstm: {name} dtype mismatch")
-            _check(t.numel() >= d_gate, f"sum_lstm: {name} must have length >= D_eff")
-            _check(t.is_contiguous(), f"sum_lstm: {name} must be contiguous")
+            if not (t.is_cuda):
+                raise RuntimeError(f"sum_lstm: {name} must be CUDA")
+            if not (t.dtype == dtype):
+                raise RuntimeError(f"sum_lstm: {name} dtype mismatch")
+            if not (t.numel() >= d_gate):
+                raise RuntimeError(f"sum_lstm: {name} must have length >= D_eff")
+            if not (t.is_contiguous()):
+                raise RuntimeError(f"sum_lstm: {name} must be contiguous")
 
-    s2 = states_4d.view(-1, hidden4)
-    z2 = z4_4d.view(-1, d_gate if _shared_z else hidden4)
-    p2 = prev_cell_d.view(-1, d_cell)
+    s2 = _rows_of(states_4d, hidden4)
+    z2 = _rows_of(z4_4d, d_gate if _shared_z else hidden4)
+    p2 = _rows_of(prev_cell_d, d_cell)
     rows = s2.size(0)
     if _token_ids is not None:
         _check(p2.size(0) == rows, "sum_lstm: row counts of the inputs differ")
@@ -481,8 +511,9 @@ def _sum_lstm_impl(
     out_cell = torch.empty_strided(p2.size(), p2.stride(), dtype=dtype, device=p2.device)
     out_state = torch.empty_strided(p2.size(), p2.stride(), dtype=dtype, device=p2.device)
     _check(out_cell.stride(0) == out_state.stride(0), "sum_lstm: internal - output strides mismatch")
-    out_cell_orig = out_cell.view(prev_cell_d.size())
-    out_state_orig = out_state.view(prev_cell_d.size())
+    flat = prev_cell_d.dim() == 2
+    out_cell_orig = out_cell if flat else out_cell.view(prev_cell_d.size())
+    out_state_orig = out_state if flat else out_state.view(prev_cell_d.size())
     if rows == 0:
         return out_state_orig, out_cell_orig
 
@@ -526,25 +557,33 @@ def _sum_lstm_embedded_impl(states_4d, emb_weight, token_ids, prev_cell_d, w_cel
 def _move_rows_impl(fn: str, sources: List[torch.Tensor], indices: torch.Tensor, outs: List[torch.Tensor],
                     scatter: bool) -> None:
     lib = _lib()
-    _check(len(sources) == len(outs), f"{fn}: {len(sources)} sources but {len(outs)} outputs")
-    _check(indices.is_cuda and indices.dim() == 1 and indices.is_contiguous(),
-           f"{fn}: indices must be a contiguous 1-D CUDA tensor")
-    _check(indices.dtype in (torch.int32, torch.int64), f"{fn}: indices must be int32 or int64")
+    if not (len(sources) == len(outs)):
+        raise RuntimeError(f"{fn}: {len(sources)} sources but {len(outs)} outputs")
+    if not (indices.is_cuda and indices.dim() == 1 and indices.is_contiguous()):
+        raise RuntimeError(f"{fn}: indices must be a contiguous 1-D CUDA tensor")
+    if not (indices.dtype in (torch.int32, torch.int64)):
+        raise RuntimeError(f"{fn}: indices must be int32 or int64")
     n = indices.numel()
     if n == 0 or not sources:
         return
     indexed_rows = None
     row_bytes, src_stride, dst_stride = [], [], []
     for k, (src, dst) in enumerate(zip(sources, outs)):
-        _check(src.is_cuda and dst.is_cuda and src.device == indices.device and dst.device == indices.device,
-               f"{fn}: tensor {k}: sources, outputs and indices must be on one CUDA device")
-        _check(src.dtype == dst.dtype, f"{fn}: tensor {k}: source and output dtypes differ")
-        _check(src.dim() >= 1 and src.shape[1:] == dst.shape[1:], f"{fn}: tensor {k}: row shapes differ")
-        _check(src.size(0) == 0 or src[0].is_contiguous(), f"{fn}: tensor {k}: source rows must be contiguous")
-        _check(dst.size(0) == 0 or dst[0].is_contiguous(), f"{fn}: tensor {k}: output rows must be contiguous")
+        if not (src.is_cuda and dst.is_cuda and src.device == indices.device and dst.device == indices.device):
+            raise RuntimeError(f"{fn}: tensor {k}: sources, outputs and indices must be on one CUDA device")
+        if not (src.dtype == dst.dtype):
+            raise RuntimeError(f"{fn}: tensor {k}: source and output dtypes differ")
+        if not (src.dim() >= 1 and src.shape[1:] == dst.shape[1:]):
+            raise RuntimeError(f"{fn}: tensor {k}: row shapes differ")
+        if not (src.size(0) == 0 or src[0].is_contiguous()):
+            raise RuntimeError(f"{fn}: tensor {k}: source rows must be contiguous")
+        if not (dst.size(0) == 0 or dst[0].is_contiguous()):
+            raise RuntimeError(f"{fn}: tensor {k}: output rows must be contiguous")
         indexed, linear = (dst, src) if scatter else (src, dst)
-        _check(linear.size(0) >= n, f"{fn}: tensor {k}: {n} indices but only {linear.size(0)} rows")
-        _check(indexed_rows in (None, indexed.size(0)), f"{fn}: indexed tensors differ in their number of rows")
+        if not (linear.size(0) >= n):
+            raise RuntimeError(f"{fn}: tensor {k}: {n} indices but only {linear.size(0)} rows")
+        if not (indexed_rows in (None, indexed.size(0))):
+            raise RuntimeError(f"{fn}: indexed tensors differ in their number of rows")
         indexed_rows = indexed.size(0)
         es = src.element_size()
         row = 1
@@ -583,7 +622,7 @@ def _speculator_argmax_impl(logits: torch.Tensor, max_index: int) -> torch.Tenso
     _check(logits.stride(-1) == 1, "speculator_argmax: last dimension must be contiguous")
     _check(max_index >= 0, "speculator_argmax: max_index must not be negative")
     cols = logits.size(-1)
-    in_2d = logits.view(-1, cols)
+    in_2d = _rows_of(logits, cols)
     rows = in_2d.size(0)
     out = torch.empty(logits.shape[:-1], dtype=torch.int64, device=logits.device)
     if rows == 0:

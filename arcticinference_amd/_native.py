@@ -15,7 +15,7 @@ from typing import Optional
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 _CSRC_DIR = os.path.join(_PKG_DIR, "csrc")
 LIB_BASENAME = "libarctic_mi355x"
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 KV_AUTO, KV_FP8_E4M3, KV_FP8_E5M2 = 0, 1, 2
@@ -83,7 +83,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         i64, i64, i32, i32, vp]  # block_stride, num_blocks, src_dtype, kv_cache_dtype, stream
     lib.arctic_reshape_and_cache_flash_bulk.restype = i32
     lib.arctic_reshape_and_cache_flash_bulk_select.argtypes = lib.arctic_reshape_and_cache_flash_bulk.argtypes[:-1] + [
-        vp, vp, vp, i64, i64, i64, vp]   # row_map, keys_out, values_out, their row strides, num_out_rows, stream
+        vp, vp, i32, i64, i64,   # row_map, indices, index_bytes, num_indices, num_src_rows
+        vp, vp, i64, i64, vp]    # keys_out, values_out, their row strides, stream
     lib.arctic_reshape_and_cache_flash_bulk_select.restype = i32
     lib.arctic_build_row_map.argtypes = [vp, i64, vp, i32, i64, vp]
     lib.arctic_build_row_map.restype = i32

@@ -25,6 +25,7 @@
 #include <algorithm>
 #include <cstdint>
 #include <cstdlib>
+#include <mutex>
 #include <type_traits>
 
 #include "common.hpp"
@@ -65,6 +66,15 @@ struct BulkParams {
   int64_t out_key_stride_bytes;
   int64_t out_value_stride_bytes;
   int64_t num_out_rows;
+  // Workgroups at or beyond main_blocks serve the index list itself: output row j whose index the row map does
+  // not credit to j (a repeated index, or a source row at or beyond num_tokens) is copied straight from source
+  // row indices[j], so the output equals index_select for every index in [0, num_src_rows).  indices == nullptr:
+  // no such workgroups are launched.
+  const void *indices;
+  int64_t num_tokens;
+  int64_t num_src_rows;
+  int64_t main_blocks;
+  int index_is_64;
 };
 
 struct __align__(16) RowDesc {
@@ -118,6 +128,46 @@ __device__ __forceinline__ void emit_chunk(const uint4 &v, const RowDesc &d, int
   }
 }
 
+// Which source row output row j wants, or -1 when the token's own workgroup already copies it (the row map
+// credits the token to j) or the index lies outside the source.
+__device__ __forceinline__ int64_t leftover_source_row(const BulkParams &p, int64_t j) {
+  const int64_t t = p.index_is_64 ? ((const int64_t *)p.indices)[j] : (int64_t)((const int32_t *)p.indices)[j];
+  if (t < 0 || t >= p.num_src_rows) return -1;
+  if (t < p.num_tokens && p.row_map[t] == j) return -1;
+  return t;
+}
+
+// Workgroup `f` beyond the token workgroups: output row j = f / groups_per_token, the same run of layers as a
+// token workgroup would own.  Almost always there is nothing to do (SwiftKV selects each token once).
+template <typename Src, bool kPow2, int kBulkThreads>
+__device__ __forceinline__ void select_leftover_rows(const BulkParams &p, int64_t f) {
+  const int64_t j = f / p.groups_per_token;
+  const int group = (int)(f - j * p.groups_per_token);
+  const int64_t t = leftover_source_row(p, j);
+  if (t < 0) return;
+  const int layer0 = group * p.layers_per_group;
+  const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
+  const int64_t layer_off = (int64_t)layer0 * p.n * Src::kBytes;
+  const char *ksrc = p.keys + t * p.key_stride_bytes + layer_off;
+  const char *vsrc = p.values + t * p.value_stride_bytes + layer_off;
+  char *kout = p.keys_out + j * p.out_key_stride_bytes + layer_off;
+  char *vout = p.values_out + j * p.out_value_stride_bytes + layer_off;
+  const int cpr = p.chunks_per_row;
+  const int total = 2 * nlayers * cpr;
+  for (int c = threadIdx.x; c < total; c += kBulkThreads) {
+    int r, col;
+    if constexpr (kPow2) {
+      r = c >> p.chunk_shift;
+      col = c & (cpr - 1);
+    } else {
+      r = c / cpr;
+      col = c - r * cpr;
+    }
+    const int64_t off = ((int64_t)(r >> 1) * cpr + col) * 16;
+    store16_stream(((r & 1) ? vout : kout) + off, load16_stream(((r & 1) ? vsrc : ksrc) + off));
+  }
+}
+
 // kBulkThreads x kUnroll 16-byte chunks form one batch of a workgroup.  Two shapes
 // are built: 512 x 2 (a workgroup moves two batches or more) and 256 x 4 (decode:
 // few tokens, a single batch per workgroup).
@@ -129,6 +179,12 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
 
   __shared__ RowDesc rows[2 * kLayersPerLaunch];
 
+  if constexpr (kSelect) {
+    if (blockIdx.x >= p.main_blocks) {  // uniform over the workgroup, before any barrier
+      select_leftover_rows<Src, kPow2, kBulkThreads>(p, blockIdx.x - p.main_blocks);
+      return;
+    }
+  }
   const int64_t token = blockIdx.x / (unsigned)p.groups_per_token;
   const int group = blockIdx.x - (unsigned)token * (unsigned)p.groups_per_token;
   const int layer0 = group * p.layers_per_group;
@@ -243,6 +299,24 @@ template <typename SrcElem, typename Dst>
 __global__ __launch_bounds__(kScalarThreads) void kv_write_bulk_scalar_kernel(
     const BulkParams p, const LayerTables tab, const int src_dtype) {
   constexpr bool kCopy = std::is_same<Dst, Copy>::value;
+  if (blockIdx.x >= p.main_blocks) {  // the index list's own workgroups (select variant only)
+    const int64_t f = blockIdx.x - p.main_blocks;
+    const int64_t j = f / p.groups_per_token;
+    const int group = (int)(f - j * p.groups_per_token);
+    const int64_t t = leftover_source_row(p, j);
+    if (t < 0) return;
+    const int layer0 = group * p.layers_per_group;
+    const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
+    const SrcElem *ks = reinterpret_cast<const SrcElem *>(p.keys + t * p.key_stride_bytes);
+    const SrcElem *vs = reinterpret_cast<const SrcElem *>(p.values + t * p.value_stride_bytes);
+    SrcElem *ko = reinterpret_cast<SrcElem *>(p.keys_out + j * p.out_key_stride_bytes);
+    SrcElem *vo = reinterpret_cast<SrcElem *>(p.values_out + j * p.out_value_stride_bytes);
+    for (int64_t i = (int64_t)layer0 * p.n + threadIdx.x; i < (int64_t)(layer0 + nlayers) * p.n; i += kScalarThreads) {
+      ko[i] = ks[i];
+      vo[i] = vs[i];
+    }
+    return;
+  }
   const int64_t token = blockIdx.x / (unsigned)p.groups_per_token;
   const int group = blockIdx.x - (unsigned)token * (unsigned)p.groups_per_token;
   const int layer0 = group * p.layers_per_group;
@@ -368,6 +442,9 @@ struct SelectArgs {
   int64_t out_key_stride;    // elements
   int64_t out_value_stride;
   int64_t num_out_rows;
+  const void *indices;       // the list row_map inverts (num_out_rows entries), or nullptr
+  int index_bytes;
+  int64_t num_src_rows;      // rows of keys / values an index may name
 };
 
 static int bulk_entry(const char *fn, const void *keys, const void *values, int64_t key_stride, int64_t value_stride,
@@ -398,6 +475,13 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
   if (sel.row_map && sel.num_out_rows == 0) sel.row_map = nullptr;   // no row to copy to: the plain write
   if (sel.row_map && (!sel.keys_out || !sel.values_out))
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null keys_out or values_out", fn);
+  if (sel.row_map && sel.indices) {
+    if (sel.index_bytes != 4 && sel.index_bytes != 8)
+      return fail(ARCTIC_ERR_UNSUPPORTED, "%s: indices must be int32 or int64", fn);
+    if (sel.num_src_rows < num_tokens)
+      return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: keys / values have fewer rows (%lld) than slot_mapping (%lld)", fn,
+                  (long long)sel.num_src_rows, (long long)num_tokens);
+  }
   const bool quant = kv_cache_dtype != ARCTIC_KV_AUTO;
   if (quant && (!k_scale_ptrs || !v_scale_ptrs))
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: fp8 cache needs k_scales and v_scales", fn);
@@ -447,6 +531,10 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
     p.out_key_stride_bytes = sel.out_key_stride * es;
     p.out_value_stride_bytes = sel.out_value_stride * es;
     p.num_out_rows = sel.row_map ? sel.num_out_rows : 0;
+    p.indices = sel.row_map ? sel.indices : nullptr;
+    p.index_is_64 = sel.index_bytes == 8;
+    p.num_tokens = num_tokens;
+    p.num_src_rows = sel.num_src_rows;
     p.key_stride_bytes = key_stride * es;
     p.value_stride_bytes = value_stride * es;
     p.block_stride = block_stride;
@@ -486,7 +574,8 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
 #endif
     p.layers_per_group = (count + groups - 1) / groups;
     p.groups_per_token = (count + p.layers_per_group - 1) / p.layers_per_group;
-    const int64_t grid = num_tokens * p.groups_per_token;
+    p.main_blocks = num_tokens * p.groups_per_token;
+    const int64_t grid = p.main_blocks + (p.indices ? p.num_out_rows * p.groups_per_token : 0);
     if (grid > 0x7fffffffLL)
       return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: too many tokens (%lld)", fn, (long long)num_tokens);
 
@@ -508,7 +597,7 @@ extern "C" int arctic_reshape_and_cache_flash_bulk(
     const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads,
     int head_size, int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype,
     int kv_cache_dtype, void *stream) {
-  const SelectArgs none = {nullptr, nullptr, nullptr, 0, 0, 0};
+  const SelectArgs none = {nullptr, nullptr, nullptr, 0, 0, 0, nullptr, 0, 0};
   return bulk_entry("reshape_and_cache_flash_bulk", keys, values, key_stride, value_stride, key_cache_ptrs,
                     value_cache_ptrs, k_scale_ptrs, v_scale_ptrs, slot_mapping, num_tokens, num_layers, num_heads,
                     head_size, block_size, block_stride, num_blocks, src_dtype, kv_cache_dtype, none, stream);
@@ -520,19 +609,20 @@ extern "C" int arctic_reshape_and_cache_flash_bulk_select(
     const float *const *k_scale_ptrs, const float *const *v_scale_ptrs,
     const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads,
     int head_size, int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype,
-    int kv_cache_dtype, const int64_t *row_map, void *keys_out, void *values_out,
-    int64_t out_key_stride, int64_t out_value_stride, int64_t num_out_rows, void *stream) {
+    int kv_cache_dtype, const int64_t *row_map, const void *indices, int index_bytes, int64_t num_indices,
+    int64_t num_src_rows, void *keys_out, void *values_out, int64_t out_key_stride, int64_t out_value_stride,
+    void *stream) {
   const char *fn = "reshape_and_cache_flash_bulk_select";
   if (num_layers != 0 && num_tokens != 0 && !row_map) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null row map", fn);
-  const SelectArgs sel = {row_map, keys_out, values_out, out_key_stride, out_value_stride, num_out_rows};
+  const SelectArgs sel = {row_map, keys_out, values_out, out_key_stride, out_value_stride, num_indices,
+                          indices, index_bytes, num_src_rows};
   return bulk_entry(fn, keys, values, key_stride, value_stride, key_cache_ptrs, value_cache_ptrs, k_scale_ptrs,
                     v_scale_ptrs, slot_mapping, num_tokens, num_layers, num_heads, head_size, block_size, block_stride,
                     num_blocks, src_dtype, kv_cache_dtype, sel, stream);
 }
 
-extern "C" int arctic_build_row_map(int64_t *row_map, int64_t num_tokens, const void *indices, int index_bytes,
-                                    int64_t num_indices, void *stream) {
-  const char *fn = "build_row_map";
+static int build_row_map(const char *fn, int64_t *row_map, int64_t num_tokens, const void *indices, int index_bytes,
+                         int64_t num_indices, void *stream) {
   if (index_bytes != 4 && index_bytes != 8) return fail(ARCTIC_ERR_UNSUPPORTED, "%s: indices must be int32 or int64", fn);
   if (num_tokens < 0 || num_indices < 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: negative size", fn);
   if (num_tokens == 0) return ARCTIC_OK;
@@ -545,4 +635,9 @@ extern "C" int arctic_build_row_map(int64_t *row_map, int64_t num_tokens, const 
     hipLaunchKernelGGL(build_row_map_kernel<int32_t>, dim3(1), dim3(1024), 0, s, row_map, num_tokens,
                        (const int32_t *)indices, num_indices);
   return check_launch(fn);
+}
+
+extern "C" int arctic_build_row_map(int64_t *row_map, int64_t num_tokens, const void *indices, int index_bytes,
+                                    int64_t num_indices, void *stream) {
+  return build_row_map("build_row_map", row_map, num_tokens, indices, index_bytes, num_indices, stream);
 }

@@ -171,7 +171,7 @@ def _reshape_and_cache_flash_bulk_impl(
     v_scales: List[torch.Tensor],
     num_heads: int,
     head_size: int,
-    _select: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor, int]] = None,
+    _select: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]] = None,
 ) -> None:
     """Host side of the bulk KV write; follows the reference's launcher
     (csrc/custom_ops/reshape_and_cache_flash_bulk.cu:77-144) up to the point
@@ -210,10 +210,23 @@ def _reshape_and_cache_flash_bulk_impl(
     if kv_code != _native.KV_AUTO:
         _check({s.dtype for s in k_scales} == {torch.float32} and {s.dtype for s in v_scales} == {torch.float32},
                "reshape_and_cache_flash_bulk: k_scales / v_scales must be float32")
-    devices = {t.device for t in key_caches}
-    devices.update(t.device for t in value_caches)
-    devices.update((values.device, slot_mapping.device, keys.device))
+    # every layer's K and V view must look like layer 0's: the kernel takes one block stride, block size and
+    # number of blocks for all of them
+    geometry = {(t.dtype, t.stride(0), t.size(0), t.size(1), t.device) for t in key_caches}
+    geometry.update((t.dtype, t.stride(0), t.size(0), t.size(1), t.device) for t in value_caches)
+    if not (len(geometry) == 1):
+        raise RuntimeError("reshape_and_cache_flash_bulk: key and value caches of all layers must share dtype, "
+                           "block stride, number of blocks, block size and device")
+    devices = {key_caches[0].device, values.device, slot_mapping.device, keys.device}
+    if kv_code != _native.KV_AUTO:
+        devices.update(s.device for s in k_scales)
+        devices.update(s.device for s in v_scales)
     _check(len(devices) == 1, "reshape_and_cache_flash_bulk: all tensors must be on the same device")
+    width = num_layers * int(num_heads) * int(head_size)
+    if not (keys.dim() == 2 and values.dim() == 2 and keys.size(0) >= num_tokens and values.size(0) >= num_tokens
+            and keys.size(1) >= width and values.size(1) >= width):
+        raise RuntimeError(f"reshape_and_cache_flash_bulk: keys and values must be 2-D with at least {num_tokens} rows "
+                           f"(one per slot) and {width} columns (layers x heads x head_size)")
 
     common = (keys.data_ptr(), values.data_ptr(), key_stride, value_stride,
               _ptr_table(key_caches), _ptr_table(value_caches),
@@ -224,10 +237,10 @@ def _reshape_and_cache_flash_bulk_impl(
         if _select is None:
             rc = lib.arctic_reshape_and_cache_flash_bulk(*common, _stream_of(keys))
         else:
-            row_map, k_out, v_out, out_rows = _select
+            row_map, idx, k_out, v_out = _select
             rc = lib.arctic_reshape_and_cache_flash_bulk_select(
-                *common, row_map.data_ptr(), k_out.data_ptr(), v_out.data_ptr(), k_out.stride(0), v_out.stride(0),
-                out_rows, _stream_of(keys))
+                *common, row_map.data_ptr(), idx.data_ptr(), idx.element_size(), idx.numel(), keys.size(0),
+                k_out.data_ptr(), v_out.data_ptr(), k_out.stride(0), v_out.stride(0), _stream_of(keys))
     _native.check(rc)
 
 
@@ -249,7 +262,9 @@ def _reshape_and_cache_flash_bulk_select_impl(
     """The bulk KV write and, in the same pass over keys / values, ``k_out[j] = keys[logits_indices[j]]`` and
     ``v_out[j] = values[logits_indices[j]]``: the two largest index_select calls of swiftkv_select
     (arctic_inference/vllm/swiftkv/llama_swiftkv.py:663-679) without a second read of k_states / v_states.
-    ``logits_indices`` must not repeat an index (SwiftKV's never do: one per request)."""
+    The selected rows equal ``torch.index_select`` for every index in ``[0, keys.size(0))``, repeated ones
+    included (SwiftKV's never repeat: one per request); a row whose index lies outside that range is left as it
+    was, where index_select would raise."""
     fn = "reshape_and_cache_flash_bulk_select"
     num_layers = len(key_caches)
     n_sel = logits_indices.numel()
@@ -264,24 +279,28 @@ def _reshape_and_cache_flash_bulk_select_impl(
             raise RuntimeError(f"{fn}: {name} must be 2-D with at least {n_sel} rows")
         if not (out.stride(1) == 1):
             raise RuntimeError(f"{fn}: rows of {name} must be contiguous")
-    if num_layers == 0 or slot_mapping.size(0) == 0:
-        # nothing is written to a cache, but the selected rows are still wanted
-        if n_sel:
-            _move_rows_impl("gather_rows", [keys, values], logits_indices, [k_out, v_out], False)
-        return
+    if num_layers == 0:
+        return  # no layer, so no column to write or to select (reshape_and_cache_flash_bulk.cu:87-89)
     width = num_layers * int(num_heads) * int(head_size)
     if not (k_out.size(1) == width and v_out.size(1) == width and keys.size(1) >= width and values.size(1) >= width):
         raise RuntimeError(f"{fn}: k_out and v_out must have {width} columns (layers x heads x head_size)")
-    # the inverse of logits_indices: which output row, if any, a token goes to
-    num_tokens = slot_mapping.size(0)
-    row_map = torch.empty(num_tokens, dtype=torch.int64, device=keys.device)
+    if not (keys.size(0) == values.size(0)):
+        raise RuntimeError(f"{fn}: keys and values differ in their number of rows")
     idx = logits_indices if logits_indices.is_contiguous() else logits_indices.contiguous()
+    num_tokens = slot_mapping.size(0)
+    if num_tokens == 0:
+        # nothing is written to a cache, but the selected rows (of the first `width` columns) are still wanted
+        if n_sel:
+            _move_rows_impl("gather_rows", [keys[:, :width], values[:, :width]], idx, [k_out, v_out], False)
+        return
+    # the inverse of logits_indices: which output row, if any, a token goes to
+    row_map = torch.empty(num_tokens, dtype=torch.int64, device=keys.device)
     with _on_device_of(keys):
         rc = _lib().arctic_build_row_map(row_map.data_ptr(), num_tokens, idx.data_ptr(), idx.element_size(), n_sel,
                                          _stream_of(keys))
     _native.check(rc)
     _reshape_and_cache_flash_bulk_impl(keys, values, key_caches, value_caches, slot_mapping, kv_cache_dtype, k_scales,
-                                       v_scales, num_heads, head_size, _select=(row_map, k_out, v_out, n_sel))
+                                       v_scales, num_heads, head_size, _select=(row_map, idx, k_out, v_out))
 
 
 def _reshape_and_cache_flash_fp4_impl(
@@ -795,8 +814,9 @@ def reshape_and_cache_flash_bulk_select(
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """``reshape_and_cache_flash_bulk(...)`` followed by ``torch.index_select(keys, 0, logits_indices,
     out=k_out[:n])`` and the same for values (arctic_inference/vllm/swiftkv/llama_swiftkv.py:617-622, 663-679),
-    with keys / values read once for both.  Returns ``(k_out[:n], v_out[:n])``.  ``logits_indices`` must not
-    repeat an index."""
+    with keys / values read once for both.  Returns ``(k_out[:n], v_out[:n])``.  Indices may repeat; a row whose
+    index lies outside ``[0, keys.size(0))`` is left as it was (index_select would raise).  With no layers there is
+    no column to select and the call does nothing."""
     _call("reshape_and_cache_flash_bulk_select", keys, values, key_caches, value_caches, slot_mapping, kv_cache_dtype,
           k_scales, v_scales, num_heads, head_size, logits_indices, k_out, v_out)
     n = logits_indices.numel()

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define ARCTIC_ABI_VERSION 1
+#define ARCTIC_ABI_VERSION 2
 
 /* element types of source / activation tensors */
 #define ARCTIC_DTYPE_F32 0
@@ -120,9 +120,16 @@ int arctic_build_row_map(int64_t *row_map, int64_t num_tokens, const void *indic
  * with row_map the inverse of logits_indices (row_map[logits_indices[j]] = j, -1 elsewhere), so k_states and
  * v_states are read once for both steps.  No single function of the reference corresponds to it.
  *
- *   row_map            device int64[num_tokens]; negative or >= num_out_rows: the token is not copied.
- *                      A token is copied whether or not its slot is padding.
- *   keys_out, values_out   device; rows of num_layers*n elements of src_dtype, out_*_stride ELEMENTS apart
+ *   row_map            device int64[num_tokens], as arctic_build_row_map leaves it for `indices`; negative or
+ *                      >= num_indices: the token is not copied.  A token is copied whether or not its slot is padding.
+ *   indices            device, num_indices entries of index_bytes (4 or 8) each, or NULL.  With the list given,
+ *                      the result is torch.index_select for EVERY index in [0, num_src_rows): output rows that
+ *                      the row map cannot serve (an index that is repeated, or one at or beyond num_tokens) are
+ *                      copied from the source by extra workgroups of the same launch.  Output rows whose index
+ *                      lies outside [0, num_src_rows) are left as they were (index_select would raise).
+ *                      NULL: the caller vouches that the indices are distinct and below num_tokens.
+ *   num_src_rows       rows of keys / values (>= num_tokens)
+ *   keys_out, values_out   device; num_indices rows of num_layers*n elements of src_dtype, out_*_stride ELEMENTS apart
  *   other arguments as arctic_reshape_and_cache_flash_bulk
  */
 int arctic_reshape_and_cache_flash_bulk_select(
@@ -131,8 +138,9 @@ int arctic_reshape_and_cache_flash_bulk_select(
     const float *const *k_scale_ptrs, const float *const *v_scale_ptrs,
     const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads,
     int head_size, int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype,
-    int kv_cache_dtype, const int64_t *row_map, void *keys_out, void *values_out,
-    int64_t out_key_stride, int64_t out_value_stride, int64_t num_out_rows, void *stream);
+    int kv_cache_dtype, const int64_t *row_map, const void *indices, int index_bytes, int64_t num_indices,
+    int64_t num_src_rows, void *keys_out, void *values_out, int64_t out_key_stride, int64_t out_value_stride,
+    void *stream);
 
 /*
  * NVFP4-style KV-cache write for ONE layer: e2m1 values, two per byte (first element

@@ -54,7 +54,7 @@ def test_no_torch_dependency():
 
 def test_header_compiles_as_plain_c(tmp_path):
     src = tmp_path / "t.c"
-    src.write_text('#include "arctic_mi355x.h"\nint main(void) { return ARCTIC_ABI_VERSION == 1 ? 0 : 1; }\n')
+    src.write_text('#include "arctic_mi355x.h"\nint main(void) { return ARCTIC_ABI_VERSION >= 1 ? 0 : 1; }\n')
     subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), "-c", str(src), "-o",
                     str(tmp_path / "t.o")], check=True)
 
@@ -84,9 +84,10 @@ def test_argument_errors_return_codes_without_launching(lib):
     assert lib.arctic_speculator_ln(None, None, None, None, 0, 128, 128, 1e-6, _native.DTYPE_BF16, None) == 0
     # the entry points of the "next" rows validate the same way
     bulk = (None, None, 0, 0, None, None, None, None, None, 4, 2, 2, 64, 16, 0, 0, _native.DTYPE_BF16, _native.KV_AUTO)
-    rc = lib.arctic_reshape_and_cache_flash_bulk_select(*bulk, None, None, None, 0, 0, 4, None)
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select(*bulk, None, None, 8, 4, 4, None, None, 0, 0, None)
     assert rc == 1 and b"null row map" in lib.arctic_last_error()
-    assert lib.arctic_reshape_and_cache_flash_bulk_select(*bulk[:10], 0, *bulk[11:], None, None, None, 0, 0, 4, None) == 0
+    assert lib.arctic_reshape_and_cache_flash_bulk_select(*bulk[:10], 0, *bulk[11:], None, None, 8, 4, 4, None, None, 0, 0,
+                                                          None) == 0
     rc = lib.arctic_build_row_map(None, 8, None, 2, 0, None)
     assert rc == 2 and b"int32 or int64" in lib.arctic_last_error()
     rc = lib.arctic_build_row_map(None, 8, None, 8, 0, None)

@@ -109,6 +109,38 @@ def test_random_configurations(ops):
             raise AssertionError(f"configuration {it}: {cfg}, {n_sel} selected: {e}") from None
 
 
+@pytest.mark.parametrize("kv", ["auto", "fp8"])
+@pytest.mark.parametrize("shape", ["vector", "element_wise"])
+def test_repeated_indices_and_rows_beyond_the_slot_mapping_match_index_select(ops, kv, shape):
+    # index_select semantics for every index inside keys / values: an index named twice fills both output rows, and
+    # a source row at or beyond slot_mapping.size(0) (keys may hold more rows than there are slots) is copied too
+    H, D, pad = (8, 128, 0) if shape == "vector" else (3, 20, 3)
+    case = make_bulk_case(T=120, L=5, H=H, D=D, bs=16, NB=16, kv_cache_dtype=kv, seed=49, pad_fraction=0.2, key_pad=pad)
+    case["slot_mapping"] = case["slot_mapping"][:100].contiguous()
+    idx = torch.tensor([5, 5, 99, 100, 119, 5, 0, 118, 99, 7, 7])
+    run_select(ops, case, idx, 16, out_pad=pad and 1)
+    # more layers than one launch holds, every index repeated
+    case = make_bulk_case(T=9, L=70, H=2, D=64, bs=16, NB=4, kv_cache_dtype=kv, seed=50)
+    run_select(ops, case, torch.tensor([8, 8, 0, 0, 3, 3, 3]), 7)
+
+
+def test_indices_outside_the_source_leave_their_rows_untouched(ops):
+    case = make_bulk_case(T=40, L=3, H=8, D=128, bs=16, NB=4, kv_cache_dtype="fp8", seed=51)
+    d = bulk_case_to(case, DEV)
+    width = case["keys"].size(1)
+    k_out = torch.full((6, width), 3.0, dtype=torch.bfloat16, device=DEV)
+    v_out = torch.full((6, width), 3.0, dtype=torch.bfloat16, device=DEV)
+    idx = torch.tensor([2, 40, -1, 39, 1 << 40, 2], device=DEV)
+    ops.reshape_and_cache_flash_bulk_select(*bulk_args(d), idx, k_out, v_out)
+    torch.cuda.synchronize()
+    oracle.reshape_and_cache_flash_bulk(*bulk_args(case))
+    assert_bulk_equal(d["bufs"], case["bufs"])
+    for out, src in ((k_out, case["keys"]), (v_out, case["values"])):
+        out = out.cpu()
+        assert torch.equal(out[0], src[2]) and torch.equal(out[5], src[2]) and torch.equal(out[3], src[39])
+        assert (out[[1, 2, 4]] == 3.0).all()
+
+
 def test_empty_selection_and_no_layers(ops):
     case = make_bulk_case(T=64, L=4, H=8, D=128, bs=16, NB=8, kv_cache_dtype="fp8", seed=46)
     run_select(ops, case, torch.empty(0, dtype=torch.int64), 4)
@@ -116,9 +148,18 @@ def test_empty_selection_and_no_layers(ops):
     k_out = torch.zeros(8, 4 * 1024, dtype=torch.bfloat16, device=DEV)
     v_out = torch.zeros_like(k_out)
     idx = torch.tensor([5, 9], device=DEV)
-    k_sel, v_sel = ops.reshape_and_cache_flash_bulk_select(d["keys"], d["values"], [], [], d["slot_mapping"], "fp8", [], [],
+    # no layers: no columns, nothing is written anywhere (whatever the width of the buffers)
+    ops.reshape_and_cache_flash_bulk_select(d["keys"], d["values"], [], [], d["slot_mapping"], "fp8", [], [], 8, 128, idx,
+                                            k_out[:, :100], v_out)
+    assert not k_out.any() and not v_out.any()
+    # no slots: no cache row is written, the first layers x heads x head_size columns are still selected
+    wide = torch.cat([d["keys"], d["keys"][:, :8]], dim=1)
+    before = [b.clone() for b in d["bufs"]]
+    k_sel, v_sel = ops.reshape_and_cache_flash_bulk_select(wide, d["values"], d["key_caches"], d["value_caches"],
+                                                           d["slot_mapping"][:0], "fp8", d["k_scales"], d["v_scales"],
                                                            8, 128, idx, k_out, v_out)
     assert torch.equal(k_sel, d["keys"][idx]) and torch.equal(v_sel, d["values"][idx])
+    assert all(torch.equal(a.view(torch.uint8), b.view(torch.uint8)) for a, b in zip(d["bufs"], before))
 
 
 def test_row_map_helper_and_out_of_range_rows_through_the_c_abi(ops):
@@ -139,7 +180,7 @@ def test_row_map_helper_and_out_of_range_rows_through_the_c_abi(ops):
     rc = lib.arctic_reshape_and_cache_flash_bulk_select(
         d["keys"].data_ptr(), d["values"].data_ptr(), 256, 256, tab(d["key_caches"]), tab(d["value_caches"]), None, None,
         d["slot_mapping"].data_ptr(), 10, 2, 2, 64, 16, d["key_caches"][0].stride(0), 2, _native.DTYPE_BF16,
-        _native.KV_AUTO, row_map.data_ptr(), k_out.data_ptr(), v_out.data_ptr(), 256, 256, 2, stream)
+        _native.KV_AUTO, row_map.data_ptr(), None, 0, 2, 10, k_out.data_ptr(), v_out.data_ptr(), 256, 256, stream)
     assert rc == 0, lib.arctic_last_error()
     torch.cuda.synchronize()
     oracle.reshape_and_cache_flash_bulk(*bulk_args(case))

@@ -26,6 +26,7 @@ EXPORTED_SYMBOLS = (
     "arctic_last_error",
     "arctic_reshape_and_cache_flash_bulk",
     "arctic_reshape_and_cache_flash_bulk_select",
+    "arctic_reshape_and_cache_flash_bulk_select_static",
     "arctic_build_row_map",
     "arctic_reshape_and_cache_flash_fp4",
     "arctic_speculator_ln",
@@ -86,6 +87,11 @@ def _declare(lib: ctypes.CDLL) -> None:
         vp, vp, i32, i64, i64,   # row_map, indices, index_bytes, num_indices, num_src_rows
         vp, vp, i64, i64, vp]    # keys_out, values_out, their row strides, stream
     lib.arctic_reshape_and_cache_flash_bulk_select.restype = i32
+    lib.arctic_reshape_and_cache_flash_bulk_select_static.argtypes = (
+        lib.arctic_reshape_and_cache_flash_bulk.argtypes[:-1] + [
+            vp, i32, i64, i64,       # indices, index_bytes, num_indices, num_src_rows
+            vp, vp, i64, i64, vp])   # keys_out, values_out, their row strides, stream
+    lib.arctic_reshape_and_cache_flash_bulk_select_static.restype = i32
     lib.arctic_build_row_map.argtypes = [vp, i64, vp, i32, i64, vp]
     lib.arctic_build_row_map.restype = i32
     lib.arctic_reshape_and_cache_flash_fp4.argtypes = [

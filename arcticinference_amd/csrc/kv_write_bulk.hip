@@ -641,3 +641,64 @@ extern "C" int arctic_build_row_map(int64_t *row_map, int64_t num_tokens, const 
                                     int64_t num_indices, void *stream) {
   return build_row_map("build_row_map", row_map, num_tokens, indices, index_bytes, num_indices, stream);
 }
+
+// ---- the select variant that allocates nothing ---------------------------------------------------------------
+// The row map of arctic_reshape_and_cache_flash_bulk_select_static lives in this array instead of a workspace
+// the caller brings in: 8 bytes per token, 2 MiB, held by every GPU the library has run on until the process
+// ends.  In host code `scratch` is only a handle for the symbol; the array's address on a device comes from
+// hipGetSymbolAddress with that device current, is looked up once per device and is what the kernels receive.
+static __device__ __align__(256) int64_t scratch[ARCTIC_SELECT_STATIC_MAX_TOKENS];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+int64_t *g_scratch_ptr[kMaxDevices];  // this device's copy of `scratch`, nullptr until first asked for
+}  // namespace
+
+static int scratch_on_current_device(const char *fn, int64_t **out) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return fail(ARCTIC_ERR_LAUNCH, "%s: hipGetDevice failed: %s", fn, hipGetErrorString(err));
+  if (dev < 0 || dev >= kMaxDevices) return fail(ARCTIC_ERR_UNSUPPORTED, "%s: device index %d not supported", fn, dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || !ptr)
+      return fail(ARCTIC_ERR_LAUNCH, "%s: hipGetSymbolAddress failed on device %d: %s", fn, dev, hipGetErrorString(err));
+    g_scratch_ptr[dev] = (int64_t *)ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return ARCTIC_OK;
+}
+
+extern "C" int arctic_reshape_and_cache_flash_bulk_select_static(
+    const void *keys, const void *values, int64_t key_stride, int64_t value_stride,
+    const void *const *key_cache_ptrs, const void *const *value_cache_ptrs,
+    const float *const *k_scale_ptrs, const float *const *v_scale_ptrs,
+    const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads,
+    int head_size, int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype,
+    int kv_cache_dtype, const void *indices, int index_bytes, int64_t num_indices, int64_t num_src_rows,
+    void *keys_out, void *values_out, int64_t out_key_stride, int64_t out_value_stride, void *stream) {
+  const char *fn = "reshape_and_cache_flash_bulk_select_static";
+  if (num_tokens > ARCTIC_SELECT_STATIC_MAX_TOKENS)
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT,
+                "%s: num_tokens=%lld exceeds the %d tokens the static row map holds; use "
+                "arctic_reshape_and_cache_flash_bulk_select with a row map of the caller's",
+                fn, (long long)num_tokens, ARCTIC_SELECT_STATIC_MAX_TOKENS);
+  if (num_indices < 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: negative number of indices", fn);
+  if (num_indices > 0 && !indices) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null indices", fn);
+  int64_t *row_map = nullptr;
+  if (num_layers != 0 && num_tokens > 0 && num_indices > 0) {
+    int rc = scratch_on_current_device(fn, &row_map);
+    if (rc) return rc;
+    // every entry below num_tokens is rewritten, so nothing of an earlier call is seen
+    rc = build_row_map(fn, row_map, num_tokens, indices, index_bytes, num_indices, stream);
+    if (rc) return rc;
+  }
+  const SelectArgs sel = {row_map, keys_out, values_out, out_key_stride, out_value_stride, num_indices,
+                          indices, index_bytes, num_src_rows};
+  return bulk_entry(fn, keys, values, key_stride, value_stride, key_cache_ptrs, value_cache_ptrs, k_scale_ptrs,
+                    v_scale_ptrs, slot_mapping, num_tokens, num_layers, num_heads, head_size, block_size, block_stride,
+                    num_blocks, src_dtype, kv_cache_dtype, sel, stream);
+}

@@ -142,6 +142,34 @@ int arctic_reshape_and_cache_flash_bulk_select(
     int64_t num_src_rows, void *keys_out, void *values_out, int64_t out_key_stride, int64_t out_value_stride,
     void *stream);
 
+/* Most tokens one call of arctic_reshape_and_cache_flash_bulk_select_static accepts. */
+#define ARCTIC_SELECT_STATIC_MAX_TOKENS 262144
+
+/*
+ * arctic_reshape_and_cache_flash_bulk_select for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The same result as arctic_build_row_map followed by arctic_reshape_and_cache_flash_bulk_select, but the row
+ * map is kept in a device array inside the library (8 bytes x ARCTIC_SELECT_STATIC_MAX_TOKENS = 2 MiB on each
+ * GPU the library runs on, held until the process ends) instead of a workspace of the caller's.  The call
+ * allocates and frees nothing; it enqueues two kernels on `stream`.
+ *
+ *   num_tokens   at most ARCTIC_SELECT_STATIC_MAX_TOKENS, else ARCTIC_ERR_INVALID_ARGUMENT
+ *   indices      device, num_indices entries of index_bytes (4 or 8) each; required when num_indices > 0
+ *   other arguments as arctic_reshape_and_cache_flash_bulk_select
+ *
+ * All calls on one GPU share that GPU's array: calls that may run at the same time on one GPU (different
+ * streams without an ordering between them) race on it and must use the workspace form instead.  The first call
+ * on a device looks the array's address up (hipGetSymbolAddress); make that call outside graph capture.
+ */
+int arctic_reshape_and_cache_flash_bulk_select_static(
+    const void *keys, const void *values, int64_t key_stride, int64_t value_stride,
+    const void *const *key_cache_ptrs, const void *const *value_cache_ptrs,
+    const float *const *k_scale_ptrs, const float *const *v_scale_ptrs,
+    const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads,
+    int head_size, int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype,
+    int kv_cache_dtype, const void *indices, int index_bytes, int64_t num_indices, int64_t num_src_rows,
+    void *keys_out, void *values_out, int64_t out_key_stride, int64_t out_value_stride, void *stream);
+
 /*
  * NVFP4-style KV-cache write for ONE layer: e2m1 values, two per byte (first element
  * in the low nibble), plus one e4m3 scale byte per 16 elements.  Replaces

@@ -88,6 +88,9 @@ def test_argument_errors_return_codes_without_launching(lib):
     assert rc == 1 and b"null row map" in lib.arctic_last_error()
     assert lib.arctic_reshape_and_cache_flash_bulk_select(*bulk[:10], 0, *bulk[11:], None, None, 8, 4, 4, None, None, 0, 0,
                                                           None) == 0
+    static = (*bulk[:9], 1 << 20, *bulk[10:], None, 8, 4, 1 << 20, None, None, 0, 0, None)
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select_static(*static)
+    assert rc == 1 and b"exceeds the 262144 tokens" in lib.arctic_last_error()
     rc = lib.arctic_build_row_map(None, 8, None, 2, 0, None)
     assert rc == 2 and b"int32 or int64" in lib.arctic_last_error()
     rc = lib.arctic_build_row_map(None, 8, None, 8, 0, None)

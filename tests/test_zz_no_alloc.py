@@ -1,0 +1,120 @@
+"""The entry point that allocates nothing, arctic_reshape_and_cache_flash_bulk_select_static, against the entry points
+it stands in for (arctic_build_row_map + arctic_reshape_and_cache_flash_bulk_select with a row map of the caller's):
+every cache byte and every selected row bit for bit, on two calls in a row, the second with a smaller input, so that
+whatever the first call left in the library's device array would show.  All calls go through the C ABI."""
+import ctypes
+
+import pytest
+import torch
+
+import oracle
+from arcticinference_amd import _native
+from helpers import assert_bulk_equal, bulk_args, bulk_case_to, make_bulk_case
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+SRC = {torch.bfloat16: _native.DTYPE_BF16, torch.float16: _native.DTYPE_F16, torch.float32: _native.DTYPE_F32}
+KV = {"auto": _native.KV_AUTO, "fp8": _native.KV_FP8_E4M3, "fp8_e5m2": _native.KV_FP8_E5M2}
+
+
+def table(tensors):
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+def common_args(d):
+    kc, vc = d["key_caches"], d["value_caches"]
+    return (d["keys"].data_ptr(), d["values"].data_ptr(), d["keys"].stride(0), d["values"].stride(0),
+            table(kc), table(vc), table(d["k_scales"]), table(d["v_scales"]),
+            d["slot_mapping"].data_ptr(), d["slot_mapping"].numel(), len(kc), d["num_heads"], d["head_size"],
+            kc[0].size(1), kc[0].stride(0), kc[0].size(0), SRC[d["keys"].dtype], KV[d["kv_cache_dtype"]])
+
+
+def out_buffers(rows, width, dtype):
+    out = []
+    for _ in range(2):
+        t = torch.empty(rows, width, dtype=dtype, device=DEV)
+        t.view(torch.uint8).fill_(0xA5)
+        out.append(t)
+    return out
+
+
+def both_ways(lib, case, idx):
+    """Runs the workspace form and the static form on two device copies of `case`; returns what each wrote."""
+    stream = torch.cuda.current_stream().cuda_stream
+    idx = idx.to(DEV)
+    width = case["keys"].size(1)
+    rows = idx.numel() + 2
+    results = []
+    for static in (False, True):
+        d = bulk_case_to(case, DEV)
+        k_out, v_out = out_buffers(rows, width, case["keys"].dtype)
+        tail = (idx.data_ptr(), idx.element_size(), idx.numel(), d["keys"].size(0), k_out.data_ptr(), v_out.data_ptr(),
+                k_out.stride(0), v_out.stride(0), stream)
+        if static:
+            rc = lib.arctic_reshape_and_cache_flash_bulk_select_static(*common_args(d), *tail)
+            assert rc == 0, lib.arctic_last_error()
+            torch.cuda.synchronize()
+        else:
+            row_map = torch.empty(d["slot_mapping"].numel(), dtype=torch.int64, device=DEV)
+            rc = lib.arctic_build_row_map(row_map.data_ptr(), row_map.numel(), idx.data_ptr(), idx.element_size(),
+                                          idx.numel(), stream)
+            assert rc == 0, lib.arctic_last_error()
+            rc = lib.arctic_reshape_and_cache_flash_bulk_select(*common_args(d), row_map.data_ptr(), *tail)
+            assert rc == 0, lib.arctic_last_error()
+            torch.cuda.synchronize()
+        results.append((d, k_out, v_out))
+    return results
+
+
+def check_pair(lib, case, idx):
+    (d_ws, k_ws, v_ws), (d_st, k_st, v_st) = both_ways(lib, case, idx)
+    bits = lambda t: t.cpu().contiguous().view(torch.uint8)
+    for a, b in zip(d_st["bufs"], d_ws["bufs"]):
+        assert torch.equal(bits(a), bits(b)), "static and workspace forms wrote different cache bytes"
+    assert torch.equal(bits(k_st), bits(k_ws)) and torch.equal(bits(v_st), bits(v_ws))
+    # and both are right: caches against the CPU oracle, selected rows against index_select
+    oracle.reshape_and_cache_flash_bulk(*bulk_args(case))
+    assert_bulk_equal(d_st["bufs"], case["bufs"])
+    n = idx.numel()
+    assert torch.equal(bits(k_st[:n]), bits(case["keys"].index_select(0, idx.long())))
+    assert torch.equal(bits(v_st[:n]), bits(case["values"].index_select(0, idx.long())))
+    assert (bits(k_st[n:]) == 0xA5).all() and (bits(v_st[n:]) == 0xA5).all()
+
+
+def test_two_calls_in_a_row_the_second_smaller(ops):
+    lib = _native.load()
+    g = torch.Generator().manual_seed(5)
+    # first call: 3000 tokens, rows 1500.. selected, some twice
+    big = make_bulk_case(T=3000, L=6, H=8, D=128, bs=16, NB=256, kv_cache_dtype="fp8", seed=60, std=1.5, pad_fraction=0.1)
+    idx_big = torch.cat([torch.randperm(3000, generator=g)[:200], torch.tensor([2999, 2999, 1500])])
+    check_pair(lib, big, idx_big)
+    # second call, smaller in every respect; its tokens 0..89 had other entries in the first call's row map
+    small = make_bulk_case(T=90, L=3, H=8, D=128, bs=16, NB=8, kv_cache_dtype="fp8", seed=61, std=1.5, pad_fraction=0.2)
+    idx_small = torch.tensor([7, 3, 88, 3, 0], dtype=torch.int32)
+    check_pair(lib, small, idx_small)
+    # third: a bf16 cache, the element-wise kernel (60-element rows), and keys with more rows than slots
+    odd = make_bulk_case(T=50, L=4, H=3, D=20, bs=4, NB=16, kv_cache_dtype="auto", seed=62, key_pad=3)
+    odd["slot_mapping"] = odd["slot_mapping"][:40].contiguous()
+    check_pair(lib, odd, torch.tensor([49, 0, 41, 12, 12]))
+    # nothing selected: the plain write
+    check_pair(lib, small, torch.empty(0, dtype=torch.int64))
+
+
+def test_size_limit_and_argument_errors(ops):
+    lib = _native.load()
+    case = make_bulk_case(T=8, L=2, H=2, D=64, bs=16, NB=2, kv_cache_dtype="fp8", seed=63)
+    d = bulk_case_to(case, DEV)
+    args = list(common_args(d))
+    idx = torch.arange(4, device=DEV)
+    out = torch.zeros(4, 256, dtype=torch.bfloat16, device=DEV)
+    tail = (idx.data_ptr(), 8, 4, 8, out.data_ptr(), out.data_ptr(), 256, 256, None)
+    too_many = list(args)
+    too_many[9] = 262144 + 1
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select_static(*too_many, *tail)
+    assert rc == 1 and b"exceeds the 262144 tokens" in lib.arctic_last_error()
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select_static(*args, None, 8, 4, 8, *tail[4:])
+    assert rc == 1 and b"null indices" in lib.arctic_last_error()
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select_static(*args, idx.data_ptr(), 2, 4, 8, *tail[4:])
+    assert rc == 2 and b"int32 or int64" in lib.arctic_last_error()
+    torch.cuda.synchronize()
+    assert not out.any()

@@ -36,6 +36,7 @@ struct LstmParams {
   int64_t z_stride;
   int64_t pc_stride;
   int64_t out_stride;
+  int64_t rows;
   int D;
   float inv_D;        // 1 / D
   float alpha;
@@ -52,27 +53,32 @@ struct LstmParams {
 // gates, as the speculator's z4 = emb.repeat(1, 1, 4) would; it is then read once, not four times.
 // kAllVectors: all four scale / shift vectors are given (the speculator always passes them)
 // AND every lane of the workgroup owns a chunk, so no select on either is needed.
-template <typename T, int E, int kChunksPerThread, bool kFastGelu, int kMaxThreads, bool kSharedZ, bool kAllVectors>
+// kRows: rows per workgroup (consecutive).  With two, the second row's loads are issued right behind the
+// first row's, so the first row's arithmetic runs while the second row is still arriving.
+// kVariant: bit 0: input gate loaded and consumed before the forget gate and the previous cell; bit 1: the
+// output gate's sigmoid ahead of the second row sum (what the library ships for rows of up to 4096: by then the
+// gate has arrived and the waves would otherwise idle at the barrier); bit 2: one reciprocal shared by the
+// sigmoids and the GELU of a phase.  Built for tuning, every combination can be selected at run time.
+template <typename C, int K>
+struct LstmRow {
+  C sc[K], zc[K], sf[K], zf[K], si[K], zi[K], pc[K], so[K], zo[K];
+};
+
+enum : int { kLstmInputGateFirst = 1, kLstmEarlyOutputGate = 2, kLstmSharedReciprocal = 4 };
+
+template <typename T, int E, int kChunksPerThread, bool kFastGelu, int kMaxThreads, bool kSharedZ, bool kAllVectors,
+          int kRows, int kVariant>
 __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmParams p) {
-  __shared__ float slots_cpre[16];
-  __shared__ float slots_cnew[16];
+  __shared__ float slots_cpre[kRows][16];
+  __shared__ float slots_cnew[kRows][16];
   constexpr int K = kChunksPerThread;
   using C = Chunk<E>;
   const int D = p.D;
   const int chunks = D / E;
-  const int64_t row = blockIdx.x;
   const int64_t gate_bytes = (int64_t)D * 2;
-  const char *s_row = p.states + row * p.s_stride * 2;
-  int64_t zr = row;
-  if (kSharedZ && p.z_index) zr = min(max(p.z_index[row], (int64_t)0), p.z_rows - 1);
-  const char *z_row = p.z4 + zr * p.z_stride * 2;
-  const char *pc_row = p.prev_cell + row * p.pc_stride * 2;
-  char *oc_row = p.out_cell + row * p.out_stride * 2;
-  char *os_row = p.out_state + row * p.out_stride * 2;
 
   bool live[K];
   int64_t off[K];
-  C sc[K], zc[K], sf[K], zf[K], si[K], zi[K], pc[K], so[K], zo[K];
   C wc[K], bc[K], ws[K], bs[K];
 #pragma unroll
   for (int k = 0; k < K; ++k) {
@@ -90,120 +96,231 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
     if (kAllVectors || p.w_state) ws[k] = C::load(p.w_state + off[k]);
     if (kAllVectors || p.b_state) bs[k] = C::load(p.b_state + off[k]);
   }
-#pragma unroll
-  for (int k = 0; k < K; ++k) {
-    zc[k] = C::load_stream(z_row + (kSharedZ ? 0 : 3 * gate_bytes) + off[k]);
-    sc[k] = C::load_stream(s_row + 3 * gate_bytes + off[k]);
-  }
-#pragma unroll
-  for (int k = 0; k < K; ++k) {
-    sf[k] = C::load_stream(s_row + off[k]);
-    zf[k] = kSharedZ ? zc[k] : C::load_stream(z_row + off[k]);
-  }
-#pragma unroll
-  // the cell comes straight from the previous step's launch and both outputs are read by the next
-  // kernels of the step, so these three accesses stay in the caches; the gates are touched once and stream
-  for (int k = 0; k < K; ++k) pc[k] = C::load(pc_row + off[k]);
-#pragma unroll
-  for (int k = 0; k < K; ++k) {
-    si[k] = C::load_stream(s_row + gate_bytes + off[k]);
-    zi[k] = kSharedZ ? zc[k] : C::load_stream(z_row + gate_bytes + off[k]);
-  }
-#pragma unroll
-  for (int k = 0; k < K; ++k) {
-    so[k] = C::load_stream(s_row + 2 * gate_bytes + off[k]);
-    zo[k] = kSharedZ ? zc[k] : C::load_stream(z_row + 2 * gate_bytes + off[k]);
-  }
 
-  // Lanes beyond the row take part in the sums with zeros.  (Each value is
-  // cleared where it is first used, not here: touching pc now would wait for it.)
-  // phase 1: pre_c and its sum of squares (reference :65-82); needs the cell gate only
-  float cact[K][E];
-  float ss = 0.f;
+  LstmRow<C, K> in[kRows];
+  auto issue_loads = [&](int64_t row, LstmRow<C, K> &r) {
+    const char *s_row = p.states + row * p.s_stride * 2;
+    int64_t zr = row;
+    if (kSharedZ && p.z_index) zr = min(max(p.z_index[row], (int64_t)0), p.z_rows - 1);
+    const char *z_row = p.z4 + zr * p.z_stride * 2;
+    const char *pc_row = p.prev_cell + row * p.pc_stride * 2;
 #pragma unroll
-  for (int k = 0; k < K; ++k) {
-    float a[E], b[E];
-    if (!live[k]) sc[k] = zc[k] = C::zero();
-    sc[k].template unpack<T>(a);
-    zc[k].template unpack<T>(b);
-#pragma unroll
-    for (int j = 0; j < E; ++j) {
-      cact[k][j] = fmaf(p.alpha, b[j], a[j]);
-      ss = fmaf(cact[k][j], cact[k][j], ss);
+    for (int k = 0; k < K; ++k) {
+      r.zc[k] = C::load_stream(z_row + (kSharedZ ? 0 : 3 * gate_bytes) + off[k]);
+      r.sc[k] = C::load_stream(s_row + 3 * gate_bytes + off[k]);
     }
-  }
-  const float inv_cpre = rsqrtf(block_sum(ss, slots_cpre) * p.inv_D + p.eps_cell);
-  // candidate = gelu(rmsnorm(pre_c)): runs while the other gates are still arriving
+    auto forget_and_cell = [&]() {
 #pragma unroll
-  for (int k = 0; k < K; ++k) {
-    // an absent scale / shift vector acts as 1 / 0 (exact), so the norm is one multiply and
-    // one fused multiply-add per element whichever vectors were given
-    float w[E], b[E];
+      for (int k = 0; k < K; ++k) {
+        r.sf[k] = C::load_stream(s_row + off[k]);
+        r.zf[k] = kSharedZ ? r.zc[k] : C::load_stream(z_row + off[k]);
+      }
+      // the cell comes straight from the previous step's launch and both outputs are read by the next
+      // kernels of the step, so these three accesses stay in the caches; the gates are touched once and stream
 #pragma unroll
-    for (int j = 0; j < E; ++j) {
-      w[j] = 1.f;
-      b[j] = 0.f;
+      for (int k = 0; k < K; ++k) r.pc[k] = C::load(pc_row + off[k]);
+    };
+    auto input_gate = [&]() {
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        r.si[k] = C::load_stream(s_row + gate_bytes + off[k]);
+        r.zi[k] = kSharedZ ? r.zc[k] : C::load_stream(z_row + gate_bytes + off[k]);
+      }
+    };
+    // the groups must reach memory in this order (it returns loads in issue order); with more than one row per
+    // workgroup the compiler would otherwise interleave the rows' loads
+    if constexpr (kRows > 1) __builtin_amdgcn_sched_barrier(0);
+    if constexpr (kVariant & kLstmInputGateFirst) {
+      input_gate();
+      if constexpr (kRows > 1) __builtin_amdgcn_sched_barrier(0);
+      forget_and_cell();
+    } else {
+      forget_and_cell();
+      if constexpr (kRows > 1) __builtin_amdgcn_sched_barrier(0);
+      input_gate();
     }
-    if (kAllVectors || p.w_cell) wc[k].template unpack<T>(w);
-    if (kAllVectors || p.b_cell) bc[k].template unpack<T>(b);
-    const float mask = live[k] ? 1.f : 0.f;  // idle lanes must add nothing to the second sum
+    if constexpr (kRows > 1) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int j = 0; j < E; ++j) {
-      const float cn = fmaf(cact[k][j] * inv_cpre, w[j], b[j]);
-      cact[k][j] = gelu<kFastGelu>(cn) * mask;
+    for (int k = 0; k < K; ++k) {
+      r.so[k] = C::load_stream(s_row + 2 * gate_bytes + off[k]);
+      r.zo[k] = kSharedZ ? r.zc[k] : C::load_stream(z_row + 2 * gate_bytes + off[k]);
     }
-  }
+    if constexpr (kRows > 1) __builtin_amdgcn_sched_barrier(0);
+  };
 
-  // phase 2: cell update; write out_cell (reference :104-140)
-  float cell[K][E];  // ends up as the ROUNDED new cell, as the state phase must see it
-  ss = 0.f;
+  auto compute = [&](int64_t row, LstmRow<C, K> &r, float *slots_a, float *slots_b) {
+    char *oc_row = p.out_cell + row * p.out_stride * 2;
+    char *os_row = p.out_state + row * p.out_stride * 2;
+    if constexpr (kRows > 1) __builtin_amdgcn_sched_barrier(0);   // one row's arithmetic after the other's
+    // Lanes beyond the row take part in the sums with zeros.  (Each value is
+    // cleared where it is first used, not here: touching pc now would wait for it.)
+    // phase 1: pre_c and its sum of squares (reference :65-82); needs the cell gate only
+    float cact[K][E];
+    float ss = 0.f;
 #pragma unroll
-  for (int k = 0; k < K; ++k) {
-    float a[E], b[E], c[E];
-    sf[k].template unpack<T>(a);
-    zf[k].template unpack<T>(b);
-    if (!live[k]) pc[k] = C::zero();
-    pc[k].template unpack<T>(c);
+    for (int k = 0; k < K; ++k) {
+      float a[E], b[E];
+      if (!live[k]) r.sc[k] = r.zc[k] = C::zero();
+      r.sc[k].template unpack<T>(a);
+      r.zc[k].template unpack<T>(b);
 #pragma unroll
-    for (int j = 0; j < E; ++j) cell[k][j] = sigmoid_f(fmaf(p.alpha, b[j], a[j])) * c[j];
-    // keep the forget-gate arithmetic ahead of the wait for the input gate: it then runs while that gate
-    // is still arriving instead of in the short stretch between the last two gates
-    __builtin_amdgcn_sched_barrier(0);
-    si[k].template unpack<T>(a);
-    zi[k].template unpack<T>(b);
-#pragma unroll
-    for (int j = 0; j < E; ++j) {
-      const float cnew = fmaf(cact[k][j], sigmoid_f(fmaf(p.alpha, b[j], a[j])), cell[k][j]);
-      ss = fmaf(cnew, cnew, ss);  // unrounded, as in the reference (:136)
-      cell[k][j] = cnew;
+      for (int j = 0; j < E; ++j) {
+        cact[k][j] = fmaf(p.alpha, b[j], a[j]);
+        ss = fmaf(cact[k][j], cact[k][j], ss);
+      }
     }
-    const C packed = C::template pack<T>(cell[k]);
-    if (live[k]) packed.store(oc_row + off[k]);
-    packed.template unpack<T>(cell[k]);
-  }
-  const float inv_cnew = rsqrtf(block_sum(ss, slots_cnew) * p.inv_D + p.eps_state);
+    const float inv_cpre = rsqrtf(block_sum(ss, slots_a) * p.inv_D + p.eps_cell);
+    // candidate = gelu(rmsnorm(pre_c)): runs while the other gates are still arriving
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      // an absent scale / shift vector acts as 1 / 0 (exact), so the norm is one multiply and
+      // one fused multiply-add per element whichever vectors were given
+      float w[E], b[E];
+#pragma unroll
+      for (int j = 0; j < E; ++j) {
+        w[j] = 1.f;
+        b[j] = 0.f;
+      }
+      if (kAllVectors || p.w_cell) wc[k].template unpack<T>(w);
+      if (kAllVectors || p.b_cell) bc[k].template unpack<T>(b);
+      const float mask = live[k] ? 1.f : 0.f;  // idle lanes must add nothing to the second sum
+#pragma unroll
+      for (int j = 0; j < E; ++j) {
+        const float cn = fmaf(cact[k][j] * inv_cpre, w[j], b[j]);
+        cact[k][j] = gelu<kFastGelu>(cn) * mask;
+      }
+    }
 
-  // phase 3: state = gelu(rmsnorm(rounded cell)) * sigmoid(pre_o) (reference :160-190);
-  // the output gate is the last load to arrive and is consumed last
+    // phase 2: cell update; write out_cell (reference :104-140)
+    float cell[K][E];  // ends up as the ROUNDED new cell, as the state phase must see it
+    ss = 0.f;
 #pragma unroll
-  for (int k = 0; k < K; ++k) {
-    float w[E], b[E], st[E];
+    for (int k = 0; k < K; ++k) {
+      float a[E], b[E], c[E];
+      if constexpr (kVariant & kLstmInputGateFirst) {
+        float gi[E];
+        r.si[k].template unpack<T>(a);
+        r.zi[k].template unpack<T>(b);
 #pragma unroll
-    for (int j = 0; j < E; ++j) {
-      w[j] = 1.f;
-      b[j] = 0.f;
+        for (int j = 0; j < E; ++j) gi[j] = sigmoid_f(fmaf(p.alpha, b[j], a[j]));
+        __builtin_amdgcn_sched_barrier(0);
+        r.sf[k].template unpack<T>(a);
+        r.zf[k].template unpack<T>(b);
+#pragma unroll
+        for (int j = 0; j < E; ++j) cell[k][j] = sigmoid_f(fmaf(p.alpha, b[j], a[j]));
+        __builtin_amdgcn_sched_barrier(0);
+        if (!live[k]) r.pc[k] = C::zero();
+        r.pc[k].template unpack<T>(c);
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+          const float cnew = fmaf(cact[k][j], gi[j], cell[k][j] * c[j]);
+          ss = fmaf(cnew, cnew, ss);  // unrounded, as in the reference (:136)
+          cell[k][j] = cnew;
+        }
+      } else {
+        r.sf[k].template unpack<T>(a);
+        r.zf[k].template unpack<T>(b);
+        if (!live[k]) r.pc[k] = C::zero();
+        r.pc[k].template unpack<T>(c);
+        if constexpr ((kVariant & kLstmSharedReciprocal) && !kFastGelu) {
+          // c_new = (pc (1 + e_i) + cand (1 + e_f)) / ((1 + e_f)(1 + e_i)): one reciprocal for both gates
+          float df[E];
+#pragma unroll
+          for (int j = 0; j < E; ++j) df[j] = sigmoid_den(fmaf(p.alpha, b[j], a[j]));
+          r.si[k].template unpack<T>(a);
+          r.zi[k].template unpack<T>(b);
+#pragma unroll
+          for (int j = 0; j < E; ++j) {
+            const float di = sigmoid_den(fmaf(p.alpha, b[j], a[j]));
+            const float num = fmaf(cact[k][j], df[j], c[j] * di);
+            const float cnew = num * __builtin_amdgcn_rcpf(df[j] * di);
+            ss = fmaf(cnew, cnew, ss);
+            cell[k][j] = cnew;
+          }
+        } else {
+#pragma unroll
+        for (int j = 0; j < E; ++j) cell[k][j] = sigmoid_f(fmaf(p.alpha, b[j], a[j])) * c[j];
+        // keep the forget-gate arithmetic ahead of the wait for the input gate: it then runs while that gate
+        // is still arriving instead of in the short stretch between the last two gates
+        __builtin_amdgcn_sched_barrier(0);
+        r.si[k].template unpack<T>(a);
+        r.zi[k].template unpack<T>(b);
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+          const float cnew = fmaf(cact[k][j], sigmoid_f(fmaf(p.alpha, b[j], a[j])), cell[k][j]);
+          ss = fmaf(cnew, cnew, ss);  // unrounded, as in the reference (:136)
+          cell[k][j] = cnew;
+        }
+        }
+      }
+      const C packed = C::template pack<T>(cell[k]);
+      if (live[k]) packed.store(oc_row + off[k]);
+      packed.template unpack<T>(cell[k]);
     }
-    if (kAllVectors || p.w_state) ws[k].template unpack<T>(w);
-    if (kAllVectors || p.b_state) bs[k].template unpack<T>(b);
+    float og[K][E];
+    if constexpr (kVariant & kLstmEarlyOutputGate) {
 #pragma unroll
-    for (int j = 0; j < E; ++j) st[j] = gelu<kFastGelu>(fmaf(cell[k][j] * inv_cnew, w[j], b[j]));
-    float a[E], g[E];
-    so[k].template unpack<T>(a);
-    zo[k].template unpack<T>(g);
+      for (int k = 0; k < K; ++k) {
+        float a[E], g[E];
+        r.so[k].template unpack<T>(a);
+        r.zo[k].template unpack<T>(g);
 #pragma unroll
-    for (int j = 0; j < E; ++j) st[j] *= sigmoid_f(fmaf(p.alpha, g[j], a[j]));
-    if (live[k]) C::template pack<T>(st).store(os_row + off[k]);
-  }
+        for (int j = 0; j < E; ++j) og[k][j] = sigmoid_f(fmaf(p.alpha, g[j], a[j]));
+      }
+    }
+    const float inv_cnew = rsqrtf(block_sum(ss, slots_b) * p.inv_D + p.eps_state);
+
+    // phase 3: state = gelu(rmsnorm(rounded cell)) * sigmoid(pre_o) (reference :160-190);
+    // the output gate is the last load to arrive and is consumed last
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      float w[E], b[E], st[E];
+#pragma unroll
+      for (int j = 0; j < E; ++j) {
+        w[j] = 1.f;
+        b[j] = 0.f;
+      }
+      if (kAllVectors || p.w_state) ws[k].template unpack<T>(w);
+      if (kAllVectors || p.b_state) bs[k].template unpack<T>(b);
+      if constexpr ((kVariant & kLstmSharedReciprocal) && !kFastGelu) {
+        // the GELU's reciprocal and the output gate's from one: 1 / (u v), times v, times u
+        float a[E], g[E];
+        r.so[k].template unpack<T>(a);
+        r.zo[k].template unpack<T>(g);
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+          const float x = fmaf(cell[k][j] * inv_cnew, w[j], b[j]);
+          const float u = gelu_erf_den(x), v = sigmoid_den(fmaf(p.alpha, g[j], a[j]));
+          const float rcp = __builtin_amdgcn_rcpf(u * v);
+          st[j] = gelu_erf_given_t(x, rcp * v) * (rcp * u);
+        }
+        if (live[k]) C::template pack<T>(st).store(os_row + off[k]);
+        continue;
+      }
+#pragma unroll
+      for (int j = 0; j < E; ++j) st[j] = gelu<kFastGelu>(fmaf(cell[k][j] * inv_cnew, w[j], b[j]));
+      if constexpr (kVariant & kLstmEarlyOutputGate) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) st[j] *= og[k][j];
+      } else {
+        float a[E], g[E];
+        r.so[k].template unpack<T>(a);
+        r.zo[k].template unpack<T>(g);
+#pragma unroll
+        for (int j = 0; j < E; ++j) st[j] *= sigmoid_f(fmaf(p.alpha, g[j], a[j]));
+      }
+      if (live[k]) C::template pack<T>(st).store(os_row + off[k]);
+    }
+  };
+
+  const int64_t row0 = (int64_t)blockIdx.x * kRows;
+  // every row's loads are issued unconditionally (a workgroup past the last row reads that row again and drops
+  // it): loads behind a branch would make the waits below count as if they had not been issued
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) issue_loads(min(row0 + r, p.rows - 1), in[r]);
+#pragma unroll
+  for (int r = 0; r < kRows; ++r)
+    if (r == 0 || row0 + r < p.rows) compute(row0 + r, in[r], slots_cpre[r], slots_cnew[r]);
 }
 
 // Any D, any alignment: element-wise, three passes like the reference's scalar
@@ -257,6 +374,25 @@ __global__ __launch_bounds__(256) void sum_lstm_scalar_kernel(const LstmParams p
 
 static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
+#ifdef ARCTIC_TUNING
+// Measurement build only: ARCTIC_LSTM_VARIANT = variant bits (see sum_lstm_vec_kernel) + 8 for two rows per workgroup
+// + 16 for two chunks per lane (256 lanes per 4096-wide row).  Read at every call.
+static int lstm_tuning_variant() {
+  const char *e = getenv("ARCTIC_LSTM_VARIANT");
+  return e ? atoi(e) : 0;
+}
+template <typename T, bool kFastGelu, bool kSharedZ, int kVariant>
+static void launch_lstm_tuned(const LstmParams &p, int64_t rows, int shape, int threads, hipStream_t s) {
+  const dim3 one((unsigned)rows), two((unsigned)((rows + 1) / 2));
+  switch (shape) {
+    case 0: hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, true, 1, kVariant>), one, dim3(threads), 0, s, p); break;
+    case 1: hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, true, 2, kVariant>), two, dim3(threads), 0, s, p); break;
+    case 2: hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 2, kFastGelu, 512, kSharedZ, true, 1, kVariant>), one, dim3(threads / 2), 0, s, p); break;
+    default: hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 2, kFastGelu, 512, kSharedZ, true, 2, kVariant>), two, dim3(threads / 2), 0, s, p); break;
+  }
+}
+#endif
+
 template <typename T, bool kFastGelu, bool kSharedZ>
 static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
   const int chunks = p.D / 8;
@@ -274,12 +410,28 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
     int threads = (chunks + cpt - 1) / cpt;
     threads = std::max(64, (threads + 63) & ~63);
     const bool all = p.w_cell && p.b_cell && p.w_state && p.b_state && threads * cpt == chunks;
+#ifdef ARCTIC_TUNING
+    if (cpt == 1 && all && threads % 128 == 0) {
+      const int v = lstm_tuning_variant();
+      const int shape = (v >> 3) & 3;
+      switch (v & 7) {
+        case 0: launch_lstm_tuned<T, kFastGelu, kSharedZ, 0>(p, rows, shape, threads, s); break;
+        case 1: launch_lstm_tuned<T, kFastGelu, kSharedZ, 1>(p, rows, shape, threads, s); break;
+        case 2: launch_lstm_tuned<T, kFastGelu, kSharedZ, 2>(p, rows, shape, threads, s); break;
+        case 3: launch_lstm_tuned<T, kFastGelu, kSharedZ, 3>(p, rows, shape, threads, s); break;
+        case 4: launch_lstm_tuned<T, kFastGelu, kSharedZ, 4>(p, rows, shape, threads, s); break;
+        default: launch_lstm_tuned<T, kFastGelu, kSharedZ, 5>(p, rows, shape, threads, s); break;
+      }
+      return;
+    }
+#endif
+    constexpr int kShipped = kLstmEarlyOutputGate;   // measured best of the variants that change no result bit
     if (cpt == 1 && all)
-      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, true>), grid, dim3(threads), 0, s, p);
+      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, true, 1, kShipped>), grid, dim3(threads), 0, s, p);
     else if (cpt == 1)
-      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, false>), grid, dim3(threads), 0, s, p);
+      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, false, 1, kShipped>), grid, dim3(threads), 0, s, p);
     else
-      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 2, kFastGelu, 1024, kSharedZ, false>), grid, dim3(threads), 0, s, p);
+      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 2, kFastGelu, 1024, kSharedZ, false, 1, 0>), grid, dim3(threads), 0, s, p);
   } else {
     hipLaunchKernelGGL((sum_lstm_scalar_kernel<T, kFastGelu>), grid, dim3(256), 0, s, p, kSharedZ ? 0 : p.D);
   }
@@ -318,6 +470,7 @@ static int sum_lstm_entry(const char *fn, bool shared_z, void *out_state, void *
   p.z_stride = z_stride;
   p.pc_stride = pc_stride;
   p.out_stride = out_stride;
+  p.rows = rows;
   p.D = D;
   p.inv_D = 1.0f / (float)D;
   p.alpha = alpha;

@@ -795,6 +795,113 @@ def placement_sweep(ops, dev, steps):
     return out
 
 
+def load_tuning_library():
+    """libarctic_tuning_mi355x.so: the library's sources compiled with -DARCTIC_TUNING (`make -C
+    arcticinference_amd/csrc tuning`, also done by __graft_entry__.build()), in which environment variables select
+    kernel variants and launch shapes.  Only the sweeps below use it."""
+    import ctypes
+    path = os.path.join(ROOT, "arcticinference_amd", "libarctic_tuning_mi355x.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    vp, i64, i32, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+    lib.arctic_sum_lstm.argtypes = [vp] * 9 + [i64, i32, i64, i64, i64, i64, f32, f32, f32, i32, i32, vp]
+    lib.arctic_sum_lstm.restype = i32
+    return lib
+
+
+# ARCTIC_LSTM_VARIANT values of the tuning build (sum_lstm.hip): bits 0-2 = arithmetic / ordering variants,
+# bits 3-4 = launch shape
+LSTM_VARIANTS = [
+    (0, "loads c f pc i o, one row per 512-lane workgroup, output gate after the second row sum"),
+    (1, "input gate loaded and consumed before forget gate and previous cell (c i f pc o)"),
+    (2, "as shipped: output gate's sigmoid ahead of the second row sum"),
+    (3, "input gate first + output gate's sigmoid ahead of the second row sum"),
+    (4, "shared reciprocals: one for the forget and input gates, one for the state GELU and the output gate"),
+    (8, "two rows per workgroup, second row's loads issued behind the first row's"),
+    (11, "two rows per workgroup + input gate first + early output gate"),
+    (16, "two 16-byte chunks per lane (256 lanes per row)"),
+    (24, "two chunks per lane and two rows per workgroup"),
+]
+
+
+def bench_lstm_variants(dev, steps):
+    """A/B of sum_lstm kernel variants on the speculator workload (512 x 4096 bf16, eight rotating buffer sets, three
+    chained steps per set inside one HIP graph), all in this process.  Each variant is also compared with the
+    first variant's outputs: share of bit-identical elements and largest difference."""
+    tuning = load_tuning_library()
+    if tuning is None:
+        return "libarctic_tuning_mi355x.so is not built"
+    T, Hd, sets = 512, 4096, 8
+    g = torch.Generator(device=dev).manual_seed(3)
+    rn = lambda *s: torch.randn(*s, generator=g, device=dev).to(torch.bfloat16)
+    S = [[rn(T, 4 * Hd) for _ in range(3)] for _ in range(sets)]
+    Z = [[rn(T, 4 * Hd) for _ in range(3)] for _ in range(sets)]
+    C0 = [rn(T, Hd) for _ in range(sets)]
+    vec = lambda m: (m + 0.02 * torch.randn(Hd, generator=g, device=dev)).to(torch.bfloat16)
+    w_cell, b_cell, w_state, b_state = vec(1.0), vec(0.0), vec(1.0), vec(0.0)
+    sw = 0.5 ** (0.5 / 3)
+    alpha = ((1 - sw * sw) * (Hd / 2)) ** 0.5 / sw
+    ST = [[torch.empty(T, Hd, dtype=torch.bfloat16, device=dev) for _ in range(3)] for _ in range(sets)]
+    CE = [[torch.empty(T, Hd, dtype=torch.bfloat16, device=dev) for _ in range(3)] for _ in range(sets)]
+    per_call = 22 * Hd * T
+
+    def run_all():
+        stream = torch.cuda.current_stream().cuda_stream
+        for i in range(sets):
+            cell = C0[i]
+            for k in range(3):
+                rc = tuning.arctic_sum_lstm(ST[i][k].data_ptr(), CE[i][k].data_ptr(), S[i][k].data_ptr(), Z[i][k].data_ptr(),
+                                            cell.data_ptr(), w_cell.data_ptr(), b_cell.data_ptr(), w_state.data_ptr(),
+                                            b_state.data_ptr(), T, Hd, 4 * Hd, 4 * Hd, Hd, Hd, alpha, 1e-6, 1e-6, 0, 2, stream)
+                assert rc == 0
+                cell = CE[i][k]
+
+    floor = load_floor_kernels()
+    out, base = {}, None
+    rounds = 3   # every variant is timed in each round, so drift over the run shows up as spread, not as a ranking
+    graphs = {}
+    for code, what in LSTM_VARIANTS:
+        os.environ["ARCTIC_LSTM_VARIANT"] = str(code)
+        run_all()
+        torch.cuda.synchronize()
+        got = [t.clone() for i in range(sets) for t in (ST[i][2], CE[i][2])]
+        if base is None:
+            base = got
+        same = sum(int((a == b).sum()) for a, b in zip(got, base)) / sum(a.numel() for a in got)
+        worst = max(float((a.float() - b.float()).abs().max()) for a, b in zip(got, base))
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            run_all()
+        graphs[code] = graph
+        out[str(code)] = {"variant": what, "bit_identical_to_variant_0": round(same, 5), "max_abs_diff": worst, "us": []}
+    os.environ.pop("ARCTIC_LSTM_VARIANT", None)
+    if floor is not None:
+        OS = [torch.empty(T, Hd, dtype=torch.bfloat16, device=dev) for _ in range(2)]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            stream = torch.cuda.current_stream().cuda_stream
+            for i in range(sets):
+                for k in range(3):
+                    floor.floor_lstm_traffic(S[i][k].data_ptr(), Z[i][k].data_ptr(), C0[i].data_ptr(), OS[0].data_ptr(),
+                                             OS[1].data_ptr(), T, Hd, stream)
+        graphs["floor"] = graph
+        out["floor"] = {"variant": "lstm_traffic_kernel: the same loads and stores, no arithmetic", "us": []}
+    for _ in range(rounds):
+        for key, graph in graphs.items():
+            for _ in range(3):
+                graph.replay()
+            torch.cuda.synchronize()
+            us = event_times_us(graph.replay, max(10, steps // 2))
+            out[str(key)]["us"].append(round(statistics.mean(us) / (sets * 3), 3))
+    for v in out.values():
+        v["us_per_call_graph_rounds"] = v.pop("us")
+        m = statistics.mean(v["us_per_call_graph_rounds"])
+        v["us_per_call_graph"] = round(m, 2)
+        v["hbm_frac_graph"] = round(per_call / m / 1e3 / HBM_PEAK_GBS, 4)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -807,6 +914,9 @@ def main():
     ap.add_argument("--placement-sweep", action="store_true",
                     help="instead of the benchmark, time the 70B-shape launch with the caches in each 8 GiB chunk "
                          "of the GPU's memory and spread over its regions; prints one JSON object")
+    ap.add_argument("--lstm-variants", action="store_true",
+                    help="instead of the benchmark, time the sum_lstm kernel variants of the tuning build against "
+                         "each other and against the traffic-only kernel; prints one JSON object")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) so that a counter run of this "
                          "command can scale FETCH_SIZE / WRITE_SIZE")
@@ -826,6 +936,9 @@ def main():
 
     if args.placement_sweep:
         print(json.dumps({"placement_sweep": placement_sweep(ops, dev, max(5, args.steps // 5))}), flush=True)
+        return
+    if args.lstm_variants:
+        print(json.dumps({"sum_lstm_variants": bench_lstm_variants(dev, args.steps)}), flush=True)
         return
 
     extras = {}

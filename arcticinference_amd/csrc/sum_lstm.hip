@@ -55,6 +55,9 @@ struct LstmParams {
 // AND every lane of the workgroup owns a chunk, so no select on either is needed.
 // kRows: rows per workgroup (consecutive).  With two, the second row's loads are issued right behind the
 // first row's, so the first row's arithmetic runs while the second row is still arriving.
+// kZeroCell: the previous cell is all zeros (the first step of a proposal round) and is not read.  Without this
+// flag a null prev_cell is still honoured: the lanes then read the forget gate's address a second time and
+// discard it.
 // kVariant: bit 0: input gate loaded and consumed before the forget gate and the previous cell; bit 1: the
 // output gate's sigmoid ahead of the second row sum (what the library ships for rows of up to 4096: by then the
 // gate has arrived and the waves would otherwise idle at the barrier); bit 2: one reciprocal shared by the
@@ -67,7 +70,7 @@ struct LstmRow {
 enum : int { kLstmInputGateFirst = 1, kLstmEarlyOutputGate = 2, kLstmSharedReciprocal = 4 };
 
 template <typename T, int E, int kChunksPerThread, bool kFastGelu, int kMaxThreads, bool kSharedZ, bool kAllVectors,
-          int kRows, int kVariant>
+          int kRows, int kVariant, bool kZeroCell = false>
 __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmParams p) {
   __shared__ float slots_cpre[kRows][16];
   __shared__ float slots_cnew[kRows][16];
@@ -103,7 +106,7 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
     int64_t zr = row;
     if (kSharedZ && p.z_index) zr = min(max(p.z_index[row], (int64_t)0), p.z_rows - 1);
     const char *z_row = p.z4 + zr * p.z_stride * 2;
-    const char *pc_row = p.prev_cell + row * p.pc_stride * 2;
+    const char *pc_row = p.prev_cell ? p.prev_cell + row * p.pc_stride * 2 : s_row;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
       r.zc[k] = C::load_stream(z_row + (kSharedZ ? 0 : 3 * gate_bytes) + off[k]);
@@ -117,8 +120,10 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
       }
       // the cell comes straight from the previous step's launch and both outputs are read by the next
       // kernels of the step, so these three accesses stay in the caches; the gates are touched once and stream
+      if constexpr (!kZeroCell) {
 #pragma unroll
-      for (int k = 0; k < K; ++k) r.pc[k] = C::load(pc_row + off[k]);
+        for (int k = 0; k < K; ++k) r.pc[k] = C::load(pc_row + off[k]);
+      }
     };
     auto input_gate = [&]() {
 #pragma unroll
@@ -209,7 +214,7 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
 #pragma unroll
         for (int j = 0; j < E; ++j) cell[k][j] = sigmoid_f(fmaf(p.alpha, b[j], a[j]));
         __builtin_amdgcn_sched_barrier(0);
-        if (!live[k]) r.pc[k] = C::zero();
+        if (kZeroCell || !live[k] || !p.prev_cell) r.pc[k] = C::zero();
         r.pc[k].template unpack<T>(c);
 #pragma unroll
         for (int j = 0; j < E; ++j) {
@@ -220,7 +225,7 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
       } else {
         r.sf[k].template unpack<T>(a);
         r.zf[k].template unpack<T>(b);
-        if (!live[k]) r.pc[k] = C::zero();
+        if (kZeroCell || !live[k] || !p.prev_cell) r.pc[k] = C::zero();
         r.pc[k].template unpack<T>(c);
         if constexpr ((kVariant & kLstmSharedReciprocal) && !kFastGelu) {
           // c_new = (pc (1 + e_i) + cand (1 + e_f)) / ((1 + e_f)(1 + e_i)): one reciprocal for both gates
@@ -356,7 +361,7 @@ __global__ __launch_bounds__(256) void sum_lstm_scalar_kernel(const LstmParams p
     float cn = cpre * inv_cpre;
     if (wc) cn *= T::lo(wc[j]);
     if (bc) cn += T::lo(bc[j]);
-    const float cnew = T::lo(pc[j]) * sigmoid_f(pre_f) + gelu<kFastGelu>(cn) * sigmoid_f(pre_i);
+    const float cnew = (p.prev_cell ? T::lo(pc[j]) : 0.f) * sigmoid_f(pre_f) + gelu<kFastGelu>(cn) * sigmoid_f(pre_i);
     ss += cnew * cnew;
     oc[j] = (uint16_t)T::round_bits(cnew);
   }
@@ -401,7 +406,7 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
                    (!multi || (p.s_stride % 8 == 0 && p.z_stride % 8 == 0 && p.pc_stride % 8 == 0 &&
                                p.out_stride % 8 == 0)) &&
                    (!p.z_index || p.z_stride % 8 == 0) &&
-                   aligned16(p.states) && aligned16(p.z4) && aligned16(p.prev_cell) &&
+                   aligned16(p.states) && aligned16(p.z4) && aligned16(p.prev_cell) &&   /* null counts as aligned */
                    aligned16(p.out_state) && aligned16(p.out_cell) && aligned16(p.w_cell) &&
                    aligned16(p.b_cell) && aligned16(p.w_state) && aligned16(p.b_state);
   const dim3 grid((unsigned)rows);
@@ -411,7 +416,7 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
     threads = std::max(64, (threads + 63) & ~63);
     const bool all = p.w_cell && p.b_cell && p.w_state && p.b_state && threads * cpt == chunks;
 #ifdef ARCTIC_TUNING
-    if (cpt == 1 && all && threads % 128 == 0) {
+    if (cpt == 1 && all && threads % 128 == 0 && p.prev_cell) {
       const int v = lstm_tuning_variant();
       const int shape = (v >> 3) & 3;
       switch (v & 7) {
@@ -426,7 +431,9 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
     }
 #endif
     constexpr int kShipped = kLstmEarlyOutputGate;   // measured best of the variants that change no result bit
-    if (cpt == 1 && all)
+    if (cpt == 1 && all && !p.prev_cell)
+      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, true, 1, kShipped, true>), grid, dim3(threads), 0, s, p);
+    else if (cpt == 1 && all)
       hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, true, 1, kShipped>), grid, dim3(threads), 0, s, p);
     else if (cpt == 1)
       hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, false, 1, kShipped>), grid, dim3(threads), 0, s, p);
@@ -451,7 +458,7 @@ static int sum_lstm_entry(const char *fn, bool shared_z, void *out_state, void *
   if (D <= 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: last dim of states must be 4*D_gate", fn);
   if (rows < 0 || rows > 0x7fffffffLL) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: bad row count", fn);
   if (rows == 0) return ARCTIC_OK;
-  if (!out_state || !out_cell || !states || !z || !prev_cell)
+  if (!out_state || !out_cell || !states || !z)   // prev_cell may be null: a cell of zeros
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
   if (z_index && z_rows <= 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: the embedding table has no rows", fn);
   LstmParams p;
@@ -468,7 +475,7 @@ static int sum_lstm_entry(const char *fn, bool shared_z, void *out_state, void *
   p.b_state = (const char *)b_state;
   p.s_stride = s_stride;
   p.z_stride = z_stride;
-  p.pc_stride = pc_stride;
+  p.pc_stride = prev_cell ? pc_stride : 0;
   p.out_stride = out_stride;
   p.rows = rows;
   p.D = D;

@@ -48,14 +48,17 @@ _SCHEMAS = {
 # Operators that fuse a caller-side step into one of the above; the reference has no such schema.
 _EXTRA_SCHEMAS = {
     "sum_lstm_shared_z_cuda":
-        "sum_lstm_shared_z_cuda(Tensor states_4d, Tensor z_d, Tensor prev_cell_d, Tensor? w_cell, "
+        "sum_lstm_shared_z_cuda(Tensor states_4d, Tensor z_d, Tensor? prev_cell_d, Tensor? w_cell, "
         "Tensor? b_cell, Tensor? w_state, Tensor? b_state, float alpha, float eps_cell, "
         "float eps_state, bool use_fast_gelu) -> (Tensor, Tensor)",
+    "sum_lstm_zero_cell_cuda":
+        "sum_lstm_zero_cell_cuda(Tensor states_4d, Tensor z4_4d, Tensor? w_cell, Tensor? b_cell, Tensor? w_state, "
+        "Tensor? b_state, float alpha, float eps_cell, float eps_state, bool use_fast_gelu) -> (Tensor, Tensor)",
     "speculator_add_ln_act_cuda":
         "speculator_add_ln_act_cuda(Tensor input, Tensor? z, Tensor? weight, Tensor? bias, float alpha, "
         "float eps, str activation, float out_scale) -> Tensor",
     "sum_lstm_embedded_cuda":
-        "sum_lstm_embedded_cuda(Tensor states_4d, Tensor emb_weight, Tensor token_ids, Tensor prev_cell_d, "
+        "sum_lstm_embedded_cuda(Tensor states_4d, Tensor emb_weight, Tensor token_ids, Tensor? prev_cell_d, "
         "Tensor? w_cell, Tensor? b_cell, Tensor? w_state, Tensor? b_state, float alpha, float eps_cell, "
         "float eps_state, bool use_fast_gelu) -> (Tensor, Tensor)",
     "speculator_embed_add_ln_act_cuda":
@@ -490,9 +493,10 @@ def _sum_lstm_impl(
     lib = _lib()
     dtype = states_4d.dtype
     _check(dtype in _HALF_DTYPES, "sum_lstm: only fp16 and bf16 are supported.")
-    _check(states_4d.is_cuda and z4_4d.is_cuda and prev_cell_d.is_cuda,
+    zero_cell = prev_cell_d is None     # not in the reference's schema: the cell of zeros a proposal round starts from
+    _check(states_4d.is_cuda and z4_4d.is_cuda and (zero_cell or prev_cell_d.is_cuda),
            "sum_lstm: inputs must be CUDA tensors")
-    _check(z4_4d.dtype == dtype and prev_cell_d.dtype == dtype,
+    _check(z4_4d.dtype == dtype and (zero_cell or prev_cell_d.dtype == dtype),
            "sum_lstm: all input dtypes must match")
     hidden4 = states_4d.size(-1)
     _check(hidden4 > 0 and hidden4 % 4 == 0, "sum_lstm: last dim of states must be 4*D_gate")
@@ -501,10 +505,10 @@ def _sum_lstm_impl(
         _check(z4_4d.size(-1) == d_gate, "sum_lstm_shared_z: z must have last dim D_gate")
     else:
         _check(z4_4d.size(-1) == hidden4, "sum_lstm: z4 must have last dim 4*D_gate")
-    d_cell = prev_cell_d.size(-1)
+    d_cell = d_gate if zero_cell else prev_cell_d.size(-1)
     if not (d_cell == d_gate):
         raise RuntimeError(f"sum_lstm: prev_cell last dim must equal D_gate. Got {d_cell} vs expected {d_gate}.")
-    _check(states_4d.stride(-1) == 1 and z4_4d.stride(-1) == 1 and prev_cell_d.stride(-1) == 1,
+    _check(states_4d.stride(-1) == 1 and z4_4d.stride(-1) == 1 and (zero_cell or prev_cell_d.stride(-1) == 1),
            "sum_lstm: last dimension must be contiguous (stride -1 == 1)")
     for t, name in ((w_cell, "w_cell"), (b_cell, "b_cell"), (w_state, "w_state"), (b_state, "b_state")):
         if t is not None:
@@ -519,44 +523,62 @@ def _sum_lstm_impl(
 
     s2 = _rows_of(states_4d, hidden4)
     z2 = _rows_of(z4_4d, d_gate if _shared_z else hidden4)
-    p2 = _rows_of(prev_cell_d, d_cell)
     rows = s2.size(0)
+    p2 = None if zero_cell else _rows_of(prev_cell_d, d_cell)
     if _token_ids is not None:
-        _check(p2.size(0) == rows, "sum_lstm: row counts of the inputs differ")
+        _check(zero_cell or p2.size(0) == rows, "sum_lstm: row counts of the inputs differ")
         _check_embedding("sum_lstm_embedded", z4_4d, _token_ids, states_4d, d_gate, rows)
     else:
-        _check(z2.size(0) == rows and p2.size(0) == rows, "sum_lstm: row counts of the inputs differ")
-    # outputs inherit prev_cell's row pitch (reference :356-365)
-    out_cell = torch.empty_strided(p2.size(), p2.stride(), dtype=dtype, device=p2.device)
-    out_state = torch.empty_strided(p2.size(), p2.stride(), dtype=dtype, device=p2.device)
-    _check(out_cell.stride(0) == out_state.stride(0), "sum_lstm: internal - output strides mismatch")
-    flat = prev_cell_d.dim() == 2
-    out_cell_orig = out_cell if flat else out_cell.view(prev_cell_d.size())
-    out_state_orig = out_state if flat else out_state.view(prev_cell_d.size())
+        _check(z2.size(0) == rows and (zero_cell or p2.size(0) == rows), "sum_lstm: row counts of the inputs differ")
+    if zero_cell:
+        # dense outputs shaped like states_4d with its last dimension cut to D_gate
+        out_cell = torch.empty((rows, d_gate), dtype=dtype, device=states_4d.device)
+        out_state = torch.empty((rows, d_gate), dtype=dtype, device=states_4d.device)
+        flat = states_4d.dim() == 2
+        shape = states_4d.shape[:-1] + (d_gate,)
+        out_cell_orig = out_cell if flat else out_cell.view(shape)
+        out_state_orig = out_state if flat else out_state.view(shape)
+    else:
+        # outputs inherit prev_cell's row pitch (reference :356-365)
+        out_cell = torch.empty_strided(p2.size(), p2.stride(), dtype=dtype, device=p2.device)
+        out_state = torch.empty_strided(p2.size(), p2.stride(), dtype=dtype, device=p2.device)
+        _check(out_cell.stride(0) == out_state.stride(0), "sum_lstm: internal - output strides mismatch")
+        flat = prev_cell_d.dim() == 2
+        out_cell_orig = out_cell if flat else out_cell.view(prev_cell_d.size())
+        out_state_orig = out_state if flat else out_state.view(prev_cell_d.size())
     if rows == 0:
         return out_state_orig, out_cell_orig
 
     def ptr(t):
         return t.data_ptr() if t is not None else None
 
+    pc_stride = 0 if zero_cell else p2.stride(0)
     entry = lib.arctic_sum_lstm_shared_z if _shared_z else lib.arctic_sum_lstm
     with _on_device_of(states_4d):
         if _token_ids is not None:
             rc = lib.arctic_sum_lstm_embedded(
                 out_state.data_ptr(), out_cell.data_ptr(), s2.data_ptr(), z4_4d.data_ptr(), _token_ids.data_ptr(),
-                p2.data_ptr(), ptr(w_cell), ptr(b_cell), ptr(w_state), ptr(b_state),
-                rows, d_gate, s2.stride(0), z4_4d.stride(0), p2.stride(0), out_cell.stride(0), z4_4d.size(0),
+                ptr(p2), ptr(w_cell), ptr(b_cell), ptr(w_state), ptr(b_state),
+                rows, d_gate, s2.stride(0), z4_4d.stride(0), pc_stride, out_cell.stride(0), z4_4d.size(0),
                 float(alpha), float(eps_cell), float(eps_state), int(bool(use_fast_gelu)),
                 _HALF_DTYPES[dtype], _stream_of(states_4d))
         else:
             rc = entry(
-                out_state.data_ptr(), out_cell.data_ptr(), s2.data_ptr(), z2.data_ptr(), p2.data_ptr(),
+                out_state.data_ptr(), out_cell.data_ptr(), s2.data_ptr(), z2.data_ptr(), ptr(p2),
                 ptr(w_cell), ptr(b_cell), ptr(w_state), ptr(b_state),
-                rows, d_gate, s2.stride(0), z2.stride(0), p2.stride(0), out_cell.stride(0),
+                rows, d_gate, s2.stride(0), z2.stride(0), pc_stride, out_cell.stride(0),
                 float(alpha), float(eps_cell), float(eps_state), int(bool(use_fast_gelu)),
                 _HALF_DTYPES[dtype], _stream_of(states_4d))
     _native.check(rc)
     return out_state_orig, out_cell_orig
+
+
+def _sum_lstm_zero_cell_impl(states_4d, z4_4d, w_cell, b_cell, w_state, b_state, alpha, eps_cell, eps_state,
+                             use_fast_gelu):
+    """sum_lstm with the cell of zeros every proposal round starts from
+    (arctic_inference/vllm/spec_dec/arctic_speculator.py:899-903) implied instead of passed."""
+    return _sum_lstm_impl(states_4d, z4_4d, None, w_cell, b_cell, w_state, b_state, alpha, eps_cell, eps_state,
+                          use_fast_gelu)
 
 
 def _sum_lstm_shared_z_impl(states_4d, z_d, prev_cell_d, w_cell, b_cell, w_state, b_state, alpha, eps_cell,
@@ -666,6 +688,7 @@ _IMPLS = {
     "reshape_and_cache_flash_fp4": _reshape_and_cache_flash_fp4_impl,
     "speculator_ln_cuda": _speculator_ln_impl,
     "sum_lstm_cuda": _sum_lstm_impl,
+    "sum_lstm_zero_cell_cuda": _sum_lstm_zero_cell_impl,
 }
 
 
@@ -680,7 +703,15 @@ def _meta_sum_lstm_embedded(states_4d, emb_weight, token_ids, prev_cell_d, *args
     return _meta_sum_lstm(states_4d, emb_weight, prev_cell_d)
 
 
+def _meta_sum_lstm_zero_cell(states_4d, z4_4d, *args):
+    return _meta_sum_lstm(states_4d, z4_4d, None)
+
+
 def _meta_sum_lstm(states_4d, z, prev_cell_d, *args):
+    if prev_cell_d is None:
+        shape = states_4d.shape[:-1] + (states_4d.size(-1) // 4,)
+        return (torch.empty(shape, dtype=states_4d.dtype, device=states_4d.device),
+                torch.empty(shape, dtype=states_4d.dtype, device=states_4d.device))
     p2 = prev_cell_d.view(-1, prev_cell_d.size(-1))
     make = lambda: torch.empty_strided(p2.size(), p2.stride(), dtype=p2.dtype, device=p2.device).view(prev_cell_d.size())
     return make(), make()
@@ -696,6 +727,7 @@ def _meta_nothing(*args):
 
 _META_IMPLS = {
     "speculator_ln_cuda": _meta_like_input,
+    "sum_lstm_zero_cell_cuda": _meta_sum_lstm_zero_cell,
     "speculator_add_ln_act_cuda": _meta_like_input,
     "sum_lstm_cuda": _meta_sum_lstm,
     "sum_lstm_shared_z_cuda": _meta_sum_lstm,
@@ -852,7 +884,7 @@ def speculator_ln(
 def sum_lstm(
     states_4d: torch.Tensor,
     z4_4d: torch.Tensor,
-    prev_cell_d: torch.Tensor,
+    prev_cell_d: Optional[torch.Tensor],
     w_cell: Optional[torch.Tensor],
     b_cell: Optional[torch.Tensor],
     w_state: Optional[torch.Tensor],
@@ -862,6 +894,14 @@ def sum_lstm(
     eps_state: float,
     use_fast_gelu: bool,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """The reference's wrapper (arctic_inference/py_custom_ops.py:101-117).  Beyond it, ``prev_cell_d=None``
+    stands for the cell of zeros a proposal round starts from (arctic_speculator.py:899-903): same result as
+    a zero tensor bit for bit, but no tensor is made, cleared or read; the outputs are then dense and shaped
+    like ``states_4d`` with its last dimension divided by four.  ``sum_lstm_shared_z`` and
+    ``sum_lstm_embedded`` take None the same way."""
+    if prev_cell_d is None:
+        return _call("sum_lstm_zero_cell_cuda", states_4d, z4_4d, w_cell, b_cell, w_state, b_state, alpha, eps_cell,
+                     eps_state, use_fast_gelu)
     return _call("sum_lstm_cuda", states_4d, z4_4d, prev_cell_d, w_cell, b_cell, w_state, b_state,
                                 alpha, eps_cell, eps_state, use_fast_gelu)
 
@@ -869,7 +909,7 @@ def sum_lstm(
 def sum_lstm_shared_z(
     states_4d: torch.Tensor,
     z_d: torch.Tensor,
-    prev_cell_d: torch.Tensor,
+    prev_cell_d: Optional[torch.Tensor],
     w_cell: Optional[torch.Tensor],
     b_cell: Optional[torch.Tensor],
     w_state: Optional[torch.Tensor],
@@ -891,7 +931,7 @@ def sum_lstm_embedded(
     states_4d: torch.Tensor,
     emb_weight: torch.Tensor,
     token_ids: torch.Tensor,
-    prev_cell_d: torch.Tensor,
+    prev_cell_d: Optional[torch.Tensor],
     w_cell: Optional[torch.Tensor],
     b_cell: Optional[torch.Tensor],
     w_state: Optional[torch.Tensor],

@@ -84,6 +84,14 @@ def _as_int32(tokens) -> np.ndarray:
     return np.ascontiguousarray(tokens, dtype=np.int32)
 
 
+def _require_int32_vector(tokens, what: str) -> None:
+    """The reference's binding takes nb::ndarray<int32_t, nb::ndim<1>, nb::c_contig> (csrc/suffix_decoding/bindings.cc:79-102)
+    and turns anything else away; here the array's memory is handed to C as it is, so the same must hold."""
+    if not (isinstance(tokens, np.ndarray) and tokens.dtype == np.int32 and tokens.ndim == 1
+            and tokens.flags["C_CONTIGUOUS"]):
+        raise TypeError(f"{what}: expected a C-contiguous 1-D numpy array of int32")
+
+
 def _check(rc: int, what: str) -> int:
     if rc < 0:
         raise MemoryError(f"{what}: out of memory") if rc == -2 else ValueError(f"{what}: invalid argument")
@@ -124,6 +132,7 @@ class SuffixTree:
         self.extend_ndarray(seq_id, _as_int32(tokens))
 
     def extend_ndarray(self, seq_id: int, tokens: np.ndarray) -> None:
+        _require_int32_vector(tokens, "extend_ndarray")
         _check(_lib.arctic_suffix_tree_extend(self._handle, seq_id, tokens.ctypes.data, tokens.size), "extend")
 
     def remove(self, seq_id: int) -> None:
@@ -136,6 +145,7 @@ class SuffixTree:
 
     def speculate_ndarray(self, context: np.ndarray, max_spec_tokens: int, max_spec_factor: float,
                           max_spec_offset: float, min_token_prob: float, use_tree_spec: bool) -> Draft:
+        _require_int32_vector(context, "speculate_ndarray")
         max_spec_tokens = int(max_spec_tokens)
         if max_spec_tokens > self._capacity:
             self._reserve(max_spec_tokens)

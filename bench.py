@@ -193,28 +193,66 @@ def cpu_baseline_bulk(w: BulkWorkload, target_seconds=10.0):
         "value": round(passes * nbytes / total_dt / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
         "sample": f"{passes} passes over {tokens} of {w.T} tokens x {L} layers of the same workload "
                   f"({passes * nbytes / 1e6:.0f} MB algorithmic) in {total_dt:.2f} s, C oracle with OpenMP",
+        "cpu_model": cpu_model(),
+        "note": "the reference has no CPU implementation of the bulk write (its fallback, llama_swiftkv.py:623-650, is "
+                "vLLM's CUDA operator), so a port of its kernel is the only CPU form there is; the speculator operators, "
+                "which do have a PyTorch fallback in the reference, are timed both ways in extras.speculator.cpu_baseline",
     }
 
 
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline_speculator():
-    """The CPU oracle (C, OpenMP) on the speculator workload: sum_lstm and speculator_ln at 512 x 4096 bf16."""
+    """CPU baselines of the speculator operators at 512 x 4096 bf16, two kinds side by side:
+    "pytorch": the reference's own PyTorch fallback (arctic_speculator.py:92-99, 784-806, restated in
+    oracle/torch_fallback.py), in bf16 on the host cores with torch's intra-op threads - the CPU path the reference has;
+    "port": the C oracle (OpenMP), a port of the reference's CUDA kernels."""
     import oracle
+    from oracle.torch_fallback import speculator_ln_fallback, sum_lstm_fallback
     T, Hd = 512, 4096
     g = torch.Generator().manual_seed(3)
     rn = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16)
     s4, z4, pc, x = rn(T, 4 * Hd), rn(T, 4 * Hd), rn(T, Hd), rn(T, Hd)
     w, b = (1 + 0.02 * torch.randn(Hd, generator=g)).to(torch.bfloat16), (0.02 * torch.randn(Hd, generator=g)).to(torch.bfloat16)
-    out = {"cores": oracle.num_threads(), "kind": "port"}
-    for name, fn in (("sum_lstm", lambda: oracle.sum_lstm(s4, z4, pc, w, b, w, b, 23.07, 1e-6, 1e-6, False)),
-                     ("speculator_ln", lambda: oracle.speculator_ln(x, w, b, 1e-6))):
+    sw = 0.5 ** (0.5 / 3)
+    alpha = ((1 - sw * sw) * (Hd / 2)) ** 0.5 / sw
+
+    def time_calls(fn, seconds):
         fn()
         times = []
-        t_end = time.perf_counter() + 1.0
+        t_end = time.perf_counter() + seconds
         while time.perf_counter() < t_end or len(times) < 5:
             t0 = time.perf_counter()
             fn()
             times.append(time.perf_counter() - t0)
-        out[name + "_us_per_call"] = round(statistics.median(times) * 1e6, 1)
+        return round(statistics.median(times) * 1e6, 1), len(times)
+
+    out = {"cpu_model": cpu_model(), "host_cores_visible": os.cpu_count()}
+    port = {"kind": "port", "cores": oracle.num_threads(), "what": "C oracle with OpenMP (a port of the reference's kernels)"}
+    for name, fn in (("sum_lstm", lambda: oracle.sum_lstm(s4, z4, pc, w, b, w, b, alpha, 1e-6, 1e-6, False)),
+                     ("speculator_ln", lambda: oracle.speculator_ln(x, w, b, 1e-6))):
+        port[name + "_us_per_call"], _ = time_calls(fn, 1.0)
+    out["port"] = port
+    threads = torch.get_num_threads()
+    pt = {"kind": "pytorch", "cores": threads, "dtype": "bf16",
+          "what": "the reference's PyTorch fallback (arctic_speculator.py:92-99, 784-806) on CPU tensors, "
+                  f"torch {torch.__version__}, {threads} intra-op threads"}
+    with torch.no_grad():
+        for name, fn in (("sum_lstm", lambda: sum_lstm_fallback(s4, z4, pc, w, b, w, b, alpha, 1e-6, 1e-6, False)),
+                         ("speculator_ln", lambda: speculator_ln_fallback(x, w, b, 1e-6))):
+            pt[name + "_us_per_call"], calls = time_calls(fn, 4.0)
+            pt[name + "_calls_timed"] = calls
+    pt["sample"] = "whole calls at the full 512 x 4096 shape, median of the calls made in about 4 s per operator"
+    out["pytorch"] = pt
     return out
 
 
@@ -599,13 +637,18 @@ def box_reference(dev):
 
 
 def bench_decode_mix(ops, dev, steps):
-    """Decode-step workload: 512 decode tokens; bulk fp8 KV write over 16 layers into
-    32768-block caches, ln0, three sum_lstm steps; one HIP graph per step."""
-    w = BulkWorkload("decode", 512, 16, 8, 128, 16, 32768, "fp8", 0.0, 4, 1.5, dev)
-    T, Hd = 512, 4096
+    """Decode-step workload: 512 decode tokens; bulk fp8 KV write over 16 layers into 32768-block caches, ln0, three
+    sum_lstm steps; one HIP graph per step.  Eight sets of everything that is read (K/V rows, slots, ln0 input,
+    pre-activations; 1.2 GB in all) rotate between replays so that no input is served from the 256 MB last-level
+    cache; the caches (17 GB) are shared, they are only written.  The first sum_lstm takes prev_cell=None (the cell
+    of zeros a proposal round starts from) unless `as_the_caller_issues_it`, where a zero tensor is cleared and
+    passed as the reference's caller does."""
+    sets, T, Hd = 8, 512, 4096
+    ws = [BulkWorkload("decode", 512, 16, 8, 128, 16, 32768, "fp8", 0.0, 4 + i, 1.5, dev) for i in range(1)]
+    for i in range(1, sets):
+        ws.append(BulkWorkload("decode", 512, 16, 8, 128, 16, 32768, "fp8", 0.0, 4 + i, 1.5, dev, bufs=ws[0].bufs))
     g = torch.Generator(device=dev).manual_seed(4)
     rn = lambda *s: torch.randn(*s, generator=g, device=dev).to(torch.bfloat16)
-    sets = 4
     S = [[rn(T, 4 * Hd) for _ in range(3)] for _ in range(sets)]
     Z = [[rn(T, 4 * Hd) for _ in range(3)] for _ in range(sets)]
     X = [rn(T, Hd) for _ in range(sets)]
@@ -613,32 +656,130 @@ def bench_decode_mix(ops, dev, steps):
     w_cell, b_cell, w_state, b_state = vec(1.0), vec(0.0), vec(1.0), vec(0.0)
     sw = 0.5 ** (0.5 / 3)
     alpha = ((1 - sw * sw) * (Hd / 2)) ** 0.5 / sw
+    nbytes = ws[0].bytes + 4 * Hd * T + 3 * 22 * Hd * T
 
-    def step(i):
-        ops.reshape_and_cache_flash_bulk(*w.args())
+    def step(i, zero_tensor):
+        ops.reshape_and_cache_flash_bulk(*ws[i].args())
         ops.speculator_ln(X[i], None, None, 1e-6)
-        cell = torch.zeros(T, Hd, dtype=torch.bfloat16, device=dev)
+        cell = torch.zeros(T, Hd, dtype=torch.bfloat16, device=dev) if zero_tensor else None
         for k in range(3):
             _, cell = ops.sum_lstm(S[i][k], Z[i][k], cell, w_cell, b_cell, w_state, b_state, alpha, 1e-6, 1e-6,
                                    False)
 
-    step(0)
+    out = {"bytes_per_step": nbytes, "sets_in_rotation": sets}
+    for name, zero_tensor in (("", False), ("_as_the_caller_issues_it", True)):
+        step(0, zero_tensor)
+        torch.cuda.synchronize()
+        graphs = []
+        for i in range(sets):
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                step(i, zero_tensor)
+            graphs.append(gr)
+        for gr in graphs:
+            gr.replay()
+        torch.cuda.synchronize()
+        counter = iter(range(10 ** 9))
+        us = event_times_us(lambda: graphs[next(counter) % sets].replay(), max(40, steps))
+        med = statistics.median(us)
+        # the same graphs replayed back to back, one pair of events around all of them: per step, without the
+        # idle gap in front of a lone replay
+        def all_sets():
+            for gr in graphs:
+                gr.replay()
+        b2b = statistics.median(event_times_us(all_sets, max(10, steps // 4))) / sets
+        out.update({f"us_per_step_graph{name}": round(med, 2), f"GBps{name}": round(nbytes / med / 1e3, 1),
+                    f"hbm_frac{name}": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4),
+                    f"us_per_step_graphs_back_to_back{name}": round(b2b, 2),
+                    f"hbm_frac_back_to_back{name}": round(nbytes / b2b / 1e3 / HBM_PEAK_GBS, 4)})
+        del graphs
+    return out
+
+
+def bench_bulk_auto(ops, dev, steps):
+    """The bf16 (`auto`) cache path: 8192 algorithmic bytes per valid token and layer (4n read, 4n written).
+    config_1: 256 tokens x 16 layers into 512-block caches (33.5 MB per launch), eight sets of sources and caches
+    (4.4 GB) rotating inside one HIP graph so that nothing is cache resident; 70B shape: 16384 tokens x 40 layers, 10 %
+    padding, 8192-block bf16 caches (21 GB), compact placement, event-timed launches."""
+    out = {}
+    sets = 8
+    ws = [BulkWorkload("config-1", 256, 16, 8, 128, 16, 512, "auto", 0.0, 100 + i, 1.0, dev) for i in range(sets)]
+
+    def run():
+        for w in ws:
+            ops.reshape_and_cache_flash_bulk(*w.args())
+    run()
     torch.cuda.synchronize()
-    graphs = []
-    for i in range(sets):
-        gr = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(gr):
-            step(i)
-        graphs.append(gr)
-    for gr in graphs:
-        gr.replay()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run()
+    for _ in range(3):
+        graph.replay()
     torch.cuda.synchronize()
-    counter = iter(range(10 ** 9))
-    us = event_times_us(lambda: graphs[next(counter) % sets].replay(), max(40, steps))
-    med = statistics.median(us)
-    nbytes = w.bytes + 4 * Hd * T + 3 * 22 * Hd * T
-    return {"us_per_step_graph": round(med, 2), "bytes_per_step": nbytes,
-            "GBps": round(nbytes / med / 1e3, 1), "hbm_frac": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
+    us = statistics.median(event_times_us(graph.replay, max(10, steps // 2))) / sets
+    out["config_1_256_tokens_16_layers"] = {"us_per_call_graph": round(us, 2), "bytes_per_call": ws[0].bytes,
+                                            "GBps": round(ws[0].bytes / us / 1e3, 1),
+                                            "hbm_frac": round(ws[0].bytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+    del ws, graph
+    torch.cuda.empty_cache()
+    w = BulkWorkload("70B-auto", 16384, 40, 8, 128, 16, 8192, "auto", 0.10, 2, 1.5, dev)
+    f = lambda: ops.reshape_and_cache_flash_bulk(*w.args())
+    for _ in range(5):
+        f()
+    out["70b_shape_compact_pool"] = dict(kernel_stats(f, steps, w.bytes), bytes_per_call=w.bytes)
+    del w, f
+    torch.cuda.empty_cache()
+    return out
+
+
+def bench_bulk_tp_heads(ops, dev, steps):
+    """The 70B shape as one GPU of a tensor-parallel group sees it: num_kv_heads / TP heads per GPU
+    (llama_swiftkv.py:598), i.e. cache rows of 128, 256 or 512 bytes instead of 1 KiB; fp8, 16384 tokens x 40 layers,
+    10 % padding, 8192-block caches, compact placement."""
+    out = {}
+    for H in (1, 2, 4, 8):
+        w = BulkWorkload(f"70B-{H}-heads", 16384, 40, H, 128, 16, 8192, "fp8", 0.10, 2, 1.5, dev)
+        f = lambda: ops.reshape_and_cache_flash_bulk(*w.args())
+        for _ in range(5):
+            f()
+        out[f"{H}_kv_heads"] = dict(kernel_stats(f, steps, w.bytes), bytes_per_call=w.bytes, cache_row_bytes=H * 128)
+        del w, f
+        torch.cuda.empty_cache()
+    return out
+
+
+def bench_lstm_rows(ops, dev, steps):
+    """sum_lstm at 4096 against the number of rows (tokens) per call: the fixed cost of a launch against the
+    90 112 bytes per row.  Enough buffer sets rotate inside one HIP graph that every call reads from HBM (at least
+    300 MB in rotation, at least eight sets)."""
+    Hd = 4096
+    g = torch.Generator(device=dev).manual_seed(9)
+    rn = lambda *s: torch.randn(*s, generator=g, device=dev).to(torch.bfloat16)
+    vec = lambda m: (m + 0.02 * torch.randn(Hd, generator=g, device=dev)).to(torch.bfloat16)
+    w_cell, b_cell, w_state, b_state = vec(1.0), vec(0.0), vec(1.0), vec(0.0)
+    out = {}
+    for T in (8, 32, 128, 256, 512, 1024, 2048, 4096):
+        per_call = 22 * Hd * T
+        sets = max(8, -(-300 * 2 ** 20 // per_call))
+        sets = min(sets, 256)
+        S, Z, C = [rn(T, 4 * Hd) for _ in range(sets)], [rn(T, 4 * Hd) for _ in range(sets)], [rn(T, Hd) for _ in range(sets)]
+
+        def run():
+            for i in range(sets):
+                ops.sum_lstm(S[i], Z[i], C[i], w_cell, b_cell, w_state, b_state, 23.07, 1e-6, 1e-6, False)
+        run()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            run()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        us = statistics.median(event_times_us(graph.replay, max(10, steps // 2))) / sets
+        out[f"{T}_rows"] = {"us_per_call_graph": round(us, 2), "GBps": round(per_call / us / 1e3, 1),
+                            "hbm_frac": round(per_call / us / 1e3 / HBM_PEAK_GBS, 4), "sets_in_rotation": sets}
+        del S, Z, C, graph
+    return out
 
 
 def bench_speculator_round_glue(ops, dev, steps):
@@ -791,6 +932,10 @@ def placement_sweep(ops, dev, steps):
                 "store_only": {f"{n}_regions": stream_GBps(1, 1, n, pieces * 65536) for n in (1, 2, 3)},
                 "load_2_store_1, loads from one region": {
                     f"stores_to_{n}_regions": stream_GBps(2, 1, n, pieces * 98304) for n in (1, 2, 3)},
+                "load_2_store_1 with the stores scattered as rows of 1 KiB (the bulk write's pattern)": {
+                    f"stores_to_{n}_regions": stream_GBps(3, 1, n, pieces * 98304) for n in (1, 2, 3)},
+                "the same with 16-byte stores (a lane loads 32 adjacent bytes)": {
+                    f"stores_to_{n}_regions": stream_GBps(4, 1, n, pieces * 98304) for n in (1, 2, 3)},
             }
     return out
 
@@ -902,6 +1047,16 @@ def bench_lstm_variants(dev, steps):
     return out
 
 
+# extras that can be run alone with --only
+ONLY = {
+    "decode_mix": lambda ops, dev, a: bench_decode_mix(ops, dev, a.steps),
+    "speculator": lambda ops, dev, a: bench_speculator(ops, dev, a.steps, a.warmup),
+    "sum_lstm_rows_sweep": lambda ops, dev, a: bench_lstm_rows(ops, dev, a.steps),
+    "bulk_auto_bf16_cache": lambda ops, dev, a: bench_bulk_auto(ops, dev, a.steps),
+    "bulk_fp8_70b_tp_sharded_heads_compact_pool": lambda ops, dev, a: bench_bulk_tp_heads(ops, dev, a.steps),
+}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -914,6 +1069,9 @@ def main():
     ap.add_argument("--placement-sweep", action="store_true",
                     help="instead of the benchmark, time the 70B-shape launch with the caches in each 8 GiB chunk "
                          "of the GPU's memory and spread over its regions; prints one JSON object")
+    ap.add_argument("--only", choices=sorted(ONLY), default=None,
+                    help="instead of the benchmark, run one of the extra measurements alone (for profiling it); "
+                         "prints one JSON object")
     ap.add_argument("--lstm-variants", action="store_true",
                     help="instead of the benchmark, time the sum_lstm kernel variants of the tuning build against "
                          "each other and against the traffic-only kernel; prints one JSON object")
@@ -940,22 +1098,27 @@ def main():
     if args.lstm_variants:
         print(json.dumps({"sum_lstm_variants": bench_lstm_variants(dev, args.steps)}), flush=True)
         return
+    if args.only:
+        print(json.dumps({args.only: ONLY[args.only](ops, dev, args)}), flush=True)
+        return
 
     extras = {}
-    if not args.no_extras:
-        # the same shape with nothing else on the GPU: 40 caches of 8192 blocks (10 GiB) right behind the
-        # source, all inside one HBM region
-        wc = BulkWorkload("70B-SwiftKV-compact", 16384, 40, 8, 128, 16, 8192, "fp8", 0.10, 2, 1.5, dev)
-        fc = lambda: ops.reshape_and_cache_flash_bulk(*wc.args())
-        for _ in range(args.warmup):
-            fc()
-        extras["bulk_fp8_70b_compact_pool"] = dict(
-            kernel_stats(fc, args.steps, wc.bytes),
-            placement="source and 40 caches of 8192 blocks allocated first in the process (13 GiB; inside one HBM "
-                      "region when the GPU was idle before)")
-        log(f"compact placement: {extras['bulk_fp8_70b_compact_pool']}")
-        del wc, fc
-        torch.cuda.empty_cache()
+    # the same shape with nothing else on the GPU: 40 caches of 8192 blocks (10 GiB) right behind the
+    # source, all inside one HBM region.  Always measured: the headline's roofline carries both placements.
+    wc = BulkWorkload("70B-SwiftKV-compact", 16384, 40, 8, 128, 16, 8192, "fp8", 0.10, 2, 1.5, dev)
+    fc = lambda: ops.reshape_and_cache_flash_bulk(*wc.args())
+    for _ in range(args.warmup):
+        fc()
+    compact_us = event_times_us(fc, args.steps)
+    compact = {"kernel_us_mean": round(statistics.mean(compact_us), 2), "kernel_us_median": round(statistics.median(compact_us), 2),
+               "GBps": round(wc.bytes / statistics.mean(compact_us) / 1e3, 1),
+               "hbm_frac": round(wc.bytes / statistics.mean(compact_us) / 1e3 / HBM_PEAK_GBS, 4),
+               "placement": "source and 40 caches of 8192 blocks allocated first in the process (13 GiB; inside one HBM "
+                            "region when the GPU was idle before)"}
+    extras["bulk_fp8_70b_compact_pool"] = compact
+    log(f"compact placement: {compact}")
+    del wc, fc
+    torch.cuda.empty_cache()
 
     # the map needs 66 + 160 GiB of the 268; should less be free, halve the pool rather than fail
     mem, pool_blocks = None, args.pool_blocks
@@ -1000,6 +1163,14 @@ def main():
     traffic = read_traffic(os.path.join(ROOT, "profiles", "kv_write_bulk_fp8_70b.traffic.txt"))
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "traffic_source": "not measured in this run: carried over from profiles/kv_write_bulk_fp8_70b.traffic.txt "
+                                  "(two rocprofv3 --pmc runs of this command, FETCH_SIZE and WRITE_SIZE scaled by a 1 GiB copy)",
+                "placement": "serving memory map (config.memory_map): the written caches span two of the HBM's three "
+                             "address regions",
+                "achieved_compact": compact["GBps"], "frac_compact": compact["hbm_frac"],
+                "kernel_us_mean_compact": compact["kernel_us_mean"],
+                "placement_compact": "the same launch with only the source and 40 caches of 8192 blocks on the GPU (13 GiB, "
+                                     "one HBM region)",
                 "kernel": "kv_write_bulk_kernel<bf16, e4m3>", "kernel_us_mean": round(kernel_us, 2),
                 "kernel_us_median": round(statistics.median(us), 2),
                 "kernel_us_p10": round(sorted(us)[len(us) // 10], 2),
@@ -1053,7 +1224,12 @@ def main():
         extras["speculator"] = bench_speculator(ops, dev, args.steps, args.warmup)
         if not args.no_cpu:
             extras["speculator"]["cpu_baseline"] = cpu_baseline_speculator()
+        extras["sum_lstm_rows_sweep"] = bench_lstm_rows(ops, dev, args.steps)
+        torch.cuda.empty_cache()
         extras["decode_mix"] = bench_decode_mix(ops, dev, args.steps)
+        torch.cuda.empty_cache()
+        extras["bulk_auto_bf16_cache"] = bench_bulk_auto(ops, dev, args.steps)
+        extras["bulk_fp8_70b_tp_sharded_heads_compact_pool"] = bench_bulk_tp_heads(ops, dev, args.steps)
         extras["swiftkv_select_decode_70b"] = bench_row_gather(ops, dev, args.steps)
         extras["bulk_write_and_select_decode_70b"] = bench_bulk_select(ops, dev, args.steps)
         torch.cuda.empty_cache()

@@ -5,7 +5,7 @@
 //                        states, z4 and prev_cell, two 16-byte stores), one workgroup per row, no arithmetic
 //   floor_stream         load-only, store-only or a 2:1 load:store stream in 64 KiB pieces, the pieces dealt
 //                        round robin over up to three buffers (which the caller places in different regions
-//                        of the HBM)
+//                        of the HBM); the 2:1 stream also with its stores scattered as rows of 1 KiB
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -34,11 +34,27 @@ struct Three {
   char *p[3];
 };
 
-// mode 0: load 64 KiB pieces; 1: store 64 KiB pieces; 2: load 64 KiB, store 32 KiB
-__global__ void stream_kernel(Three src, int nsrc, Three dst, int ndst, int64_t pieces, int mode, unsigned *sink) {
+// mode 0: load 64 KiB pieces; 1: store 64 KiB pieces; 2: load 64 KiB, store 32 KiB; 3: load 64 KiB, store 32 KiB as 32
+// rows of 1 KiB scattered over the destination - the bulk KV write's pattern, contiguous K/V rows in and random
+// 1 KiB cache rows out.  Row g of the stream goes to the row whose low `scatter_bits` bits are those of g times an
+// odd constant (a permutation of every aligned group of 2^scatter_bits rows; the host passes the number of trailing
+// zero bits of the row count).
+__global__ void stream_kernel(Three src, int nsrc, Three dst, int ndst, int64_t pieces, int mode, int scatter_bits,
+                              unsigned *sink) {
   unsigned acc = 0;
   for (int64_t k = blockIdx.x; k < pieces; k += gridDim.x) {
     const u32x4 *from = (const u32x4 *)(src.p[k % nsrc] + (k / nsrc) * 65536);
+    if (mode == 4) {
+      // as mode 3 with 16-byte stores: a lane takes two adjacent 16-byte loads
+      for (int i = threadIdx.x; i < 2048; i += blockDim.x) {
+        const u32x4 v = __builtin_nontemporal_load(from + 2 * i), v2 = __builtin_nontemporal_load(from + 2 * i + 1);
+        const u32x4 w = {v.x ^ v.z, v.y ^ v.w, v2.x ^ v2.z, v2.y ^ v2.w};
+        const unsigned g = (unsigned)k * 32u + (unsigned)i / 64u, mask = (1u << scatter_bits) - 1u;
+        const unsigned row = (g & ~mask) | ((g * 40503u) & mask);
+        __builtin_nontemporal_store(w, (u32x4 *)(dst.p[row % ndst] + (row / ndst) * 1024) + i % 64);
+      }
+      continue;
+    }
     for (int i = threadIdx.x; i < 4096; i += blockDim.x) {
       u32x4 v = {1u, 2u, 3u, (unsigned)i};
       if (mode != 1) v = __builtin_nontemporal_load(from + i);
@@ -47,6 +63,12 @@ __global__ void stream_kernel(Three src, int nsrc, Three dst, int ndst, int64_t 
       if (mode == 2) {
         const u32x2 w = {v.x ^ v.z, v.y ^ v.w};
         __builtin_nontemporal_store(w, (u32x2 *)(dst.p[k % ndst] + (k / ndst) * 32768) + i);
+      }
+      if (mode == 3) {
+        const u32x2 w = {v.x ^ v.z, v.y ^ v.w};
+        const unsigned g = (unsigned)k * 32u + (unsigned)i / 128u, mask = (1u << scatter_bits) - 1u;
+        const unsigned row = (g & ~mask) | ((g * 40503u) & mask);
+        __builtin_nontemporal_store(w, (u32x2 *)(dst.p[row % ndst] + (row / ndst) * 1024) + i % 128);
       }
     }
   }
@@ -65,11 +87,13 @@ extern "C" int floor_lstm_traffic(const void *s, const void *z, const void *pc, 
 // Each buffer must hold ceil(pieces / n) * 64 KiB.  `sink` is 4 bytes of device memory.
 extern "C" int floor_stream(void *const *src, int nsrc, void *const *dst, int ndst, int64_t pieces, int mode,
                             void *sink, void *stream) {
-  if (nsrc < 1 || nsrc > 3 || ndst < 1 || ndst > 3 || pieces <= 0 || mode < 0 || mode > 2 || !sink) return 1;
+  if (nsrc < 1 || nsrc > 3 || ndst < 1 || ndst > 3 || pieces <= 0 || mode < 0 || mode > 4 || !sink) return 1;
   Three a = {}, b = {};
   for (int i = 0; i < nsrc; ++i) a.p[i] = (char *)src[i];
   for (int i = 0; i < ndst; ++i) b.p[i] = (char *)dst[i];
+  if (mode >= 3 && pieces * 32 >= (1LL << 31)) return 1;
+  const int scatter_bits = __builtin_ctzll((unsigned long long)(pieces * 32));
   hipLaunchKernelGGL(stream_kernel, dim3(8192), dim3(256), 0, (hipStream_t)stream, a, nsrc, b, ndst, pieces, mode,
-                     (unsigned *)sink);
+                     scatter_bits, (unsigned *)sink);
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }

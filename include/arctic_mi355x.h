@@ -281,7 +281,9 @@ int arctic_speculator_embed_add_ln_act(void *out, const void *in, const void *em
  * gelu is the exact erf form, or the tanh form when fast_gelu != 0.
  *
  *   states, z4     device; rows of 4*D elements, s_stride / z_stride apart
- *   prev_cell      device; rows of D elements, pc_stride apart
+ *   prev_cell      device; rows of D elements, pc_stride apart.  NULL = a cell of zeros, which is what the
+ *                  speculator starts every proposal round from (arctic_speculator.py:899-903): the result is that
+ *                  of a zero tensor bit for bit, without the tensor, its clearing or its read; pc_stride is ignored
  *   out_state, out_cell   device; rows of D elements, out_stride apart
  *   w_cell, b_cell, w_state, b_state   device [>= D] or NULL
  * All strides are in ELEMENTS.  dtype is F16 or BF16.

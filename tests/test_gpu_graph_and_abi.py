@@ -230,3 +230,40 @@ def test_operators_trace_under_torch_compile(ops, backend):
     assert torch.equal(out, k * 2)
     for a, b in zip(traced, eager):
         assert torch.equal(a, b) and a.any()
+
+
+def test_reference_schemas_through_the_dispatcher(ops):
+    """One eager call of each of the reference's four operators as torch.ops.arctic_inference.<op> (schema parsing,
+    dispatch on the CUDA key, the shim), compared with the oracle."""
+    t = torch.ops.arctic_inference
+    for kv in ("fp8", "auto"):
+        case = make_bulk_case(T=130, L=5, H=8, D=128, bs=16, NB=16, kv_cache_dtype=kv, seed=80, std=1.5, pad_fraction=0.1)
+        d = bulk_case_to(case, DEV)
+        assert t.reshape_and_cache_flash_bulk(*bulk_args(d)) is None
+        torch.cuda.synchronize()
+        oracle.reshape_and_cache_flash_bulk(*bulk_args(case))
+        assert_bulk_equal(d["bufs"], case["bufs"])
+    c = make_lstm_case(rows=40, D=512, seed=81)
+    dc = {k: None if v is None else v.to(DEV) for k, v in c.items()}
+    state, cell = t.sum_lstm_cuda(dc["states"], dc["z4"], dc["prev_cell"], dc["w_cell"], dc["b_cell"], dc["w_state"],
+                                  dc["b_state"], 0.35, 1e-6, 1e-6, False)
+    want_state, want_cell = oracle.sum_lstm(c["states"], c["z4"], c["prev_cell"], c["w_cell"], c["b_cell"], c["w_state"],
+                                            c["b_state"], 0.35, 1e-6, 1e-6, False)
+    assert_close(state, want_state, what="state")
+    assert_close(cell, want_cell, what="cell")
+    y = t.speculator_ln_cuda(dc["prev_cell"], dc["w_cell"], dc["b_cell"], 1e-6)
+    assert_close(y, oracle.speculator_ln(c["prev_cell"], c["w_cell"], c["b_cell"], 1e-6), what="norm")
+    T, H, D, bs, NB = 48, 4, 64, 16, 4
+    g = torch.Generator().manual_seed(82)
+    key, value = torch.randn(T, H, D, generator=g).bfloat16(), torch.randn(T, H, D, generator=g).bfloat16()
+    slots = torch.randperm(NB * bs, generator=g)[:T]
+    caches = [torch.zeros(NB, bs, H, D // 2, dtype=torch.uint8) for _ in range(2)] + \
+             [torch.zeros(NB, bs, H, D // 16, dtype=torch.uint8) for _ in range(2)]
+    dcaches = [x.to(DEV) for x in caches]
+    one = torch.ones(())
+    t.reshape_and_cache_flash_fp4(key.to(DEV), value.to(DEV), dcaches[0], dcaches[1], slots.to(DEV), "fp4", one.to(DEV),
+                                  one.to(DEV), dcaches[2], dcaches[3])
+    torch.cuda.synchronize()
+    oracle.reshape_and_cache_flash_fp4(key, value, caches[0], caches[1], caches[2], caches[3], slots, "fp4", one, one)
+    for a, b in zip(dcaches, caches):
+        assert torch.equal(a.cpu(), b)

@@ -1,7 +1,9 @@
 """GPU parity of the bulk KV-cache write against the CPU oracle: bit-exact.
 
-Every call goes torch.ops.arctic_inference.reshape_and_cache_flash_bulk ->
-Python shim -> C ABI of libarctic_mi355x.so.
+The calls go through the module's wrapper functions, as the reference's callers do: for GPU tensors outside
+torch.compile those call the Python shim directly (shim -> C ABI of libarctic_mi355x.so); the same shim is what the
+dispatcher runs for torch.ops.arctic_inference.reshape_and_cache_flash_bulk, which
+tests/test_gpu_graph_and_abi.py::test_reference_schemas_through_the_dispatcher calls explicitly.
 """
 import pytest
 import torch

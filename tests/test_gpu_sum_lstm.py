@@ -214,3 +214,46 @@ def test_random_configurations(ops):
         except AssertionError as e:
             raise AssertionError(f"configuration {it}: rows={rows} D={D} {dtype} pads=({pad4},{padD}) alpha={alpha} "
                                  f"fast={fast}: {e}") from None
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(rows=64, D=4096),                       # the speculator's shape: the kernel that does not read the cell at all
+    dict(rows=5, D=512, wb_cell=False),          # a scale / shift pair missing
+    dict(rows=3, D=8200),                        # two chunks per lane
+    dict(rows=7, D=12),                          # element-wise kernel
+    dict(rows=4, D=128, pad4=7),                 # element-wise kernel through unaligned pitches
+])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("fast", [False, True])
+def test_no_previous_cell_equals_a_cell_of_zeros(ops, cfg, dtype, fast):
+    """prev_cell_d=None (not in the reference's schema) stands for the zero cell every proposal round starts from
+    (arctic_speculator.py:899-903): bit-identical to passing zeros, for all three forms of the operator, and within
+    tolerance of the oracle run on zeros."""
+    c = make_lstm_case(dtype=dtype, seed=77, **cfg)
+    rows, D = cfg["rows"], cfg["D"]
+    d = {k: dev(v) for k, v in c.items()}
+    zeros = torch.zeros(rows, D, dtype=dtype, device=DEV)
+    tail = (d["w_cell"], d["b_cell"], d["w_state"], d["b_state"], 0.35, 1e-6, 1e-5, fast)
+    want = ops.sum_lstm(d["states"], d["z4"], zeros, *tail)
+    got = ops.sum_lstm(d["states"], d["z4"], None, *tail)
+    via_op = torch.ops.arctic_inference.sum_lstm_zero_cell_cuda(d["states"], d["z4"], *tail)
+    for g, v, w in zip(got, via_op, want):
+        assert g.shape == (rows, D) and g.is_contiguous() and torch.equal(g, w) and torch.equal(v, w)
+    o_state, o_cell = oracle.sum_lstm(c["states"], c["z4"], torch.zeros(rows, D, dtype=dtype), c["w_cell"], c["b_cell"],
+                                      c["w_state"], c["b_state"], 0.35, 1e-6, 1e-5, fast)
+    assert_close(got[0], o_state, RTOL, ATOL, "state")
+    assert_close(got[1], o_cell, RTOL, ATOL, "cell")
+    z = d["z4"][:, :D].contiguous()
+    want = ops.sum_lstm_shared_z(d["states"], z, zeros, *tail)
+    got = ops.sum_lstm_shared_z(d["states"], z, None, *tail)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+    table = torch.randn(50, D, generator=torch.Generator().manual_seed(3)).to(dtype).to(DEV)
+    ids = torch.randint(0, 50, (rows,), generator=torch.Generator().manual_seed(4)).to(DEV)
+    want = ops.sum_lstm_embedded(d["states"], table, ids, zeros, *tail)
+    got = ops.sum_lstm_embedded(d["states"], table, ids, None, *tail)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+    # rank-3 states: outputs take their leading dimensions
+    s3 = d["states"][: rows - rows % 1].contiguous().view(rows, 1, 4 * D) if d["states"].is_contiguous() else None
+    if s3 is not None:
+        g3 = ops.sum_lstm(s3, d["z4"].contiguous().view(rows, 1, 4 * D), None, *tail)
+        assert g3[0].shape == (rows, 1, D) and torch.equal(g3[1].view(rows, D), ops.sum_lstm(d["states"], d["z4"], zeros, *tail)[1])

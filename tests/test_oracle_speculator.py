@@ -289,3 +289,30 @@ def test_glue_rejects_unknown_modes():
         oracle.speculator_add_ln_act(x, None, None, None, 0.0, 1e-6, "none", 1.0)   # fp32
     with pytest.raises(KeyError):
         oracle.speculator_add_ln_act(x.bfloat16(), None, None, None, 0.0, 1e-6, "relu", 1.0)
+
+
+def test_reference_pytorch_fallbacks_agree_with_the_oracle():
+    """The reference's own PyTorch fallback (what it runs without its compiled operators, and what the benchmark
+    times as the CPU baseline of the speculator operators) computes the same function as the C oracle: in fp32 it
+    agrees to rounding, in bf16 (every intermediate rounded) within a few bf16 ulps."""
+    from oracle.torch_fallback import speculator_ln_fallback, sum_lstm_fallback
+    c = make_lstm_case(rows=24, D=512, seed=91)
+    alpha = 1.3
+    want_state, want_cell = oracle.sum_lstm(c["states"], c["z4"], c["prev_cell"], c["w_cell"], c["b_cell"], c["w_state"],
+                                            c["b_state"], alpha, 1e-6, 1e-6, False)
+    f32 = {k: (None if v is None else v.float()) for k, v in c.items()}
+    st, ce = sum_lstm_fallback(f32["states"], f32["z4"], f32["prev_cell"], f32["w_cell"], f32["b_cell"], f32["w_state"],
+                               f32["b_state"], alpha, 1e-6, 1e-6, False)
+    # the oracle rounds the cell to bf16 before the state phase (sum_lstm.cu:163,174); the fallback in fp32 does not
+    assert_close(ce, want_cell, rtol=4e-3, atol=4e-3, what="fp32 fallback cell")
+    assert_close(st, want_state, rtol=8e-3, atol=8e-3, what="fp32 fallback state")
+    st, ce = sum_lstm_fallback(c["states"], c["z4"], c["prev_cell"], c["w_cell"], c["b_cell"], c["w_state"], c["b_state"],
+                               alpha, 1e-6, 1e-6, False)
+    assert st.dtype == torch.bfloat16 and ce.dtype == torch.bfloat16
+    assert_close(ce, want_cell, rtol=3e-2, atol=3e-2, what="bf16 fallback cell")
+    assert_close(st, want_state, rtol=3e-2, atol=3e-2, what="bf16 fallback state")
+    x = c["prev_cell"]
+    assert_close(speculator_ln_fallback(x.float(), c["w_cell"].float(), c["b_cell"].float(), 1e-6),
+                 oracle.speculator_ln(x, c["w_cell"], c["b_cell"], 1e-6), rtol=4e-3, atol=4e-3, what="fp32 fallback norm")
+    assert_close(speculator_ln_fallback(x, None, None, 1e-6), oracle.speculator_ln(x, None, None, 1e-6), rtol=2e-2,
+                 atol=2e-2, what="bf16 fallback norm")

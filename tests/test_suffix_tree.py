@@ -291,3 +291,18 @@ def test_c_abi_rejects_bad_arguments():
     assert lib.arctic_suffix_tree_speculate(h, ctx.ctypes.data, 2, 4, 1.0, 0.0, 0.1, 0, None, None, None, None, None) == -1
     lib.arctic_suffix_tree_destroy(h)
     lib.arctic_suffix_tree_destroy(None)
+
+
+def test_ndarray_entry_points_turn_away_what_is_not_an_int32_vector():
+    import numpy as np
+    from arcticinference_amd.suffix_decoding import SuffixTree
+    tree = SuffixTree(8)
+    tree.extend_ndarray(0, np.array([1, 2, 3, 1, 2], dtype=np.int32))
+    for bad in (np.array([1, 2, 3], dtype=np.int64), np.zeros((2, 2), dtype=np.int32),
+                np.arange(10, dtype=np.int32)[::2], [1, 2, 3]):
+        with pytest.raises(TypeError):
+            tree.extend_ndarray(1, bad)
+        with pytest.raises(TypeError):
+            tree.speculate_ndarray(bad, 4, 1.0, 0.0, 0.1, False)
+    assert tree.speculate_ndarray(np.array([1, 2], dtype=np.int32), 4, 1.0, 0.0, 0.1, False).token_ids[:1] == [3]
+    assert tree.check_integrity() == ""

@@ -66,14 +66,15 @@ struct BulkParams {
   int64_t out_key_stride_bytes;
   int64_t out_value_stride_bytes;
   int64_t num_out_rows;
-  // Workgroups at or beyond main_blocks serve the index list itself: output row j whose index the row map does
-  // not credit to j (a repeated index, or a source row at or beyond num_tokens) is copied straight from source
-  // row indices[j], so the output equals index_select for every index in [0, num_src_rows).  indices == nullptr:
-  // no such workgroups are launched.
+  // The first index_blocks workgroups serve the index list itself, one output row per lane: output row j whose
+  // index the row map does not credit to j (a repeated index, or a source row at or beyond num_tokens) is copied
+  // straight from source row indices[j], so the output equals index_select for every index in [0, num_src_rows).
+  // A handful of workgroups, first in the grid so that their two dependent lookups overlap the token workgroups'
+  // streaming instead of trailing it.  indices == nullptr: no such workgroups are launched.
   const void *indices;
   int64_t num_tokens;
   int64_t num_src_rows;
-  int64_t main_blocks;
+  unsigned index_blocks;
   int index_is_64;
 };
 
@@ -137,34 +138,50 @@ __device__ __forceinline__ int64_t leftover_source_row(const BulkParams &p, int6
   return t;
 }
 
-// Workgroup `f` beyond the token workgroups: output row j = f / groups_per_token, the same run of layers as a
-// token workgroup would own.  Almost always there is nothing to do (SwiftKV selects each token once).
-template <typename Src, bool kPow2, int kBulkThreads>
-__device__ __forceinline__ void select_leftover_rows(const BulkParams &p, int64_t f) {
-  const int64_t j = f / p.groups_per_token;
-  const int group = (int)(f - j * p.groups_per_token);
-  const int64_t t = leftover_source_row(p, j);
-  if (t < 0) return;
-  const int layer0 = group * p.layers_per_group;
-  const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
-  const int64_t layer_off = (int64_t)layer0 * p.n * Src::kBytes;
-  const char *ksrc = p.keys + t * p.key_stride_bytes + layer_off;
-  const char *vsrc = p.values + t * p.value_stride_bytes + layer_off;
-  char *kout = p.keys_out + j * p.out_key_stride_bytes + layer_off;
-  char *vout = p.values_out + j * p.out_value_stride_bytes + layer_off;
-  const int cpr = p.chunks_per_row;
-  const int total = 2 * nlayers * cpr;
-  for (int c = threadIdx.x; c < total; c += kBulkThreads) {
-    int r, col;
-    if constexpr (kPow2) {
-      r = c >> p.chunk_shift;
-      col = c & (cpr - 1);
-    } else {
-      r = c / cpr;
-      col = c - r * cpr;
+// Index workgroup `b`: its lanes look at output rows b * kThreads ... (one each); almost always none of them is
+// left over (SwiftKV selects each token once) and the workgroup is done after two dependent lookups.  The rows that
+// are left over are listed in LDS and copied by the whole workgroup, all layers of the launch, one row after the other.
+template <int kThreads>
+__device__ __forceinline__ int list_leftover_rows(const BulkParams &p, unsigned b, int64_t (&todo_j)[kThreads],
+                                                  int64_t (&todo_t)[kThreads], int &count) {
+  if (threadIdx.x == 0) count = 0;
+  __syncthreads();
+  const int64_t j = (int64_t)b * kThreads + threadIdx.x;
+  if (j < p.num_out_rows) {
+    const int64_t t = leftover_source_row(p, j);
+    if (t >= 0) {
+      const int k = atomicAdd(&count, 1);
+      todo_j[k] = j;
+      todo_t[k] = t;
     }
-    const int64_t off = ((int64_t)(r >> 1) * cpr + col) * 16;
-    store16_stream(((r & 1) ? vout : kout) + off, load16_stream(((r & 1) ? vsrc : ksrc) + off));
+  }
+  __syncthreads();
+  return count;
+}
+
+template <typename Src, bool kPow2, int kBulkThreads>
+__device__ __forceinline__ void select_leftover_rows(const BulkParams &p, unsigned b) {
+  __shared__ int64_t todo_j[kBulkThreads], todo_t[kBulkThreads];
+  __shared__ int count;
+  const int n = list_leftover_rows<kBulkThreads>(p, b, todo_j, todo_t, count);
+  const int cpr = p.chunks_per_row;
+  const int total = 2 * p.num_layers * cpr;
+  for (int e = 0; e < n; ++e) {
+    const int64_t j = todo_j[e], t = todo_t[e];
+    const char *ksrc = p.keys + t * p.key_stride_bytes, *vsrc = p.values + t * p.value_stride_bytes;
+    char *kout = p.keys_out + j * p.out_key_stride_bytes, *vout = p.values_out + j * p.out_value_stride_bytes;
+    for (int c = threadIdx.x; c < total; c += kBulkThreads) {
+      int r, col;
+      if constexpr (kPow2) {
+        r = c >> p.chunk_shift;
+        col = c & (cpr - 1);
+      } else {
+        r = c / cpr;
+        col = c - r * cpr;
+      }
+      const int64_t off = ((int64_t)(r >> 1) * cpr + col) * 16;
+      store16_stream(((r & 1) ? vout : kout) + off, load16_stream(((r & 1) ? vsrc : ksrc) + off));
+    }
   }
 }
 
@@ -179,14 +196,16 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
 
   __shared__ RowDesc rows[2 * kLayersPerLaunch];
 
+  unsigned block = blockIdx.x;
   if constexpr (kSelect) {
-    if (blockIdx.x >= p.main_blocks) {  // uniform over the workgroup, before any barrier
-      select_leftover_rows<Src, kPow2, kBulkThreads>(p, blockIdx.x - p.main_blocks);
+    if (block < p.index_blocks) {  // uniform over the workgroup, before any barrier
+      select_leftover_rows<Src, kPow2, kBulkThreads>(p, block);
       return;
     }
+    block -= p.index_blocks;
   }
-  const int64_t token = blockIdx.x / (unsigned)p.groups_per_token;
-  const int group = blockIdx.x - (unsigned)token * (unsigned)p.groups_per_token;
+  const int64_t token = block / (unsigned)p.groups_per_token;
+  const int group = block - (unsigned)token * (unsigned)p.groups_per_token;
   const int layer0 = group * p.layers_per_group;
   const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
 
@@ -299,26 +318,26 @@ template <typename SrcElem, typename Dst>
 __global__ __launch_bounds__(kScalarThreads) void kv_write_bulk_scalar_kernel(
     const BulkParams p, const LayerTables tab, const int src_dtype) {
   constexpr bool kCopy = std::is_same<Dst, Copy>::value;
-  if (blockIdx.x >= p.main_blocks) {  // the index list's own workgroups (select variant only)
-    const int64_t f = blockIdx.x - p.main_blocks;
-    const int64_t j = f / p.groups_per_token;
-    const int group = (int)(f - j * p.groups_per_token);
-    const int64_t t = leftover_source_row(p, j);
-    if (t < 0) return;
-    const int layer0 = group * p.layers_per_group;
-    const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
-    const SrcElem *ks = reinterpret_cast<const SrcElem *>(p.keys + t * p.key_stride_bytes);
-    const SrcElem *vs = reinterpret_cast<const SrcElem *>(p.values + t * p.value_stride_bytes);
-    SrcElem *ko = reinterpret_cast<SrcElem *>(p.keys_out + j * p.out_key_stride_bytes);
-    SrcElem *vo = reinterpret_cast<SrcElem *>(p.values_out + j * p.out_value_stride_bytes);
-    for (int64_t i = (int64_t)layer0 * p.n + threadIdx.x; i < (int64_t)(layer0 + nlayers) * p.n; i += kScalarThreads) {
-      ko[i] = ks[i];
-      vo[i] = vs[i];
+  if (blockIdx.x < p.index_blocks) {  // the index list's own workgroups (select variant only)
+    __shared__ int64_t todo_j[kScalarThreads], todo_t[kScalarThreads];
+    __shared__ int count;
+    const int n = list_leftover_rows<kScalarThreads>(p, blockIdx.x, todo_j, todo_t, count);
+    for (int e = 0; e < n; ++e) {
+      const int64_t j = todo_j[e], t = todo_t[e];
+      const SrcElem *ks = reinterpret_cast<const SrcElem *>(p.keys + t * p.key_stride_bytes);
+      const SrcElem *vs = reinterpret_cast<const SrcElem *>(p.values + t * p.value_stride_bytes);
+      SrcElem *ko = reinterpret_cast<SrcElem *>(p.keys_out + j * p.out_key_stride_bytes);
+      SrcElem *vo = reinterpret_cast<SrcElem *>(p.values_out + j * p.out_value_stride_bytes);
+      for (int64_t i = threadIdx.x; i < (int64_t)p.num_layers * p.n; i += kScalarThreads) {
+        ko[i] = ks[i];
+        vo[i] = vs[i];
+      }
     }
     return;
   }
-  const int64_t token = blockIdx.x / (unsigned)p.groups_per_token;
-  const int group = blockIdx.x - (unsigned)token * (unsigned)p.groups_per_token;
+  const unsigned block = blockIdx.x - p.index_blocks;
+  const int64_t token = block / (unsigned)p.groups_per_token;
+  const int group = block - (unsigned)token * (unsigned)p.groups_per_token;
   const int layer0 = group * p.layers_per_group;
   const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
   const int64_t slot = p.slot_mapping[token];
@@ -574,8 +593,10 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
 #endif
     p.layers_per_group = (count + groups - 1) / groups;
     p.groups_per_token = (count + p.layers_per_group - 1) / p.layers_per_group;
-    p.main_blocks = num_tokens * p.groups_per_token;
-    const int64_t grid = p.main_blocks + (p.indices ? p.num_out_rows * p.groups_per_token : 0);
+    const int lanes = !vec ? kScalarThreads : (wide && p.chunk_shift >= 0) ? 512 : 256;   // of the shape launched below
+    const int64_t index_blocks = p.indices ? (p.num_out_rows + lanes - 1) / lanes : 0;
+    const int64_t grid = num_tokens * p.groups_per_token + index_blocks;
+    p.index_blocks = (unsigned)index_blocks;
     if (grid > 0x7fffffffLL)
       return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: too many tokens (%lld)", fn, (long long)num_tokens);
 

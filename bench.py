@@ -297,6 +297,7 @@ def load_floor_kernels():
     vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
     lib.floor_lstm_traffic.argtypes = [vp, vp, vp, vp, vp, i64, i32, vp]
     lib.floor_stream.argtypes = [vp, i32, vp, i32, i64, i32, vp, vp]
+    lib.floor_valu_rate.argtypes = [i32, i32, i32, vp, vp]
     return lib
 
 
@@ -729,6 +730,20 @@ def bench_bulk_auto(ops, dev, steps):
     out["70b_shape_compact_pool"] = dict(kernel_stats(f, steps, w.bytes), bytes_per_call=w.bytes)
     del w, f
     torch.cuda.empty_cache()
+    # the same launch on the serving map of the headline: 66 GiB of weights, then a bf16 pool of the same size in
+    # bytes (80 layers x [2, 32768, 16, 8, 128] bf16 = 2 GiB each), layers 40-79 written
+    try:
+        mem = ServingMemoryMap(dev, 66, 80, 40, 32768, 16, 8, 128, torch.bfloat16)
+        w = BulkWorkload("70B-auto-serving", 16384, 40, 8, 128, 16, 32768, "auto", 0.10, 2, 1.5, dev, bufs=mem.written_layers())
+        f = lambda: ops.reshape_and_cache_flash_bulk(*w.args())
+        for _ in range(5):
+            f()
+        out["70b_shape_serving_map"] = dict(kernel_stats(f, steps, w.bytes), bytes_per_call=w.bytes,
+                                            memory_map=mem.describe())
+        del mem, w, f
+    except torch.OutOfMemoryError:
+        out["70b_shape_serving_map"] = "not enough free device memory"
+    torch.cuda.empty_cache()
     return out
 
 
@@ -940,6 +955,34 @@ def placement_sweep(ops, dev, steps):
     return out
 
 
+def bench_valu_rates(dev, steps):
+    """Issue cost of vector-ALU operations on this GPU, in nanoseconds per wave-instruction per SIMD, from chains of one
+    operation at 1, 2 and 4 waves per SIMD (bench_floor.hip).  What sum_lstm's arithmetic costs follows from these:
+    a reciprocal or exp2 that stands between full-rate operations costs an issue slot like they do (the
+    transcendental pipe runs beside the main one), so the kernel's arithmetic time is its instruction count, not its
+    count of transcendentals."""
+    floor = load_floor_kernels()
+    if floor is None:
+        return "bench_floor.so is not built"
+    out_buf = torch.zeros(16, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    iters = 4096
+    names = {0: "v_mul_f32", 1: "v_fma_f32", 2: "v_rcp_f32", 3: "v_exp_f32",
+             4: "v_rcp_f32 + 3 dependent full-rate operations (per instruction)", 5: "v_lshlrev_b32"}
+    per_round = {0: 1, 1: 1, 2: 1, 3: 1, 4: 4, 5: 1}
+    out = {"compute_units": cus}
+    for op, name in names.items():
+        row = {}
+        for waves in (1, 2, 4):
+            f = lambda: floor.floor_valu_rate(op, cus * waves, iters, out_buf.data_ptr(), stream)
+            f()
+            us = statistics.median(event_times_us(f, max(5, steps // 10)))
+            row[f"{waves}_waves_per_simd"] = round(us * 1e3 / (iters * 8 * per_round[op] * waves), 2)
+        out[name] = row
+    return out
+
+
 def load_tuning_library():
     """libarctic_tuning_mi355x.so: the library's sources compiled with -DARCTIC_TUNING (`make -C
     arcticinference_amd/csrc tuning`, also done by __graft_entry__.build()), in which environment variables select
@@ -1047,12 +1090,24 @@ def bench_lstm_variants(dev, steps):
     return out
 
 
+def calibration_copy(dev):
+    """A plain 1 GiB device copy: known bytes that a counter run of the same command scales FETCH_SIZE / WRITE_SIZE by."""
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
+
 # extras that can be run alone with --only
 ONLY = {
+    "valu_issue_ns_per_wave_instruction": lambda ops, dev, a: bench_valu_rates(dev, a.steps),
     "decode_mix": lambda ops, dev, a: bench_decode_mix(ops, dev, a.steps),
     "speculator": lambda ops, dev, a: bench_speculator(ops, dev, a.steps, a.warmup),
     "sum_lstm_rows_sweep": lambda ops, dev, a: bench_lstm_rows(ops, dev, a.steps),
     "bulk_auto_bf16_cache": lambda ops, dev, a: bench_bulk_auto(ops, dev, a.steps),
+    "bulk_write_and_select_decode_70b": lambda ops, dev, a: bench_bulk_select(ops, dev, a.steps),
     "bulk_fp8_70b_tp_sharded_heads_compact_pool": lambda ops, dev, a: bench_bulk_tp_heads(ops, dev, a.steps),
 }
 
@@ -1099,6 +1154,8 @@ def main():
         print(json.dumps({"sum_lstm_variants": bench_lstm_variants(dev, args.steps)}), flush=True)
         return
     if args.only:
+        if args.calibrate_copy:
+            calibration_copy(dev)
         print(json.dumps({args.only: ONLY[args.only](ops, dev, args)}), flush=True)
         return
 
@@ -1154,12 +1211,7 @@ def main():
     if not args.no_extras:
         extras["bulk_fp8_70b_decode_sizes_serving_map"] = bench_decode_sizes(ops, dev, mem, args.steps)
     if args.calibrate_copy:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        calibration_copy(dev)
     traffic = read_traffic(os.path.join(ROOT, "profiles", "kv_write_bulk_fp8_70b.traffic.txt"))
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,

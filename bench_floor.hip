@@ -3,6 +3,7 @@
 //
 //   floor_lstm_traffic   the loads and stores of sum_lstm (nine 16-byte loads per lane from the rows of
 //                        states, z4 and prev_cell, two 16-byte stores), one workgroup per row, no arithmetic
+//   floor_valu_rate      chains of one vector-ALU operation, for its issue rate per SIMD
 //   floor_stream         load-only, store-only or a 2:1 load:store stream in 64 KiB pieces, the pieces dealt
 //                        round robin over up to three buffers (which the caller places in different regions
 //                        of the HBM); the 2:1 stream also with its stores scattered as rows of 1 KiB
@@ -73,6 +74,53 @@ __global__ void stream_kernel(Three src, int nsrc, Three dst, int ndst, int64_t 
     }
   }
   if (mode == 0 && acc == 0x12345677u) *sink = acc;
+}
+
+// Issue rates of the vector ALU: every lane runs `iters` rounds of eight independent chains of one operation
+// (0 multiply, 1 fused multiply-add, 2 reciprocal, 3 exp2, 4 one reciprocal followed by three dependent full-rate
+// operations, 5 16-bit unpack by shift).  The host times it with 1, 2 and 4 waves per SIMD.
+template <int OP>
+__global__ __launch_bounds__(256) void valu_rate_kernel(float *out, int iters, float seed) {
+  float a[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) a[j] = seed + threadIdx.x * 1e-3f + j;
+  for (int i = 0; i < iters; ++i) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (OP == 0) a[j] = a[j] * 1.0001f;
+      if (OP == 1) a[j] = __builtin_fmaf(a[j], 1.0001f, 0.5f);
+      if (OP == 2) a[j] = __builtin_amdgcn_rcpf(a[j]);
+      if (OP == 3) a[j] = __builtin_amdgcn_exp2f(a[j]);
+      if (OP == 4) {
+        a[j] = __builtin_amdgcn_rcpf(a[j]);
+        a[j] = a[j] * 1.0001f;
+        a[j] = a[j] + 0.25f;
+        a[j] = a[j] * a[j];
+      }
+      if (OP == 5) a[j] = __uint_as_float(__float_as_uint(a[j]) << 1);
+    }
+  }
+  float s = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) s += a[j];
+  if (s == 123.456f) out[0] = s;   // never true: keeps the chains alive
+}
+
+// `blocks` workgroups of 256 lanes (one wave per SIMD of a CU each); returns 0 or an error code.
+extern "C" int floor_valu_rate(int op, int blocks, int iters, void *out, void *stream) {
+  if (blocks <= 0 || iters <= 0 || !out) return 1;
+  const dim3 g((unsigned)blocks), b(256);
+  hipStream_t s = (hipStream_t)stream;
+  switch (op) {
+    case 0: hipLaunchKernelGGL(valu_rate_kernel<0>, g, b, 0, s, (float *)out, iters, 1.5f); break;
+    case 1: hipLaunchKernelGGL(valu_rate_kernel<1>, g, b, 0, s, (float *)out, iters, 1.5f); break;
+    case 2: hipLaunchKernelGGL(valu_rate_kernel<2>, g, b, 0, s, (float *)out, iters, 1.5f); break;
+    case 3: hipLaunchKernelGGL(valu_rate_kernel<3>, g, b, 0, s, (float *)out, iters, 1.5f); break;
+    case 4: hipLaunchKernelGGL(valu_rate_kernel<4>, g, b, 0, s, (float *)out, iters, 1.5f); break;
+    case 5: hipLaunchKernelGGL(valu_rate_kernel<5>, g, b, 0, s, (float *)out, iters, 1.5f); break;
+    default: return 1;
+  }
+  return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 
 extern "C" int floor_lstm_traffic(const void *s, const void *z, const void *pc, void *out_state, void *out_cell,

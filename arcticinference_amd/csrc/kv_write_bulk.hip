@@ -76,6 +76,9 @@ struct BulkParams {
   int64_t num_src_rows;
   unsigned index_blocks;
   int index_is_64;
+#ifdef ARCTIC_TUNING
+  int stores_before_loads;  // measurement build: a batch is converted and stored before the next one is requested
+#endif
 };
 
 struct __align__(16) RowDesc {
@@ -293,6 +296,9 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
   while (c < total) {
     const int cn = c + kUnroll * kBulkThreads;
     uint4 nxt[kUnroll];
+#ifdef ARCTIC_TUNING
+    if (!p.stores_before_loads)
+#endif
     load_batch(cn, nxt);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
@@ -306,6 +312,9 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
         }
       }
     }
+#ifdef ARCTIC_TUNING
+    if (p.stores_before_loads) load_batch(cn, nxt);
+#endif
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) cur[u] = nxt[u];
     c = cn;
@@ -590,6 +599,8 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
 #ifdef ARCTIC_TUNING
     if (const char *e = getenv("ARCTIC_BULK_GROUPS")) groups = std::max(1, std::min(count, atoi(e)));
     if (const char *e = getenv("ARCTIC_BULK_WIDE")) wide = atoi(e) != 0;
+    p.stores_before_loads = 0;
+    if (const char *e = getenv("ARCTIC_BULK_STORES_FIRST")) p.stores_before_loads = atoi(e) != 0;
 #endif
     p.layers_per_group = (count + groups - 1) / groups;
     p.groups_per_token = (count + p.layers_per_group - 1) / p.layers_per_group;

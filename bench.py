@@ -995,7 +995,50 @@ def load_tuning_library():
     vp, i64, i32, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
     lib.arctic_sum_lstm.argtypes = [vp] * 9 + [i64, i32, i64, i64, i64, i64, f32, f32, f32, i32, i32, vp]
     lib.arctic_sum_lstm.restype = i32
+    lib.arctic_reshape_and_cache_flash_bulk.argtypes = [vp, vp, i64, i64, vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i64,
+                                                        i64, i32, i32, vp]
+    lib.arctic_reshape_and_cache_flash_bulk.restype = i32
     return lib
+
+
+def bench_bulk_variants(dev, steps):
+    """A/B of launch variants of the bulk write in the compact placement (70B shape, fp8, 40 caches of 8192 blocks and
+    the source allocated first in this process: one HBM region on an idle GPU), through the tuning build: the order of
+    a batch's stores and the next batch's loads, the workgroup shape, and the number of layer groups per token."""
+    import ctypes
+    tuning = load_tuning_library()
+    if tuning is None:
+        return "libarctic_tuning_mi355x.so is not built"
+    w = BulkWorkload("70B-SwiftKV-compact", 16384, 40, 8, 128, 16, 8192, "fp8", 0.10, 2, 1.5, dev)
+    tab = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+    kc, vc, ks, vs = tab(w.key_caches), tab(w.value_caches), tab(w.k_scales), tab(w.v_scales)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = tuning.arctic_reshape_and_cache_flash_bulk(
+            w.keys.data_ptr(), w.values.data_ptr(), w.keys.stride(0), w.values.stride(0), kc, vc, ks, vs,
+            w.slots.data_ptr(), w.T, w.L, w.H, w.D, w.bs, w.key_caches[0].stride(0), w.NB, 2, 1, stream)
+        assert rc == 0
+
+    cases = [("as shipped (512 lanes x 2 chunks, 2 groups of 20 layers, next loads before this batch's stores)", {}),
+             ("this batch's stores before the next batch's loads", {"ARCTIC_BULK_STORES_FIRST": "1"}),
+             ("256 lanes x 4 chunks", {"ARCTIC_BULK_WIDE": "0"}),
+             ("one group of 40 layers per token", {"ARCTIC_BULK_GROUPS": "1"}),
+             ("4 groups of 10 layers per token", {"ARCTIC_BULK_GROUPS": "4"}),
+             ("8 groups of 5 layers per token", {"ARCTIC_BULK_GROUPS": "8"})]
+    out = {name: [] for name, _ in cases}
+    for _ in range(3):
+        for name, env in cases:
+            for k in ("ARCTIC_BULK_STORES_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS"):
+                os.environ.pop(k, None)
+            os.environ.update(env)
+            for _ in range(3):
+                launch()
+            out[name].append(round(statistics.mean(event_times_us(launch, max(10, steps // 4))), 1))
+    for k in ("ARCTIC_BULK_STORES_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS"):
+        os.environ.pop(k, None)
+    return {name: {"kernel_us_rounds": v, "GBps": round(w.bytes / statistics.mean(v) / 1e3),
+                   "hbm_frac": round(w.bytes / statistics.mean(v) / 1e3 / HBM_PEAK_GBS, 4)} for name, v in out.items()}
 
 
 # ARCTIC_LSTM_VARIANT values of the tuning build (sum_lstm.hip): bits 0-2 = arithmetic / ordering variants,
@@ -1130,6 +1173,9 @@ def main():
     ap.add_argument("--lstm-variants", action="store_true",
                     help="instead of the benchmark, time the sum_lstm kernel variants of the tuning build against "
                          "each other and against the traffic-only kernel; prints one JSON object")
+    ap.add_argument("--bulk-variants", action="store_true",
+                    help="instead of the benchmark, time launch variants of the bulk write in the compact placement "
+                         "through the tuning build; prints one JSON object")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) so that a counter run of this "
                          "command can scale FETCH_SIZE / WRITE_SIZE")
@@ -1152,6 +1198,9 @@ def main():
         return
     if args.lstm_variants:
         print(json.dumps({"sum_lstm_variants": bench_lstm_variants(dev, args.steps)}), flush=True)
+        return
+    if args.bulk_variants:
+        print(json.dumps({"bulk_write_variants_compact_pool": bench_bulk_variants(dev, args.steps)}), flush=True)
         return
     if args.only:
         if args.calibrate_copy:

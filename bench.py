@@ -643,7 +643,8 @@ def bench_decode_mix(ops, dev, steps):
     pre-activations; 1.2 GB in all) rotate between replays so that no input is served from the 256 MB last-level
     cache; the caches (17 GB) are shared, they are only written.  The first sum_lstm takes prev_cell=None (the cell
     of zeros a proposal round starts from) unless `as_the_caller_issues_it`, where a zero tensor is cleared and
-    passed as the reference's caller does."""
+    passed as the reference's caller does.  `kv_write_on_a_second_stream` forks the KV write, which nothing in the
+    step depends on, onto a second stream inside the captured graph."""
     sets, T, Hd = 8, 512, 4096
     ws = [BulkWorkload("decode", 512, 16, 8, 128, 16, 32768, "fp8", 0.0, 4 + i, 1.5, dev) for i in range(1)]
     for i in range(1, sets):
@@ -659,16 +660,28 @@ def bench_decode_mix(ops, dev, steps):
     alpha = ((1 - sw * sw) * (Hd / 2)) ** 0.5 / sw
     nbytes = ws[0].bytes + 4 * Hd * T + 3 * 22 * Hd * T
 
-    def step(i, zero_tensor):
-        ops.reshape_and_cache_flash_bulk(*ws[i].args())
+    side = torch.cuda.Stream()   # default priority
+
+    def step(i, mode):
+        main = torch.cuda.current_stream()
+        if mode == "fork":
+            # the KV write on a second captured stream, beside the speculator's kernels
+            side.wait_stream(main)
+            with torch.cuda.stream(side):
+                ops.reshape_and_cache_flash_bulk(*ws[i].args())
+        else:
+            ops.reshape_and_cache_flash_bulk(*ws[i].args())
         ops.speculator_ln(X[i], None, None, 1e-6)
-        cell = torch.zeros(T, Hd, dtype=torch.bfloat16, device=dev) if zero_tensor else None
+        cell = torch.zeros(T, Hd, dtype=torch.bfloat16, device=dev) if mode == "zeros" else None
         for k in range(3):
             _, cell = ops.sum_lstm(S[i][k], Z[i][k], cell, w_cell, b_cell, w_state, b_state, alpha, 1e-6, 1e-6,
                                    False)
+        if mode == "fork":
+            main.wait_stream(side)
 
     out = {"bytes_per_step": nbytes, "sets_in_rotation": sets}
-    for name, zero_tensor in (("", False), ("_as_the_caller_issues_it", True)):
+    for name, zero_tensor in (("", "chain"), ("_as_the_caller_issues_it", "zeros"),
+                              ("_kv_write_on_a_second_stream", "fork")):
         step(0, zero_tensor)
         torch.cuda.synchronize()
         graphs = []

@@ -157,6 +157,42 @@ struct Chunk<8> {
   __device__ static __forceinline__ Chunk pack(const float (&f)[8]) { return Chunk{pack8<T>(f)}; }
 };
 
+#ifdef ARCTIC_TUNING
+// measurement build only: 8-byte units (4 elements per lane), to time them against the 16-byte ones
+__device__ __forceinline__ uint2 load8(const void *p) {
+  const u32x2 v = *(const ARCTIC_GLOBAL u32x2 *)p;
+  return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ uint2 load8_stream(const void *p) {
+  const u32x2 v = __builtin_nontemporal_load((const ARCTIC_GLOBAL u32x2 *)p);
+  return make_uint2(v.x, v.y);
+}
+template <>
+struct Chunk<4> {
+  static constexpr int kBytes = 8;
+  uint2 v;
+  __device__ static __forceinline__ Chunk zero() { return Chunk{make_uint2(0, 0)}; }
+  __device__ static __forceinline__ Chunk load(const void *p) { return Chunk{load8(p)}; }
+  __device__ static __forceinline__ Chunk load_stream(const void *p) { return Chunk{load8_stream(p)}; }
+  __device__ __forceinline__ void store_stream(void *p) const { store8_stream(p, v); }
+  __device__ __forceinline__ void store(void *p) const {
+    const u32x2 t = {v.x, v.y};
+    *(ARCTIC_GLOBAL u32x2 *)p = t;
+  }
+  template <typename T>
+  __device__ __forceinline__ void unpack(float (&f)[4]) const {
+    f[0] = T::lo(v.x);
+    f[1] = T::hi(v.x);
+    f[2] = T::lo(v.y);
+    f[3] = T::hi(v.y);
+  }
+  template <typename T>
+  __device__ static __forceinline__ Chunk pack(const float (&f)[4]) {
+    return Chunk{make_uint2(T::pack(f[0], f[1]), T::pack(f[2], f[3]))};
+  }
+};
+#endif
+
 // ---- wave64 / workgroup reductions ------------------------------------------
 // DPP butterfly inside each row of 16 lanes, then the four row totals are read
 // with v_readlane.  Every lane returns the same wave total.

@@ -381,7 +381,8 @@ static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 #ifdef ARCTIC_TUNING
 // Measurement build only: ARCTIC_LSTM_VARIANT = variant bits (see sum_lstm_vec_kernel) + 8 for two rows per workgroup
-// + 16 for two chunks per lane (256 lanes per 4096-wide row).  Read at every call.
+// + 16 for two chunks per lane (256 lanes per 4096-wide row), or + 32 for 8-byte chunks (1024 lanes per 4096-wide
+// row).  Read at every call.
 static int lstm_tuning_variant() {
   const char *e = getenv("ARCTIC_LSTM_VARIANT");
   return e ? atoi(e) : 0;
@@ -393,7 +394,8 @@ static void launch_lstm_tuned(const LstmParams &p, int64_t rows, int shape, int 
     case 0: hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, true, 1, kVariant>), one, dim3(threads), 0, s, p); break;
     case 1: hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, true, 2, kVariant>), two, dim3(threads), 0, s, p); break;
     case 2: hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 2, kFastGelu, 512, kSharedZ, true, 1, kVariant>), one, dim3(threads / 2), 0, s, p); break;
-    default: hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 2, kFastGelu, 512, kSharedZ, true, 2, kVariant>), two, dim3(threads / 2), 0, s, p); break;
+    case 3: hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 2, kFastGelu, 512, kSharedZ, true, 2, kVariant>), two, dim3(threads / 2), 0, s, p); break;
+    default: hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 4, 1, kFastGelu, 1024, kSharedZ, true, 1, kVariant>), one, dim3(threads * 2), 0, s, p); break;
   }
 }
 #endif
@@ -418,7 +420,7 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
 #ifdef ARCTIC_TUNING
     if (cpt == 1 && all && threads % 128 == 0 && p.prev_cell) {
       const int v = lstm_tuning_variant();
-      const int shape = (v >> 3) & 3;
+      const int shape = (v >> 3) & 7;   // 4: 8-byte units, twice the lanes (rows of up to 4096)
       switch (v & 7) {
         case 0: launch_lstm_tuned<T, kFastGelu, kSharedZ, 0>(p, rows, shape, threads, s); break;
         case 1: launch_lstm_tuned<T, kFastGelu, kSharedZ, 1>(p, rows, shape, threads, s); break;

@@ -1066,6 +1066,7 @@ LSTM_VARIANTS = [
     (11, "two rows per workgroup + input gate first + early output gate"),
     (16, "two 16-byte chunks per lane (256 lanes per row)"),
     (24, "two chunks per lane and two rows per workgroup"),
+    (34, "8-byte chunks, 1024 lanes per row (twice the waves, half the work each), early output gate"),
 ]
 
 

@@ -298,6 +298,7 @@ def load_floor_kernels():
     lib.floor_lstm_traffic.argtypes = [vp, vp, vp, vp, vp, i64, i32, vp]
     lib.floor_stream.argtypes = [vp, i32, vp, i32, i64, i32, vp, vp]
     lib.floor_valu_rate.argtypes = [i32, i32, i32, vp, vp]
+    lib.floor_node.argtypes = [vp, vp, i32, i32, i32, vp]
     return lib
 
 
@@ -968,6 +969,38 @@ def placement_sweep(ops, dev, steps):
     return out
 
 
+def bench_node_floor(dev, steps):
+    """What one kernel node of a HIP graph costs on this GPU when it moves next to nothing: 64 nodes of 512 workgroups x
+    512 lanes (the speculator operators' launch shape) in one graph, empty, and with one memory round trip each.  The
+    fixed part of every small operator's time."""
+    floor = load_floor_kernels()
+    if floor is None:
+        return "bench_floor.so is not built"
+    blocks, nodes = 512, 64
+    a = torch.zeros(nodes, blocks * 1024, dtype=torch.uint8, device=dev)
+    b = torch.zeros(nodes, blocks * 1024, dtype=torch.uint8, device=dev)
+    out = {}
+    for name, touch in (("empty_kernel", 0), ("one_16_byte_load_and_store_per_workgroup_wave", 1)):
+        def run():
+            stream = torch.cuda.current_stream().cuda_stream
+            for i in range(nodes):
+                floor.floor_node(a[i].data_ptr(), b[i].data_ptr(), blocks, 512, touch, stream)
+        run()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            run()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        us = statistics.median(event_times_us(graph.replay, max(10, steps // 2)))
+        out[name] = {"us_per_node_in_a_graph": round(us / nodes, 2)}
+        us = event_times_us(lambda: floor.floor_node(a[0].data_ptr(), b[0].data_ptr(), blocks, 512, touch,
+                                                     torch.cuda.current_stream().cuda_stream), max(20, steps))
+        out[name]["us_per_eager_launch_between_events"] = round(statistics.median(us), 2)
+    return out
+
+
 def bench_valu_rates(dev, steps):
     """Issue cost of vector-ALU operations on this GPU, in nanoseconds per wave-instruction per SIMD, from chains of one
     operation at 1, 2 and 4 waves per SIMD (bench_floor.hip).  What sum_lstm's arithmetic costs follows from these:
@@ -1159,6 +1192,7 @@ def calibration_copy(dev):
 
 # extras that can be run alone with --only
 ONLY = {
+    "graph_node_floor": lambda ops, dev, a: bench_node_floor(dev, a.steps),
     "valu_issue_ns_per_wave_instruction": lambda ops, dev, a: bench_valu_rates(dev, a.steps),
     "decode_mix": lambda ops, dev, a: bench_decode_mix(ops, dev, a.steps),
     "speculator": lambda ops, dev, a: bench_speculator(ops, dev, a.steps, a.warmup),

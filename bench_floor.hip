@@ -3,6 +3,7 @@
 //
 //   floor_lstm_traffic   the loads and stores of sum_lstm (nine 16-byte loads per lane from the rows of
 //                        states, z4 and prev_cell, two 16-byte stores), one workgroup per row, no arithmetic
+//   floor_node           an empty kernel, or one that makes a single memory round trip: the fixed cost of a node
 //   floor_valu_rate      chains of one vector-ALU operation, for its issue rate per SIMD
 //   floor_stream         load-only, store-only or a 2:1 load:store stream in 64 KiB pieces, the pieces dealt
 //                        round robin over up to three buffers (which the caller places in different regions
@@ -120,6 +121,20 @@ extern "C" int floor_valu_rate(int op, int blocks, int iters, void *out, void *s
     case 5: hipLaunchKernelGGL(valu_rate_kernel<5>, g, b, 0, s, (float *)out, iters, 1.5f); break;
     default: return 1;
   }
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+// What a kernel node costs when it moves (almost) nothing: `touch` = 0 an empty kernel, 1 one 16-byte load and one
+// 16-byte store per lane of the first wave of every workgroup (a first byte's round trip, no bandwidth).
+__global__ void node_floor_kernel(const u32x4 *in, u32x4 *out, int touch) {
+  if (touch && threadIdx.x < 64) out[blockIdx.x * 64 + threadIdx.x] = in[blockIdx.x * 64 + threadIdx.x];
+}
+
+// in / out: blocks * 1 KiB each
+extern "C" int floor_node(const void *in, void *out, int blocks, int threads, int touch, void *stream) {
+  if (blocks <= 0 || threads < 64 || threads > 1024) return 1;
+  hipLaunchKernelGGL(node_floor_kernel, dim3((unsigned)blocks), dim3((unsigned)threads), 0, (hipStream_t)stream,
+                     (const u32x4 *)in, (u32x4 *)out, touch);
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 

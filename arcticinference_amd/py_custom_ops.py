@@ -163,6 +163,10 @@ def _ptr_table(tensors: List[torch.Tensor]):
     return (ctypes.c_void_p * len(tensors))(*map(_data_ptr, tensors))
 
 
+# sets of per-layer cache / scale tensors (by address) whose layers have been compared with layer 0 already
+_validated_layer_sets: dict = {}
+
+
 def _reshape_and_cache_flash_bulk_impl(
     keys: torch.Tensor,
     values: torch.Tensor,
@@ -210,32 +214,40 @@ def _reshape_and_cache_flash_bulk_impl(
     if not (cache_elem == want_elem and value_caches[0].element_size() == want_elem):
         raise RuntimeError(f"reshape_and_cache_flash_bulk: cache element size {cache_elem} does not match "
                            f"kv_cache_dtype '{kv_cache_dtype}' (expected {want_elem})")
-    if kv_code != _native.KV_AUTO:
-        _check({s.dtype for s in k_scales} == {torch.float32} and {s.dtype for s in v_scales} == {torch.float32},
-               "reshape_and_cache_flash_bulk: k_scales / v_scales must be float32")
-    # every layer's K and V view must look like layer 0's: the kernel takes one block stride, block size and
-    # number of blocks for all of them
-    geometry = {(t.dtype, t.stride(0), t.size(0), t.size(1), t.device) for t in key_caches}
-    geometry.update((t.dtype, t.stride(0), t.size(0), t.size(1), t.device) for t in value_caches)
-    if not (len(geometry) == 1):
-        raise RuntimeError("reshape_and_cache_flash_bulk: key and value caches of all layers must share dtype, "
-                           "block stride, number of blocks, block size and device")
-    devices = {key_caches[0].device, values.device, slot_mapping.device, keys.device}
-    if kv_code != _native.KV_AUTO:
-        devices.update(s.device for s in k_scales)
-        devices.update(s.device for s in v_scales)
-    _check(len(devices) == 1, "reshape_and_cache_flash_bulk: all tensors must be on the same device")
+    first = key_caches[0]
+    _check(first.device == keys.device and values.device == keys.device and slot_mapping.device == keys.device,
+           "reshape_and_cache_flash_bulk: all tensors must be on the same device")
     width = num_layers * int(num_heads) * int(head_size)
     if not (keys.dim() == 2 and values.dim() == 2 and keys.size(0) >= num_tokens and values.size(0) >= num_tokens
             and keys.size(1) >= width and values.size(1) >= width):
         raise RuntimeError(f"reshape_and_cache_flash_bulk: keys and values must be 2-D with at least {num_tokens} rows "
                            f"(one per slot) and {width} columns (layers x heads x head_size)")
+    tables = (_ptr_table(key_caches), _ptr_table(value_caches), _ptr_table(k_scales), _ptr_table(v_scales))
+    # Every layer's K and V view must look like layer 0's (the kernel takes one block stride, block size and number
+    # of blocks for all of them), and the scales must be fp32 on the device.  Looking at 4 x num_layers tensors costs
+    # more host time than the rest of the call, and a serving process passes the same tensors every step, so a set of
+    # per-layer tensors, identified by its addresses, is looked at once; after that only layer 0 is compared with
+    # what was seen then.
+    seen_key = tuple(map(bytes, tables))
+    geometry0 = (first.dtype, block_stride, first.size(0), block_size, first.device, kv_code)
+    if _validated_layer_sets.get(seen_key) != geometry0:
+        geometry = {(t.dtype, t.stride(0), t.size(0), t.size(1), t.device) for t in key_caches}
+        geometry.update((t.dtype, t.stride(0), t.size(0), t.size(1), t.device) for t in value_caches)
+        if not (len(geometry) == 1):
+            raise RuntimeError("reshape_and_cache_flash_bulk: key and value caches of all layers must share dtype, "
+                               "block stride, number of blocks, block size and device")
+        if kv_code != _native.KV_AUTO:
+            _check({s.dtype for s in k_scales} == {torch.float32} and {s.dtype for s in v_scales} == {torch.float32},
+                   "reshape_and_cache_flash_bulk: k_scales / v_scales must be float32")
+            _check({s.device for s in k_scales} | {s.device for s in v_scales} == {first.device},
+                   "reshape_and_cache_flash_bulk: all tensors must be on the same device")
+        if len(_validated_layer_sets) >= 64:
+            _validated_layer_sets.clear()
+        _validated_layer_sets[seen_key] = geometry0
 
-    common = (keys.data_ptr(), values.data_ptr(), key_stride, value_stride,
-              _ptr_table(key_caches), _ptr_table(value_caches),
-              _ptr_table(k_scales), _ptr_table(v_scales),
+    common = (keys.data_ptr(), values.data_ptr(), key_stride, value_stride, *tables,
               slot_mapping.data_ptr(), num_tokens, num_layers, int(num_heads), int(head_size),
-              int(block_size), int(block_stride), int(key_caches[0].size(0)), src_code, kv_code)
+              int(block_size), int(block_stride), int(first.size(0)), src_code, kv_code)
     with _on_device_of(keys):
         if _select is None:
             rc = lib.arctic_reshape_and_cache_flash_bulk(*common, _stream_of(keys))

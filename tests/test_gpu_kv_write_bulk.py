@@ -290,3 +290,26 @@ def test_errors(ops):
         ops.reshape_and_cache_flash_bulk(*a[:5], "fp8", *a[6:])            # bf16 cache passed as fp8
     torch.cuda.synchronize()
     assert_bulk_equal(d["bufs"], case["bufs"])                              # nothing was written
+
+
+def test_layers_that_do_not_look_like_layer_0_are_turned_away(ops):
+    """The kernel takes one block stride, block count and block size for all layers; a layer that differs, or a scale
+    that is not an fp32 device tensor, is an error here (the reference would write out of bounds).  A set of layers
+    that passed is remembered by its addresses, so the same wrong set must fail on every call, and a good set must
+    still work after a bad one."""
+    case = make_bulk_case(T=6, L=3, H=2, D=64, bs=16, NB=4, kv_cache_dtype="fp8", seed=21)
+    d = bulk_case_to(case, DEV)
+    a = list(bulk_args(d))
+    small = torch.zeros(2, 2, 16, 2, 64, dtype=torch.uint8, device=DEV)          # 2 blocks instead of 4
+    for _ in range(2):
+        with pytest.raises(RuntimeError, match="must share dtype, block stride, number of blocks"):
+            ops.reshape_and_cache_flash_bulk(a[0], a[1], [a[2][0], small[0], a[2][2]], [a[3][0], small[1], a[3][2]], *a[4:])
+        with pytest.raises(RuntimeError, match="must be float32"):
+            ops.reshape_and_cache_flash_bulk(*a[:6], [a[6][0], a[6][1].double(), a[6][2]], *a[7:])
+        with pytest.raises(RuntimeError, match="same device"):
+            ops.reshape_and_cache_flash_bulk(*a[:7], [a[7][0].cpu(), a[7][1], a[7][2]], *a[8:])
+        with pytest.raises(RuntimeError, match="at least 6 rows"):
+            ops.reshape_and_cache_flash_bulk(a[0][:4], *a[1:])
+        with pytest.raises(RuntimeError, match="384 columns"):
+            ops.reshape_and_cache_flash_bulk(a[0][:, :256], *a[1:])
+    run_both(ops, case)

@@ -58,7 +58,8 @@ struct BulkParams {
   int block_size;
   int chunks_per_row;    // 16-byte source chunks per (token, layer) row
   int chunk_shift;       // log2(chunks_per_row) or -1
-  // select variant: token t's source rows are also copied, unconverted, to row row_map[t] of keys_out /
+  // select variants: token t's source rows are also copied, unconverted, to the rows j of keys_out / values_out with
+  // indices[j] == t.  With a row map (kSelectByRowMap) that is row row_map[t] of keys_out /
   // values_out (already offset to the first layer of this launch); a negative row or one >= num_out_rows = none
   const int64_t *row_map;
   char *keys_out;
@@ -76,10 +77,16 @@ struct BulkParams {
   int64_t num_src_rows;
   unsigned index_blocks;
   int index_is_64;
+  int select_mode;   // kSelectNone / kSelectByRowMap / kSelectByScan (the vector kernels take it as a template argument)
 #ifdef ARCTIC_TUNING
   int stores_before_loads;  // measurement build: a batch is converted and stored before the next one is requested
 #endif
 };
+
+// How a launch finds the output rows of a token: not at all, through the inverse of the index list that the caller
+// built beforehand, or by scanning the index list itself (short lists: one or a few loads per lane, no launch and
+// no workspace for the inverse).
+enum : int { kSelectNone = 0, kSelectByRowMap = 1, kSelectByScan = 2 };
 
 struct __align__(16) RowDesc {
   char *dst;    // first byte of this token's row in the layer's K or V cache
@@ -132,26 +139,28 @@ __device__ __forceinline__ void emit_chunk(const uint4 &v, const RowDesc &d, int
   }
 }
 
-// Which source row output row j wants, or -1 when the token's own workgroup already copies it (the row map
-// credits the token to j) or the index lies outside the source.
+// Which source row output row j wants, or -1 when the token workgroups already copy it or the index lies outside
+// the source.  By row map: the token's workgroup serves the one output row the map credits the token with.  By scan:
+// it serves every output row that names the token, so only source rows beyond the slot mapping are left.
+template <int kSelect>
 __device__ __forceinline__ int64_t leftover_source_row(const BulkParams &p, int64_t j) {
   const int64_t t = p.index_is_64 ? ((const int64_t *)p.indices)[j] : (int64_t)((const int32_t *)p.indices)[j];
   if (t < 0 || t >= p.num_src_rows) return -1;
-  if (t < p.num_tokens && p.row_map[t] == j) return -1;
+  if (t < p.num_tokens && (kSelect == kSelectByScan || p.row_map[t] == j)) return -1;
   return t;
 }
 
 // Index workgroup `b`: its lanes look at output rows b * kThreads ... (one each); almost always none of them is
 // left over (SwiftKV selects each token once) and the workgroup is done after two dependent lookups.  The rows that
 // are left over are listed in LDS and copied by the whole workgroup, all layers of the launch, one row after the other.
-template <int kThreads>
+template <int kThreads, int kSelect>
 __device__ __forceinline__ int list_leftover_rows(const BulkParams &p, unsigned b, int64_t (&todo_j)[kThreads],
                                                   int64_t (&todo_t)[kThreads], int &count) {
   if (threadIdx.x == 0) count = 0;
   __syncthreads();
   const int64_t j = (int64_t)b * kThreads + threadIdx.x;
   if (j < p.num_out_rows) {
-    const int64_t t = leftover_source_row(p, j);
+    const int64_t t = leftover_source_row<kSelect>(p, j);
     if (t >= 0) {
       const int k = atomicAdd(&count, 1);
       todo_j[k] = j;
@@ -162,11 +171,11 @@ __device__ __forceinline__ int list_leftover_rows(const BulkParams &p, unsigned 
   return count;
 }
 
-template <typename Src, bool kPow2, int kBulkThreads>
+template <typename Src, bool kPow2, int kBulkThreads, int kSelect>
 __device__ __forceinline__ void select_leftover_rows(const BulkParams &p, unsigned b) {
   __shared__ int64_t todo_j[kBulkThreads], todo_t[kBulkThreads];
   __shared__ int count;
-  const int n = list_leftover_rows<kBulkThreads>(p, b, todo_j, todo_t, count);
+  const int n = list_leftover_rows<kBulkThreads, kSelect>(p, b, todo_j, todo_t, count);
   const int cpr = p.chunks_per_row;
   const int total = 2 * p.num_layers * cpr;
   for (int e = 0; e < n; ++e) {
@@ -191,7 +200,7 @@ __device__ __forceinline__ void select_leftover_rows(const BulkParams &p, unsign
 // kBulkThreads x kUnroll 16-byte chunks form one batch of a workgroup.  Two shapes
 // are built: 512 x 2 (a workgroup moves two batches or more) and 256 x 4 (decode:
 // few tokens, a single batch per workgroup).
-template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll, bool kSelect>
+template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll, int kSelect>
 __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
     const BulkParams p, const LayerTables tab) {
   constexpr bool kCopy = std::is_same<Dst, Copy>::value;
@@ -202,7 +211,7 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
   unsigned block = blockIdx.x;
   if constexpr (kSelect) {
     if (block < p.index_blocks) {  // uniform over the workgroup, before any barrier
-      select_leftover_rows<Src, kPow2, kBulkThreads>(p, block);
+      select_leftover_rows<Src, kPow2, kBulkThreads, kSelect>(p, block);
       return;
     }
     block -= p.index_blocks;
@@ -246,14 +255,40 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
   // its first batch away.)
   const int64_t slot = p.slot_mapping[token];
   int64_t out_row = -1;
-  if constexpr (kSelect) out_row = p.row_map[token];
+  if constexpr (kSelect == kSelectByRowMap) out_row = p.row_map[token];
+  // by scan: every lane requests its share of the index list ahead of the source rows, like the slot, and compares
+  // it with the token once the first batch is on its way; the output rows that name this token end up in `hits`
+  constexpr int kIndicesPerLane = ARCTIC_SELECT_SCAN_MAX_INDICES / kBulkThreads;
+  __shared__ int hits[kSelect == kSelectByScan ? ARCTIC_SELECT_SCAN_MAX_INDICES : 1];
+  __shared__ int num_hits;
+  int64_t mine[kIndicesPerLane];
+  if constexpr (kSelect == kSelectByScan) {
+#pragma unroll
+    for (int k = 0; k < kIndicesPerLane; ++k) {
+      const int j = threadIdx.x + k * kBulkThreads;
+      mine[k] = -1;   // no token
+      if (j < (int)p.num_out_rows)
+        mine[k] = p.index_is_64 ? ((const int64_t *)p.indices)[j] : (int64_t)((const int32_t *)p.indices)[j];
+    }
+    if (threadIdx.x == 0) num_hits = 0;
+  }
   int c = threadIdx.x;
   uint4 cur[kUnroll];
   load_batch(c, cur);
+  int nhits = 0;
+  if constexpr (kSelect == kSelectByScan) {
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kIndicesPerLane; ++k)
+      if (mine[k] == token) hits[atomicAdd(&num_hits, 1)] = threadIdx.x + k * kBulkThreads;
+    __syncthreads();
+    nhits = num_hits;
+  }
   // padding (or a slot outside the cache) writes no cache row; both tests are uniform over the workgroup
   const bool to_cache = slot >= 0 && slot < p.num_slots;
-  const bool to_out = kSelect && out_row >= 0 && out_row < p.num_out_rows;
-  if (!to_cache && !to_out) return;  // before any barrier
+  const bool to_out = kSelect == kSelectByScan ? nhits > 0
+                                               : (kSelect == kSelectByRowMap && out_row >= 0 && out_row < p.num_out_rows);
+  if (!to_cache && !to_out) return;  // uniform, and behind the scan's barriers
 
   if (to_cache) {
     int64_t blk, off;
@@ -284,11 +319,15 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
     __syncthreads();
   }
   char *kout = nullptr, *vout = nullptr;
-  if constexpr (kSelect) {
+  if constexpr (kSelect == kSelectByRowMap) {
     if (to_out) {
       kout = p.keys_out + out_row * p.out_key_stride_bytes + (int64_t)layer0 * p.n * Src::kBytes;
       vout = p.values_out + out_row * p.out_value_stride_bytes + (int64_t)layer0 * p.n * Src::kBytes;
     }
+  }
+  if constexpr (kSelect == kSelectByScan) {   // the columns of this workgroup's layers; the row is added per hit
+    kout = p.keys_out + (int64_t)layer0 * p.n * Src::kBytes;
+    vout = p.values_out + (int64_t)layer0 * p.n * Src::kBytes;
   }
 
   // software-pipelined main loop: the next batch is in flight while this one
@@ -307,8 +346,16 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
         int r, col;
         locate(cu, r, col);
         if (!kSelect || to_cache) emit_chunk<Src, Dst>(cur[u], rows[r], col);
-        if constexpr (kSelect) {
+        if constexpr (kSelect == kSelectByRowMap) {
           if (to_out) store16_stream(((r & 1) ? vout : kout) + ((int64_t)(r >> 1) * cpr + col) * 16, cur[u]);
+        }
+        if constexpr (kSelect == kSelectByScan) {
+          const int64_t off = ((int64_t)(r >> 1) * cpr + col) * 16;
+          for (int h = 0; h < nhits; ++h) {   // one hit unless the list names the token more than once
+            const int64_t j = hits[h];
+            store16_stream((r & 1) ? vout + j * p.out_value_stride_bytes + off : kout + j * p.out_key_stride_bytes + off,
+                           cur[u]);
+          }
         }
       }
     }
@@ -330,7 +377,9 @@ __global__ __launch_bounds__(kScalarThreads) void kv_write_bulk_scalar_kernel(
   if (blockIdx.x < p.index_blocks) {  // the index list's own workgroups (select variant only)
     __shared__ int64_t todo_j[kScalarThreads], todo_t[kScalarThreads];
     __shared__ int count;
-    const int n = list_leftover_rows<kScalarThreads>(p, blockIdx.x, todo_j, todo_t, count);
+    const int n = p.select_mode == kSelectByScan
+                      ? list_leftover_rows<kScalarThreads, kSelectByScan>(p, blockIdx.x, todo_j, todo_t, count)
+                      : list_leftover_rows<kScalarThreads, kSelectByRowMap>(p, blockIdx.x, todo_j, todo_t, count);
     for (int e = 0; e < n; ++e) {
       const int64_t j = todo_j[e], t = todo_t[e];
       const SrcElem *ks = reinterpret_cast<const SrcElem *>(p.keys + t * p.key_stride_bytes);
@@ -350,13 +399,33 @@ __global__ __launch_bounds__(kScalarThreads) void kv_write_bulk_scalar_kernel(
   const int layer0 = group * p.layers_per_group;
   const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
   const int64_t slot = p.slot_mapping[token];
-  const int64_t out_row = p.row_map ? p.row_map[token] : -1;
+  // output rows of this token: the one the row map names, or all that a scan of the index list finds
+  __shared__ int hits[ARCTIC_SELECT_SCAN_MAX_INDICES];
+  __shared__ int num_hits;
+  int nhits = 0;
+  if (p.select_mode == kSelectByScan) {   // uniform
+    if (threadIdx.x == 0) num_hits = 0;
+    __syncthreads();
+    for (int j = threadIdx.x; j < (int)p.num_out_rows; j += kScalarThreads) {
+      const int64_t t = p.index_is_64 ? ((const int64_t *)p.indices)[j] : (int64_t)((const int32_t *)p.indices)[j];
+      if (t == token) hits[atomicAdd(&num_hits, 1)] = j;
+    }
+    __syncthreads();
+    nhits = num_hits;
+  } else if (p.select_mode == kSelectByRowMap) {
+    const int64_t out_row = p.row_map[token];
+    if (out_row >= 0 && out_row < p.num_out_rows) {
+      if (threadIdx.x == 0) hits[0] = (int)out_row;
+      nhits = 1;
+    }
+    __syncthreads();
+  }
   const bool to_cache = slot >= 0 && slot < p.num_slots;
-  const bool to_out = out_row >= 0 && out_row < p.num_out_rows;
-  if (!to_cache && !to_out) return;
+  if (!to_cache && nhits == 0) return;
   const SrcElem *ks = reinterpret_cast<const SrcElem *>(p.keys + token * p.key_stride_bytes);
   const SrcElem *vs = reinterpret_cast<const SrcElem *>(p.values + token * p.value_stride_bytes);
-  if (to_out) {
+  for (int h = 0; h < nhits; ++h) {
+    const int64_t out_row = hits[h];
     SrcElem *ko = reinterpret_cast<SrcElem *>(p.keys_out + out_row * p.out_key_stride_bytes);
     SrcElem *vo = reinterpret_cast<SrcElem *>(p.values_out + out_row * p.out_value_stride_bytes);
     for (int64_t i = (int64_t)layer0 * p.n + threadIdx.x; i < (int64_t)(layer0 + nlayers) * p.n; i += kScalarThreads) {
@@ -402,7 +471,7 @@ __global__ __launch_bounds__(kScalarThreads) void kv_write_bulk_scalar_kernel(
   }
 }
 
-template <typename Src, typename Dst, bool kSelect>
+template <typename Src, typename Dst, int kSelect>
 static void launch_vec_shape(const BulkParams &p, const LayerTables &tab, int64_t grid, bool wide, hipStream_t s) {
   const dim3 g((unsigned)grid);
   if (p.chunk_shift >= 0) {
@@ -416,8 +485,11 @@ static void launch_vec_shape(const BulkParams &p, const LayerTables &tab, int64_
 }
 template <typename Src, typename Dst>
 static void launch_vec(const BulkParams &p, const LayerTables &tab, int64_t grid, bool wide, hipStream_t s) {
-  if (p.row_map) launch_vec_shape<Src, Dst, true>(p, tab, grid, wide, s);
-  else launch_vec_shape<Src, Dst, false>(p, tab, grid, wide, s);
+  switch (p.select_mode) {
+    case kSelectByScan: launch_vec_shape<Src, Dst, kSelectByScan>(p, tab, grid, wide, s); break;
+    case kSelectByRowMap: launch_vec_shape<Src, Dst, kSelectByRowMap>(p, tab, grid, wide, s); break;
+    default: launch_vec_shape<Src, Dst, kSelectNone>(p, tab, grid, wide, s); break;
+  }
 }
 template <typename SrcElem, typename Dst>
 static void launch_scalar(const BulkParams &p, const LayerTables &tab, int64_t grid, int src_dtype,
@@ -464,13 +536,14 @@ using namespace arctic;
 
 // The rows a launch may also copy out (the select variant); row_map == nullptr: none.
 struct SelectArgs {
-  const int64_t *row_map;
+  int mode;                  // kSelectNone / kSelectByRowMap / kSelectByScan
+  const int64_t *row_map;    // kSelectByRowMap only
   void *keys_out;
   void *values_out;
   int64_t out_key_stride;    // elements
   int64_t out_value_stride;
   int64_t num_out_rows;
-  const void *indices;       // the list row_map inverts (num_out_rows entries), or nullptr
+  const void *indices;       // the index list (num_out_rows entries); with a row map it may be nullptr
   int index_bytes;
   int64_t num_src_rows;      // rows of keys / values an index may name
 };
@@ -498,17 +571,24 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
   if (!keys || !values || !slot_mapping || !key_cache_ptrs || !value_cache_ptrs)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
   SelectArgs sel = sel_in;
-  if (sel.row_map && (sel.num_out_rows < 0 || sel.out_key_stride < 0 || sel.out_value_stride < 0))
-    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: negative number of output rows or row pitch", fn);
-  if (sel.row_map && sel.num_out_rows == 0) sel.row_map = nullptr;   // no row to copy to: the plain write
-  if (sel.row_map && (!sel.keys_out || !sel.values_out))
-    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null keys_out or values_out", fn);
-  if (sel.row_map && sel.indices) {
-    if (sel.index_bytes != 4 && sel.index_bytes != 8)
-      return fail(ARCTIC_ERR_UNSUPPORTED, "%s: indices must be int32 or int64", fn);
-    if (sel.num_src_rows < num_tokens)
-      return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: keys / values have fewer rows (%lld) than slot_mapping (%lld)", fn,
-                  (long long)sel.num_src_rows, (long long)num_tokens);
+  if (sel.mode != kSelectNone) {
+    if (sel.num_out_rows < 0 || sel.out_key_stride < 0 || sel.out_value_stride < 0)
+      return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: negative number of output rows or row pitch", fn);
+    if (sel.num_out_rows == 0) sel.mode = kSelectNone;   // no row to copy to: the plain write
+  }
+  if (sel.mode != kSelectNone) {
+    if (!sel.keys_out || !sel.values_out) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null keys_out or values_out", fn);
+    if (sel.mode == kSelectByRowMap && !sel.row_map) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null row map", fn);
+    if (sel.mode == kSelectByScan && (!sel.indices || sel.num_out_rows > ARCTIC_SELECT_SCAN_MAX_INDICES))
+      return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: the index list is missing or longer than %d entries and there is no row map",
+                  fn, ARCTIC_SELECT_SCAN_MAX_INDICES);
+    if (sel.indices) {
+      if (sel.index_bytes != 4 && sel.index_bytes != 8)
+        return fail(ARCTIC_ERR_UNSUPPORTED, "%s: indices must be int32 or int64", fn);
+      if (sel.num_src_rows < num_tokens)
+        return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: keys / values have fewer rows (%lld) than slot_mapping (%lld)", fn,
+                    (long long)sel.num_src_rows, (long long)num_tokens);
+    }
   }
   const bool quant = kv_cache_dtype != ARCTIC_KV_AUTO;
   if (quant && (!k_scale_ptrs || !v_scale_ptrs))
@@ -533,7 +613,7 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
              ((value_stride * es) % 16 == 0 || num_tokens == 1) && ((block_stride * des) % store_bytes == 0);
   for (int l = 0; vec && l < num_layers; ++l)
     vec = aligned(key_cache_ptrs[l], store_bytes) && aligned(value_cache_ptrs[l], store_bytes);
-  if (vec && sel.row_map)
+  if (vec && sel.mode != kSelectNone)
     vec = aligned(sel.keys_out, 16) && aligned(sel.values_out, 16) &&
           ((sel.out_key_stride * es) % 16 == 0 || sel.num_out_rows <= 1) &&
           ((sel.out_value_stride * es) % 16 == 0 || sel.num_out_rows <= 1);
@@ -553,13 +633,15 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
     p.keys = (const char *)keys + (int64_t)first * n * es;
     p.values = (const char *)values + (int64_t)first * n * es;
     p.slot_mapping = slot_mapping;
-    p.row_map = sel.row_map;
-    p.keys_out = sel.row_map ? (char *)sel.keys_out + (int64_t)first * n * es : nullptr;
-    p.values_out = sel.row_map ? (char *)sel.values_out + (int64_t)first * n * es : nullptr;
+    const bool select = sel.mode != kSelectNone;
+    p.select_mode = sel.mode;
+    p.row_map = sel.mode == kSelectByRowMap ? sel.row_map : nullptr;
+    p.keys_out = select ? (char *)sel.keys_out + (int64_t)first * n * es : nullptr;
+    p.values_out = select ? (char *)sel.values_out + (int64_t)first * n * es : nullptr;
     p.out_key_stride_bytes = sel.out_key_stride * es;
     p.out_value_stride_bytes = sel.out_value_stride * es;
-    p.num_out_rows = sel.row_map ? sel.num_out_rows : 0;
-    p.indices = sel.row_map ? sel.indices : nullptr;
+    p.num_out_rows = select ? sel.num_out_rows : 0;
+    p.indices = select ? sel.indices : nullptr;
     p.index_is_64 = sel.index_bytes == 8;
     p.num_tokens = num_tokens;
     p.num_src_rows = sel.num_src_rows;
@@ -629,7 +711,7 @@ extern "C" int arctic_reshape_and_cache_flash_bulk(
     const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads,
     int head_size, int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype,
     int kv_cache_dtype, void *stream) {
-  const SelectArgs none = {nullptr, nullptr, nullptr, 0, 0, 0, nullptr, 0, 0};
+  const SelectArgs none = {kSelectNone, nullptr, nullptr, nullptr, 0, 0, 0, nullptr, 0, 0};
   return bulk_entry("reshape_and_cache_flash_bulk", keys, values, key_stride, value_stride, key_cache_ptrs,
                     value_cache_ptrs, k_scale_ptrs, v_scale_ptrs, slot_mapping, num_tokens, num_layers, num_heads,
                     head_size, block_size, block_stride, num_blocks, src_dtype, kv_cache_dtype, none, stream);
@@ -645,9 +727,9 @@ extern "C" int arctic_reshape_and_cache_flash_bulk_select(
     int64_t num_src_rows, void *keys_out, void *values_out, int64_t out_key_stride, int64_t out_value_stride,
     void *stream) {
   const char *fn = "reshape_and_cache_flash_bulk_select";
-  if (num_layers != 0 && num_tokens != 0 && !row_map) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null row map", fn);
-  const SelectArgs sel = {row_map, keys_out, values_out, out_key_stride, out_value_stride, num_indices,
-                          indices, index_bytes, num_src_rows};
+  // a row map is used when one is given; without one the token workgroups scan the index list themselves
+  const SelectArgs sel = {row_map ? kSelectByRowMap : kSelectByScan, row_map, keys_out, values_out, out_key_stride,
+                          out_value_stride, num_indices, indices, index_bytes, num_src_rows};
   return bulk_entry(fn, keys, values, key_stride, value_stride, key_cache_ptrs, value_cache_ptrs, k_scale_ptrs,
                     v_scale_ptrs, slot_mapping, num_tokens, num_layers, num_heads, head_size, block_size, block_stride,
                     num_blocks, src_dtype, kv_cache_dtype, sel, stream);
@@ -720,16 +802,17 @@ extern "C" int arctic_reshape_and_cache_flash_bulk_select_static(
                 fn, (long long)num_tokens, ARCTIC_SELECT_STATIC_MAX_TOKENS);
   if (num_indices < 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: negative number of indices", fn);
   if (num_indices > 0 && !indices) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null indices", fn);
+  // short index lists are scanned by the token workgroups and need no row map; longer ones get theirs in `scratch`
   int64_t *row_map = nullptr;
-  if (num_layers != 0 && num_tokens > 0 && num_indices > 0) {
+  if (num_layers != 0 && num_tokens > 0 && num_indices > ARCTIC_SELECT_SCAN_MAX_INDICES) {
     int rc = scratch_on_current_device(fn, &row_map);
     if (rc) return rc;
     // every entry below num_tokens is rewritten, so nothing of an earlier call is seen
     rc = build_row_map(fn, row_map, num_tokens, indices, index_bytes, num_indices, stream);
     if (rc) return rc;
   }
-  const SelectArgs sel = {row_map, keys_out, values_out, out_key_stride, out_value_stride, num_indices,
-                          indices, index_bytes, num_src_rows};
+  const SelectArgs sel = {row_map ? kSelectByRowMap : kSelectByScan, row_map, keys_out, values_out, out_key_stride,
+                          out_value_stride, num_indices, indices, index_bytes, num_src_rows};
   return bulk_entry(fn, keys, values, key_stride, value_stride, key_cache_ptrs, value_cache_ptrs, k_scale_ptrs,
                     v_scale_ptrs, slot_mapping, num_tokens, num_layers, num_heads, head_size, block_size, block_stride,
                     num_blocks, src_dtype, kv_cache_dtype, sel, stream);

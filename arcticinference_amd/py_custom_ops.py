@@ -80,6 +80,7 @@ _SRC_DTYPES = {
     torch.bfloat16: _native.DTYPE_BF16,
 }
 _HALF_DTYPES = {torch.float16: _native.DTYPE_F16, torch.bfloat16: _native.DTYPE_BF16}
+_SELECT_SCAN_MAX_INDICES = 2048   # ARCTIC_SELECT_SCAN_MAX_INDICES of the C ABI
 
 _torch_lib: Optional[torch.library.Library] = None
 _registered = False
@@ -178,7 +179,7 @@ def _reshape_and_cache_flash_bulk_impl(
     v_scales: List[torch.Tensor],
     num_heads: int,
     head_size: int,
-    _select: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]] = None,
+    _select: Optional[Tuple[Optional[torch.Tensor], torch.Tensor, torch.Tensor, torch.Tensor]] = None,
 ) -> None:
     """Host side of the bulk KV write; follows the reference's launcher
     (csrc/custom_ops/reshape_and_cache_flash_bulk.cu:77-144) up to the point
@@ -254,7 +255,8 @@ def _reshape_and_cache_flash_bulk_impl(
         else:
             row_map, idx, k_out, v_out = _select
             rc = lib.arctic_reshape_and_cache_flash_bulk_select(
-                *common, row_map.data_ptr(), idx.data_ptr(), idx.element_size(), idx.numel(), keys.size(0),
+                *common, row_map.data_ptr() if row_map is not None else None, idx.data_ptr(), idx.element_size(),
+                idx.numel(), keys.size(0),
                 k_out.data_ptr(), v_out.data_ptr(), k_out.stride(0), v_out.stride(0), _stream_of(keys))
     _native.check(rc)
 
@@ -308,12 +310,15 @@ def _reshape_and_cache_flash_bulk_select_impl(
         if n_sel:
             _move_rows_impl("gather_rows", [keys[:, :width], values[:, :width]], idx, [k_out, v_out], False)
         return
-    # the inverse of logits_indices: which output row, if any, a token goes to
-    row_map = torch.empty(num_tokens, dtype=torch.int64, device=keys.device)
-    with _on_device_of(keys):
-        rc = _lib().arctic_build_row_map(row_map.data_ptr(), num_tokens, idx.data_ptr(), idx.element_size(), n_sel,
-                                         _stream_of(keys))
-    _native.check(rc)
+    row_map = None
+    if n_sel > _SELECT_SCAN_MAX_INDICES:
+        # a long list: the inverse of logits_indices (which output row, if any, a token goes to) is built first;
+        # up to that length every token's workgroup scans the list itself and nothing is allocated or launched here
+        row_map = torch.empty(num_tokens, dtype=torch.int64, device=keys.device)
+        with _on_device_of(keys):
+            rc = _lib().arctic_build_row_map(row_map.data_ptr(), num_tokens, idx.data_ptr(), idx.element_size(), n_sel,
+                                             _stream_of(keys))
+        _native.check(rc)
     _reshape_and_cache_flash_bulk_impl(keys, values, key_caches, value_caches, slot_mapping, kv_cache_dtype, k_scales,
                                        v_scales, num_heads, head_size, _select=(row_map, idx, k_out, v_out))
 

@@ -111,23 +111,30 @@ int arctic_reshape_and_cache_flash_bulk(
 int arctic_build_row_map(int64_t *row_map, int64_t num_tokens, const void *indices, int index_bytes,
                          int64_t num_indices, void *stream);
 
+/* Longest index list that arctic_reshape_and_cache_flash_bulk_select serves without a row map. */
+#define ARCTIC_SELECT_SCAN_MAX_INDICES 2048
+
 /*
  * The bulk KV-cache write with the row selection that follows it in the caller folded in.  Everything
- * arctic_reshape_and_cache_flash_bulk does, and in the same pass over the source: token t's rows are also
- * copied, unconverted, to row row_map[t] of keys_out / values_out, which is
+ * arctic_reshape_and_cache_flash_bulk does, and in the same pass over the source
+ *   keys_out[j] = keys[indices[j]],  values_out[j] = values[indices[j]]        for j < num_indices
+ * which is
  *   index_fn("k_states", k_states, logits_indices), index_fn("v_states", v_states, logits_indices)
  *        arctic_inference/vllm/swiftkv/llama_swiftkv.py:663-679
- * with row_map the inverse of logits_indices (row_map[logits_indices[j]] = j, -1 elsewhere), so k_states and
- * v_states are read once for both steps.  No single function of the reference corresponds to it.
+ * so k_states and v_states are read once for both steps.  No single function of the reference corresponds to it.
+ * The result is torch.index_select's for EVERY index in [0, num_src_rows), repeated ones included; a token is
+ * copied whether or not its slot is padding.  Output rows whose index lies outside [0, num_src_rows) are left as
+ * they were (index_select would raise).
  *
- *   row_map            device int64[num_tokens], as arctic_build_row_map leaves it for `indices`; negative or
- *                      >= num_indices: the token is not copied.  A token is copied whether or not its slot is padding.
- *   indices            device, num_indices entries of index_bytes (4 or 8) each, or NULL.  With the list given,
- *                      the result is torch.index_select for EVERY index in [0, num_src_rows): output rows that
- *                      the row map cannot serve (an index that is repeated, or one at or beyond num_tokens) are
- *                      copied from the source by extra workgroups of the same launch.  Output rows whose index
- *                      lies outside [0, num_src_rows) are left as they were (index_select would raise).
- *                      NULL: the caller vouches that the indices are distinct and below num_tokens.
+ *   indices            device, num_indices entries of index_bytes (4 or 8) each.
+ *   row_map            NULL, or device int64[num_tokens] as arctic_build_row_map leaves it for `indices`.
+ *                      NULL (num_indices <= ARCTIC_SELECT_SCAN_MAX_INDICES: one index per request of a serving
+ *                      batch): every token's workgroup scans the index list itself for the output rows that name
+ *                      its token; one launch, no workspace.  Given: a token's workgroup looks its output row up
+ *                      in the map, whatever the list's length; rows that the map cannot serve (an index that is
+ *                      repeated, a source row at or beyond num_tokens) are copied from the source by a few index
+ *                      workgroups of the same launch.  With a row map `indices` may be NULL: the caller then
+ *                      vouches that the indices are distinct and below num_tokens.
  *   num_src_rows       rows of keys / values (>= num_tokens)
  *   keys_out, values_out   device; num_indices rows of num_layers*n elements of src_dtype, out_*_stride ELEMENTS apart
  *   other arguments as arctic_reshape_and_cache_flash_bulk
@@ -147,19 +154,22 @@ int arctic_reshape_and_cache_flash_bulk_select(
 
 /*
  * arctic_reshape_and_cache_flash_bulk_select for callers that cannot allocate device memory (code under HIP
- * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
- * The same result as arctic_build_row_map followed by arctic_reshape_and_cache_flash_bulk_select, but the row
- * map is kept in a device array inside the library (8 bytes x ARCTIC_SELECT_STATIC_MAX_TOKENS = 2 MiB on each
- * GPU the library runs on, held until the process ends) instead of a workspace of the caller's.  The call
- * allocates and frees nothing; it enqueues two kernels on `stream`.
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc) and whose index lists may be longer than
+ * ARCTIC_SELECT_SCAN_MAX_INDICES.  It has no counterpart in the reference.  The same result as
+ * arctic_reshape_and_cache_flash_bulk_select; where that needs a row map (lists beyond
+ * ARCTIC_SELECT_SCAN_MAX_INDICES) the map is built by this call and kept in a device array inside the library
+ * (8 bytes x ARCTIC_SELECT_STATIC_MAX_TOKENS = 2 MiB on each GPU the library runs on, held until the process ends)
+ * instead of a workspace of the caller's.  The call allocates and frees nothing; it enqueues one or two kernels on
+ * `stream`.
  *
  *   num_tokens   at most ARCTIC_SELECT_STATIC_MAX_TOKENS, else ARCTIC_ERR_INVALID_ARGUMENT
  *   indices      device, num_indices entries of index_bytes (4 or 8) each; required when num_indices > 0
  *   other arguments as arctic_reshape_and_cache_flash_bulk_select
  *
- * All calls on one GPU share that GPU's array: calls that may run at the same time on one GPU (different
- * streams without an ordering between them) race on it and must use the workspace form instead.  The first call
- * on a device looks the array's address up (hipGetSymbolAddress); make that call outside graph capture.
+ * All calls on one GPU share that GPU's array: calls with long index lists that may run at the same time on one
+ * GPU (different streams without an ordering between them) race on it and must use the workspace form instead.
+ * The first such call on a device looks the array's address up (hipGetSymbolAddress); make that call outside graph
+ * capture.
  */
 int arctic_reshape_and_cache_flash_bulk_select_static(
     const void *keys, const void *values, int64_t key_stride, int64_t value_stride,

@@ -85,7 +85,17 @@ def test_argument_errors_return_codes_without_launching(lib):
     # the entry points of the "next" rows validate the same way
     bulk = (None, None, 0, 0, None, None, None, None, None, 4, 2, 2, 64, 16, 0, 0, _native.DTYPE_BF16, _native.KV_AUTO)
     rc = lib.arctic_reshape_and_cache_flash_bulk_select(*bulk, None, None, 8, 4, 4, None, None, 0, 0, None)
-    assert rc == 1 and b"null row map" in lib.arctic_last_error()
+    assert rc == 1 and b"null tensor pointer" in lib.arctic_last_error()
+    fake = ctypes.c_void_p(256)        # never dereferenced: the calls below are refused on their other arguments
+    held = (fake, fake, 0, 0, fake, fake, None, None, fake) + bulk[9:]
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select(*held, None, fake, 8, 4, 4, None, None, 0, 0, None)
+    assert rc == 1 and b"null keys_out or values_out" in lib.arctic_last_error()
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select(*held, None, None, 8, 4, 4, fake, fake, 0, 0, None)
+    assert rc == 1 and b"index list is missing" in lib.arctic_last_error()
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select(*held, None, fake, 8, 5000, 5000, fake, fake, 0, 0, None)
+    assert rc == 1 and b"longer than 2048 entries" in lib.arctic_last_error()
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select(*held, None, fake, 2, 4, 4, fake, fake, 0, 0, None)
+    assert rc == 2 and b"int32 or int64" in lib.arctic_last_error()
     assert lib.arctic_reshape_and_cache_flash_bulk_select(*bulk[:10], 0, *bulk[11:], None, None, 8, 4, 4, None, None, 0, 0,
                                                           None) == 0
     static = (*bulk[:9], 1 << 20, *bulk[10:], None, 8, 4, 1 << 20, None, None, 0, 0, None)

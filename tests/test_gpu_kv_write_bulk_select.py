@@ -100,7 +100,10 @@ def test_random_configurations(ops):
         T = cfg["T"]
         g = torch.Generator().manual_seed(it)
         n_sel = rnd.choice([0, 1, max(1, T // 3), T])
-        idx = torch.randperm(T, generator=g)[:n_sel]
+        if rnd.random() < 0.3:
+            idx = torch.randint(0, T, (n_sel,), generator=g)       # with repeats
+        else:
+            idx = torch.randperm(T, generator=g)[:n_sel]
         if rnd.random() < 0.6:
             idx = torch.sort(idx).values
         try:
@@ -122,6 +125,51 @@ def test_repeated_indices_and_rows_beyond_the_slot_mapping_match_index_select(op
     # more layers than one launch holds, every index repeated
     case = make_bulk_case(T=9, L=70, H=2, D=64, bs=16, NB=4, kv_cache_dtype=kv, seed=50)
     run_select(ops, case, torch.tensor([8, 8, 0, 0, 3, 3, 3]), 7)
+
+
+@pytest.mark.parametrize("kv", ["auto", "fp8"])
+def test_index_lists_too_long_to_scan_go_through_the_row_map(ops, kv):
+    # more than 2048 indices: the operator builds the inverse of the list first; repeats and rows beyond the slot
+    # mapping are then served by the index workgroups
+    case = make_bulk_case(T=3300, L=3, H=8, D=128, bs=16, NB=256, kv_cache_dtype=kv, seed=52, pad_fraction=0.1)
+    case["slot_mapping"] = case["slot_mapping"][:3200].contiguous()
+    g = torch.Generator().manual_seed(6)
+    idx = torch.cat([torch.randperm(3300, generator=g)[:2600], torch.randint(0, 3300, (150,), generator=g)])
+    assert idx.numel() > 2048
+    run_select(ops, case, idx, idx.numel() + 3)
+    # the element-wise kernel with a long list
+    case = make_bulk_case(T=2200, L=2, H=1, D=20, bs=4, NB=600, kv_cache_dtype=kv, seed=53, key_pad=3)
+    idx = torch.cat([torch.arange(2200), torch.tensor([7, 7, 2199])])
+    run_select(ops, case, idx, idx.numel(), out_pad=1)
+
+
+def test_scan_and_row_map_agree_through_the_c_abi(ops):
+    # the same short list served both ways: without a row map (the token workgroups scan the list) and with one
+    lib = _native.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    case = make_bulk_case(T=200, L=5, H=8, D=128, bs=16, NB=16, kv_cache_dtype="fp8", seed=54, pad_fraction=0.2)
+    idx = torch.tensor([5, 199, 5, 0, 77, 5, 198, 0], device=DEV)
+    tab = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+    outs = []
+    for with_map in (False, True):
+        d = bulk_case_to(case, DEV)
+        k_out = torch.zeros(8, 5 * 1024, dtype=torch.bfloat16, device=DEV)
+        v_out = torch.zeros_like(k_out)
+        row_map = torch.empty(200, dtype=torch.int64, device=DEV)
+        assert lib.arctic_build_row_map(row_map.data_ptr(), 200, idx.data_ptr(), 8, 8, stream) == 0
+        rc = lib.arctic_reshape_and_cache_flash_bulk_select(
+            d["keys"].data_ptr(), d["values"].data_ptr(), d["keys"].stride(0), d["values"].stride(0), tab(d["key_caches"]),
+            tab(d["value_caches"]), tab(d["k_scales"]), tab(d["v_scales"]), d["slot_mapping"].data_ptr(), 200, 5, 8, 128, 16,
+            d["key_caches"][0].stride(0), 16, _native.DTYPE_BF16, _native.KV_FP8_E4M3,
+            row_map.data_ptr() if with_map else None, idx.data_ptr(), 8, 8, 200, k_out.data_ptr(), v_out.data_ptr(),
+            k_out.stride(0), v_out.stride(0), stream)
+        assert rc == 0, lib.arctic_last_error()
+        torch.cuda.synchronize()
+        outs.append((d, k_out, v_out))
+    oracle.reshape_and_cache_flash_bulk(*bulk_args(case))
+    for d, k_out, v_out in outs:
+        assert_bulk_equal(d["bufs"], case["bufs"])
+        assert torch.equal(k_out.cpu(), case["keys"][idx.cpu()]) and torch.equal(v_out.cpu(), case["values"][idx.cpu()])
 
 
 def test_indices_outside_the_source_leave_their_rows_untouched(ops):

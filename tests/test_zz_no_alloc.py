@@ -84,20 +84,25 @@ def check_pair(lib, case, idx):
 def test_two_calls_in_a_row_the_second_smaller(ops):
     lib = _native.load()
     g = torch.Generator().manual_seed(5)
-    # first call: 3000 tokens, rows 1500.. selected, some twice
-    big = make_bulk_case(T=3000, L=6, H=8, D=128, bs=16, NB=256, kv_cache_dtype="fp8", seed=60, std=1.5, pad_fraction=0.1)
-    idx_big = torch.cat([torch.randperm(3000, generator=g)[:200], torch.tensor([2999, 2999, 1500])])
+    # Index lists of more than 2048 entries are what makes the entry point use its device array (shorter lists are
+    # scanned by the token workgroups and need no row map).  First call: 3000 tokens, 2600 of them selected, some twice.
+    big = make_bulk_case(T=3000, L=4, H=8, D=128, bs=16, NB=256, kv_cache_dtype="fp8", seed=60, std=1.5, pad_fraction=0.1)
+    idx_big = torch.cat([torch.randperm(3000, generator=g)[:2600], torch.tensor([2999, 2999, 1500])])
     check_pair(lib, big, idx_big)
-    # second call, smaller in every respect; its tokens 0..89 had other entries in the first call's row map
-    small = make_bulk_case(T=90, L=3, H=8, D=128, bs=16, NB=8, kv_cache_dtype="fp8", seed=61, std=1.5, pad_fraction=0.2)
-    idx_small = torch.tensor([7, 3, 88, 3, 0], dtype=torch.int32)
+    # second call, smaller in every respect and again through the array: tokens 0..2399 had other entries in the
+    # first call's row map, entries 2400..2999 of the array still hold the first call's
+    small = make_bulk_case(T=2400, L=3, H=8, D=128, bs=16, NB=160, kv_cache_dtype="fp8", seed=61, std=1.5, pad_fraction=0.2)
+    idx_small = torch.cat([torch.randperm(2400, generator=g)[:2100], torch.tensor([7, 3, 2399, 3, 0])]).to(torch.int32)
+    assert idx_small.numel() > 2048
     check_pair(lib, small, idx_small)
-    # third: a bf16 cache, the element-wise kernel (60-element rows), and keys with more rows than slots
-    odd = make_bulk_case(T=50, L=4, H=3, D=20, bs=4, NB=16, kv_cache_dtype="auto", seed=62, key_pad=3)
-    odd["slot_mapping"] = odd["slot_mapping"][:40].contiguous()
-    check_pair(lib, odd, torch.tensor([49, 0, 41, 12, 12]))
-    # nothing selected: the plain write
-    check_pair(lib, small, torch.empty(0, dtype=torch.int64))
+    # third: a bf16 cache, the element-wise kernel (60-element rows), keys with more rows than slots, a long list
+    odd = make_bulk_case(T=2300, L=2, H=3, D=20, bs=4, NB=600, kv_cache_dtype="auto", seed=62, key_pad=3)
+    odd["slot_mapping"] = odd["slot_mapping"][:2250].contiguous()
+    check_pair(lib, odd, torch.cat([torch.arange(2300), torch.tensor([49, 0, 2260, 12, 12])]))
+    # short lists (no row map in either form) and an empty one (the plain write)
+    tiny = make_bulk_case(T=90, L=3, H=8, D=128, bs=16, NB=8, kv_cache_dtype="fp8", seed=64, std=1.5, pad_fraction=0.2)
+    check_pair(lib, tiny, torch.tensor([7, 3, 88, 3, 0], dtype=torch.int32))
+    check_pair(lib, tiny, torch.empty(0, dtype=torch.int64))
 
 
 def test_size_limit_and_argument_errors(ops):

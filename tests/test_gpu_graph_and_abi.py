@@ -213,6 +213,17 @@ def test_operators_trace_under_torch_compile(ops, backend):
     for a, b in zip(got, want):
         assert torch.equal(a, b)
 
+    def first_step(s4, z4, x, w):
+        # no previous cell, in all three forms (the optional argument traces as None)
+        a = ops.sum_lstm(s4, z4, None, w, w, w, w, 0.5, 1e-6, 1e-6, False)
+        b = ops.sum_lstm_shared_z(s4, x, None, w, w, w, w, 0.5, 1e-6, 1e-6, False)
+        return a[0] + b[0], a[1], b[1]
+
+    want = first_step(s4, z4, x, w)
+    got = torch.compile(first_step, backend=backend, fullgraph=True)(s4, z4, x, w)
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+
     layers = 3
     k, v = rn(16, layers * 128), rn(16, layers * 128)
     slots = torch.randperm(64, generator=g)[:16].to(DEV)

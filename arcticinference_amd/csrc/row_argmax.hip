@@ -13,6 +13,7 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <cstdlib>
 
 #include "common.hpp"
 
@@ -71,7 +72,8 @@ struct HalfElem {
 
 // kVec: rows are 16-byte aligned, so the body of a row is read in 16-byte chunks; the elements behind
 // the last whole chunk (and everything when !kVec) are read one by one.
-template <typename Elem, bool kVec>
+// kUnroll chunks per lane form a batch; kPipelined: the next batch is requested before the current one is looked at.
+template <typename Elem, bool kVec, int kUnroll = 4, bool kPipelined = false>
 __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ out, const char *__restrict__ in,
                                                           int64_t row_stride_bytes, int cols, int64_t max_index) {
   __shared__ float wave_value[16];
@@ -95,14 +97,15 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
   };
   int done = 0;
   if (kVec) {
-    constexpr int kUnroll = 4;
-    for (int c0 = threadIdx.x; c0 < chunks; c0 += kUnroll * blockDim.x) {
-      uint4 raw[kUnroll];
+    const int stride = kUnroll * blockDim.x;
+    auto request = [&](int c0, uint4 (&raw)[kUnroll]) {
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         const int c = c0 + u * blockDim.x;
         if (c < chunks) raw[u] = load16_stream(row + (int64_t)c * 16);
       }
+    };
+    auto look_at = [&](int c0, const uint4 (&raw)[kUnroll]) {
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         const int c = c0 + u * blockDim.x;
@@ -121,6 +124,24 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
               if (f[j] != f[j]) nan_at = min(nan_at, c * P + j);
           }
         }
+      }
+    };
+    if constexpr (kPipelined) {
+      uint4 cur[kUnroll], nxt[kUnroll];
+      int c0 = threadIdx.x;
+      request(c0, cur);
+      while (c0 < chunks) {
+        request(c0 + stride, nxt);
+        look_at(c0, cur);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) cur[u] = nxt[u];
+        c0 += stride;
+      }
+    } else {
+      for (int c0 = threadIdx.x; c0 < chunks; c0 += stride) {
+        uint4 raw[kUnroll];
+        request(c0, raw);
+        look_at(c0, raw);
       }
     }
     done = chunks * P;
@@ -172,11 +193,33 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
   int threads = (int)std::min<int64_t>(1024, std::max<int64_t>(64, ((cols / per_chunk / 4 + 63) / 64) * 64));
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)rows), block((unsigned)threads);
+#ifdef ARCTIC_TUNING
+  // measurement build: ARCTIC_ARGMAX_VARIANT = 1 pipelined batches of 4, 2 batches of 8, 3 pipelined batches of 8,
+  // 4 pipelined batches of 2; + 8: half the lanes
+  int variant = 0;
+  if (const char *e = getenv("ARCTIC_ARGMAX_VARIANT")) variant = atoi(e);
+  if (variant & 8) threads = std::max(64, threads / 2);
+  variant &= 7;
+#define ARCTIC_ARGMAX_VEC(ELEM)                                                                                          \
+  do {                                                                                                                   \
+    const dim3 b((unsigned)threads);                                                                                     \
+    switch (variant) {                                                                                                   \
+      case 1: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
+      case 2: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 8, false>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
+      case 3: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 8, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
+      case 4: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 2, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
+      default: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
+    }                                                                                                                    \
+  } while (0)
+#else
+#define ARCTIC_ARGMAX_VEC(ELEM)                                                                             \
+  hipLaunchKernelGGL((row_argmax_kernel<ELEM, true>), grid, block, 0, s, out, (const char *)logits, stride_bytes, cols, \
+                     max_index)
+#endif
 #define ARCTIC_ARGMAX_LAUNCH(ELEM)                                                                          \
   do {                                                                                                      \
     if (vec)                                                                                                \
-      hipLaunchKernelGGL((row_argmax_kernel<ELEM, true>), grid, block, 0, s, out, (const char *)logits,     \
-                         stride_bytes, cols, max_index);                                                    \
+      ARCTIC_ARGMAX_VEC(ELEM);                                                                              \
     else                                                                                                    \
       hipLaunchKernelGGL((row_argmax_kernel<ELEM, false>), grid, block, 0, s, out, (const char *)logits,    \
                          stride_bytes, cols, max_index);                                                    \
@@ -185,5 +228,6 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
   else if (dtype == ARCTIC_DTYPE_BF16) ARCTIC_ARGMAX_LAUNCH(HalfElem<BF16>);
   else ARCTIC_ARGMAX_LAUNCH(HalfElem<F16>);
 #undef ARCTIC_ARGMAX_LAUNCH
+#undef ARCTIC_ARGMAX_VEC
   return check_launch(fn);
 }

@@ -1044,6 +1044,8 @@ def load_tuning_library():
     lib.arctic_reshape_and_cache_flash_bulk.argtypes = [vp, vp, i64, i64, vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i64,
                                                         i64, i32, i32, vp]
     lib.arctic_reshape_and_cache_flash_bulk.restype = i32
+    lib.arctic_argmax_clamp.argtypes = [vp, vp, i64, i32, i64, i64, i32, vp]
+    lib.arctic_argmax_clamp.restype = i32
     return lib
 
 
@@ -1085,6 +1087,52 @@ def bench_bulk_variants(dev, steps):
         os.environ.pop(k, None)
     return {name: {"kernel_us_rounds": v, "GBps": round(w.bytes / statistics.mean(v) / 1e3),
                    "hbm_frac": round(w.bytes / statistics.mean(v) / 1e3 / HBM_PEAK_GBS, 4)} for name, v in out.items()}
+
+
+def bench_argmax_variants(dev, steps):
+    """A/B of the row-argmax kernel's loop shapes through the tuning build: 512 rows x 128256 bf16 logits (131 MB),
+    three rotating sets in one graph per variant, three rounds over all variants; results compared with torch's."""
+    tuning = load_tuning_library()
+    if tuning is None:
+        return "libarctic_tuning_mi355x.so is not built"
+    T, V, sets = 512, 128256, 3
+    g = torch.Generator(device=dev).manual_seed(8)
+    logits = [torch.randn(T, V, generator=g, device=dev).to(torch.bfloat16) for _ in range(sets)]
+    outs = [torch.empty(T, dtype=torch.int64, device=dev) for _ in range(sets)]
+    want = [torch.argmax(x, dim=-1).clamp_(0, V - 1) for x in logits]
+    nbytes = T * V * 2 + T * 8
+    cases = [(0, "batches of 4 chunks per lane, 1024 lanes (the previous kernel)"), (1, "the same, next batch requested first"),
+             (2, "batches of 8"), (3, "batches of 8, next batch requested first"),
+             (4, "batches of 2, next batch requested first"), (9, "512 lanes, batches of 4, next batch first"),
+             (11, "512 lanes, batches of 8, next batch first")]
+
+    def run():
+        stream = torch.cuda.current_stream().cuda_stream
+        for i in range(sets):
+            assert tuning.arctic_argmax_clamp(outs[i].data_ptr(), logits[i].data_ptr(), T, V, V, V - 1, 2, stream) == 0
+
+    graphs, out = {}, {}
+    for code, what in cases:
+        os.environ["ARCTIC_ARGMAX_VARIANT"] = str(code)
+        run()
+        torch.cuda.synchronize()
+        ok = all(torch.equal(a, b) for a, b in zip(outs, want))
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            run()
+        graphs[code] = graph
+        out[str(code)] = {"variant": what, "equals_torch": ok, "us": []}
+    os.environ.pop("ARCTIC_ARGMAX_VARIANT", None)
+    for _ in range(3):
+        for code, graph in graphs.items():
+            for _ in range(2):
+                graph.replay()
+            torch.cuda.synchronize()
+            out[str(code)]["us"].append(round(statistics.mean(event_times_us(graph.replay, max(10, steps // 2))) / sets, 2))
+    for v in out.values():
+        m = statistics.mean(v["us"])
+        v.update({"us_per_call_graph_rounds": v.pop("us"), "GBps": round(nbytes / m / 1e3), "hbm_frac": round(nbytes / m / 1e3 / HBM_PEAK_GBS, 4)})
+    return out
 
 
 # ARCTIC_LSTM_VARIANT values of the tuning build (sum_lstm.hip): bits 0-2 = arithmetic / ordering variants,
@@ -1221,6 +1269,8 @@ def main():
     ap.add_argument("--lstm-variants", action="store_true",
                     help="instead of the benchmark, time the sum_lstm kernel variants of the tuning build against "
                          "each other and against the traffic-only kernel; prints one JSON object")
+    ap.add_argument("--argmax-variants", action="store_true",
+                    help="instead of the benchmark, time loop shapes of the row-argmax kernel through the tuning build")
     ap.add_argument("--bulk-variants", action="store_true",
                     help="instead of the benchmark, time launch variants of the bulk write in the compact placement "
                          "through the tuning build; prints one JSON object")
@@ -1246,6 +1296,9 @@ def main():
         return
     if args.lstm_variants:
         print(json.dumps({"sum_lstm_variants": bench_lstm_variants(dev, args.steps)}), flush=True)
+        return
+    if args.argmax_variants:
+        print(json.dumps({"row_argmax_variants": bench_argmax_variants(dev, args.steps)}), flush=True)
         return
     if args.bulk_variants:
         print(json.dumps({"bulk_write_variants_compact_pool": bench_bulk_variants(dev, args.steps)}), flush=True)

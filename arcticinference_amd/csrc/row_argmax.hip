@@ -41,18 +41,38 @@ __device__ __forceinline__ void offer(Winner &w, float v, int i) {
   }
 }
 
-__device__ __forceinline__ Winner wave_winner(Winner w) {
-#pragma unroll
-  for (int step = 32; step >= 1; step >>= 1) {
-    const float ov = __shfl_xor(w.value, step, 64);
-    const int oi = __shfl_xor(w.index, step, 64);
-    offer(w, ov, oi);
-  }
-  return w;
+// The wave's winner in every lane.  Inside each row of 16 lanes the candidates meet through DPP lane exchanges
+// (vector-ALU moves, no LDS round trip): partners at distance 1 and 2 inside a quad, then the mirrored half and the
+// mirrored row, after which all 16 lanes of a row agree; the four row winners are read with v_readlane.
+template <int kCtrl>
+__device__ __forceinline__ void meet(Winner &w) {
+  const float ov = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(w.value), kCtrl, 0xf, 0xf, true));
+  const int oi = __builtin_amdgcn_update_dpp(0, w.index, kCtrl, 0xf, 0xf, true);
+  offer(w, ov, oi);
 }
+
+__device__ __forceinline__ Winner wave_winner(Winner w) {
+  meet<0xB1>(w);   // quad_perm [1,0,3,2]
+  meet<0x4E>(w);   // quad_perm [2,3,0,1]
+  meet<0x141>(w);  // row_half_mirror
+  meet<0x140>(w);  // row_mirror
+  const int vb = __float_as_int(w.value);
+  Winner r = {__int_as_float(__builtin_amdgcn_readlane(vb, 0)), __builtin_amdgcn_readlane(w.index, 0)};
+#pragma unroll
+  for (int lane = 16; lane < 64; lane += 16)
+    offer(r, __int_as_float(__builtin_amdgcn_readlane(vb, lane)), __builtin_amdgcn_readlane(w.index, lane));
+  return r;
+}
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 
 struct F32Elem {
   static constexpr int kPerChunk = 4;
+  // NaN exactly when the chunk holds a NaN or infinities of both signs
+  __device__ static __forceinline__ float probe(const uint4 &v) {
+    return (__uint_as_float(v.x) + __uint_as_float(v.y)) + (__uint_as_float(v.z) + __uint_as_float(v.w));
+  }
   __device__ static __forceinline__ void unpack(const uint4 &v, float (&f)[8]) {
     f[0] = __uint_as_float(v.x);
     f[1] = __uint_as_float(v.y);
@@ -64,6 +84,23 @@ struct F32Elem {
 template <typename T>
 struct HalfElem {
   static constexpr int kPerChunk = 8;
+  // the sum of the chunk's eight values, two per instruction straight from the packed words (v_dot2c_f32_bf16 /
+  // v_dot2c_f32_f16 with a vector of ones): NaN exactly when the chunk holds a NaN or infinities of both signs
+  __device__ static __forceinline__ float probe(const uint4 &v) {
+    float acc = 0.f;
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if constexpr (T::kCode == ARCTIC_DTYPE_BF16) {
+        const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
+        acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[k]), ones, acc, false);
+      } else {
+        const f16x2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, w[k]), ones, acc, false);
+      }
+    }
+    return acc;
+  }
   __device__ static __forceinline__ void unpack(const uint4 &v, float (&f)[8]) { unpack8<T>(v, f); }
   __device__ static __forceinline__ float one(const void *p, int64_t i) {
     return T::lo((uint32_t)((const uint16_t *)p)[i]);
@@ -72,22 +109,22 @@ struct HalfElem {
 
 // kVec: rows are 16-byte aligned, so the body of a row is read in 16-byte chunks; the elements behind
 // the last whole chunk (and everything when !kVec) are read one by one.
-// kUnroll chunks per lane form a batch; kPipelined: the next batch is requested before the current one is looked at.
-template <typename Elem, bool kVec, int kUnroll = 4, bool kPipelined = false>
+// kUnroll chunks per lane form a batch; kPipelined: the next batch is requested before the current one is looked at;
+// kStaggered: the odd waves take half a batch on its own first, so that neighbouring waves are half a batch apart.
+template <typename Elem, bool kVec, int kUnroll = 4, bool kPipelined = false, bool kStaggered = false>
 __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ out, const char *__restrict__ in,
                                                           int64_t row_stride_bytes, int cols, int64_t max_index) {
   __shared__ float wave_value[16];
   __shared__ int wave_index[16];
   const char *row = in + (int64_t)blockIdx.x * row_stride_bytes;
-  // Per lane: the largest number seen and where (a strict ">" keeps the earlier of equal values, the
-  // lane's indices only grow), and apart from that the first NaN.  A chunk's sum is NaN only if the
-  // chunk holds a NaN (or infinities of both signs), so the per-element NaN test runs almost never.
+  // Per lane: the largest number seen, the chunk it was first seen in and that chunk's words (a strict ">" keeps the
+  // earlier of equal values, the lane's chunk indices only grow); which of the chunk's elements it was is worked out
+  // once, after the loop.  Apart from that the first NaN: a chunk's sum is NaN only if the chunk holds a NaN (or
+  // infinities of both signs), so the per-element NaN test runs almost never.
   constexpr int P = Elem::kPerChunk;
   const int chunks = kVec ? cols / P : 0;
-  // the lane's first element stands in for "nothing below -inf here": a row of -inf must answer 0
   float best = -__builtin_inff();
-  int best_at = (int)threadIdx.x < chunks ? (int)threadIdx.x * P
-                                           : (chunks * P + (int)threadIdx.x < cols ? chunks * P + (int)threadIdx.x : -1);
+  int best_at = -1;
   int nan_at = 0x7fffffff;
   auto number = [&](float v, int i) {
     if (v > best) {
@@ -97,6 +134,8 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
   };
   int done = 0;
   if (kVec) {
+    int best_chunk = -1;
+    uint4 best_words = make_uint4(0, 0, 0, 0);
     const int stride = kUnroll * blockDim.x;
     auto request = [&](int c0, uint4 (&raw)[kUnroll]) {
 #pragma unroll
@@ -105,25 +144,29 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
         if (c < chunks) raw[u] = load16_stream(row + (int64_t)c * 16);
       }
     };
+    auto look_at_chunk = [&](int c, const uint4 &words) {
+      float f[8];
+      Elem::unpack(words, f);
+      float top = best;   // fmaxf drops NaNs: they are found through the sum below
+#pragma unroll
+      for (int j = 0; j < P; j += 2) top = fmaxf(fmaxf(top, f[j]), f[j + 1]);
+      if (top > best) {
+        best_chunk = c;
+        best_words = words;
+      }
+      best = top;
+      const float sum = Elem::probe(words);
+      if (sum != sum) {
+#pragma unroll
+        for (int j = 0; j < P; ++j)
+          if (f[j] != f[j]) nan_at = min(nan_at, c * P + j);
+      }
+    };
     auto look_at = [&](int c0, const uint4 (&raw)[kUnroll]) {
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         const int c = c0 + u * blockDim.x;
-        if (c < chunks) {
-          float f[8];
-          Elem::unpack(raw[u], f);
-          float sum = 0.f;
-#pragma unroll
-          for (int j = 0; j < P; ++j) {
-            number(f[j], c * P + j);
-            sum += f[j];
-          }
-          if (sum != sum) {
-#pragma unroll
-            for (int j = 0; j < P; ++j)
-              if (f[j] != f[j]) nan_at = min(nan_at, c * P + j);
-          }
-        }
+        if (c < chunks) look_at_chunk(c, raw[u]);
       }
     };
     if constexpr (kPipelined) {
@@ -138,14 +181,46 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
         c0 += stride;
       }
     } else {
-      for (int c0 = threadIdx.x; c0 < chunks; c0 += stride) {
+      int c0 = threadIdx.x;
+      if constexpr (kStaggered) {
+        if ((threadIdx.x >> 6) & 1) {
+          constexpr int kLead = kUnroll / 2;
+          uint4 lead[kLead];
+#pragma unroll
+          for (int u = 0; u < kLead; ++u) {
+            const int c = c0 + u * (int)blockDim.x;
+            if (c < chunks) lead[u] = load16_stream(row + (int64_t)c * 16);
+          }
+#pragma unroll
+          for (int u = 0; u < kLead; ++u) {
+            const int c = c0 + u * (int)blockDim.x;
+            if (c < chunks) look_at_chunk(c, lead[u]);
+          }
+          c0 += kLead * (int)blockDim.x;
+        }
+      }
+      for (; c0 < chunks; c0 += stride) {
         uint4 raw[kUnroll];
         request(c0, raw);
         look_at(c0, raw);
       }
     }
     done = chunks * P;
+    if (best_chunk >= 0) {
+      // the first element of that chunk that equals the lane's maximum
+      float f[8];
+      Elem::unpack(best_words, f);
+      int j = P - 1;
+#pragma unroll
+      for (int k = P - 2; k >= 0; --k)
+        if (f[k] == best) j = k;
+      best_at = best_chunk * P + j;
+    } else if ((int)threadIdx.x < chunks) {
+      best_at = (int)threadIdx.x * P;   // nothing above -inf here: the lane's first element stands for its chunks
+    }
   }
+  // (a lane without chunks takes its first tail element, if it has one, the same way: a row of -inf must answer 0)
+  if (best_at < 0 && done + (int)threadIdx.x < cols) best_at = done + (int)threadIdx.x;
   for (int i = done + threadIdx.x; i < cols; i += blockDim.x) {
     const float v = Elem::one(row, i);
     number(v, i);
@@ -195,7 +270,7 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
   const dim3 grid((unsigned)rows), block((unsigned)threads);
 #ifdef ARCTIC_TUNING
   // measurement build: ARCTIC_ARGMAX_VARIANT = 1 pipelined batches of 4, 2 batches of 8, 3 pipelined batches of 8,
-  // 4 pipelined batches of 2; + 8: half the lanes
+  // 4 pipelined batches of 2, 5 batches of 2, 6 batches of 4 with the odd waves half a batch ahead; + 8: half the lanes
   int variant = 0;
   if (const char *e = getenv("ARCTIC_ARGMAX_VARIANT")) variant = atoi(e);
   if (variant & 8) threads = std::max(64, threads / 2);
@@ -208,6 +283,8 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
       case 2: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 8, false>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
       case 3: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 8, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
       case 4: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 2, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
+      case 5: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 2, false>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
+      case 6: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
       default: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
     }                                                                                                                    \
   } while (0)

@@ -299,6 +299,7 @@ def load_floor_kernels():
     lib.floor_stream.argtypes = [vp, i32, vp, i32, i64, i32, vp, vp]
     lib.floor_valu_rate.argtypes = [i32, i32, i32, vp, vp]
     lib.floor_node.argtypes = [vp, vp, i32, i32, i32, vp]
+    lib.floor_row_read.argtypes = [vp, i64, i64, i32, vp, vp]
     return lib
 
 
@@ -603,8 +604,15 @@ def bench_argmax(ops, dev, steps):
     logits = [torch.randn(T, V, generator=g, device=dev).to(torch.bfloat16) for _ in range(sets)]
     nbytes = T * V * 2 + T * 8
     out = {"bytes_per_call": nbytes}
-    for name, fn in (("speculator_argmax", lambda i: ops.speculator_argmax(logits[i % sets], V)),
-                     ("torch_argmax_clamp", lambda i: torch.argmax(logits[i % sets], dim=-1).clamp_(0, V - 1))):
+    floor = load_floor_kernels()
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    cases = [("speculator_argmax", lambda i: ops.speculator_argmax(logits[i % sets], V)),
+             ("torch_argmax_clamp", lambda i: torch.argmax(logits[i % sets], dim=-1).clamp_(0, V - 1))]
+    if floor is not None:
+        # the kernel's loads with nothing computed: what reading the rows costs in this launch shape
+        cases.append(("row_read_only_floor", lambda i: floor.floor_row_read(
+            logits[i % sets].data_ptr(), T, V * 2, 1024, sink.data_ptr(), torch.cuda.current_stream().cuda_stream)))
+    for name, fn in cases:
         for i in range(3):
             fn(i)
         graph = torch.cuda.CUDAGraph()
@@ -1101,9 +1109,11 @@ def bench_argmax_variants(dev, steps):
     outs = [torch.empty(T, dtype=torch.int64, device=dev) for _ in range(sets)]
     want = [torch.argmax(x, dim=-1).clamp_(0, V - 1) for x in logits]
     nbytes = T * V * 2 + T * 8
-    cases = [(0, "batches of 4 chunks per lane, 1024 lanes (the previous kernel)"), (1, "the same, next batch requested first"),
+    cases = [(0, "batches of 4 chunks per lane, 1024 lanes (as shipped)"), (1, "the same, next batch requested first"),
              (2, "batches of 8"), (3, "batches of 8, next batch requested first"),
-             (4, "batches of 2, next batch requested first"), (9, "512 lanes, batches of 4, next batch first"),
+             (4, "batches of 2, next batch requested first"), (5, "batches of 2"),
+             (6, "batches of 4, odd waves half a batch ahead of the even ones"),
+             (9, "512 lanes, batches of 4, next batch first"),
              (11, "512 lanes, batches of 8, next batch first")]
 
     def run():
@@ -1246,6 +1256,7 @@ ONLY = {
     "speculator": lambda ops, dev, a: bench_speculator(ops, dev, a.steps, a.warmup),
     "sum_lstm_rows_sweep": lambda ops, dev, a: bench_lstm_rows(ops, dev, a.steps),
     "bulk_auto_bf16_cache": lambda ops, dev, a: bench_bulk_auto(ops, dev, a.steps),
+    "speculator_argmax_512x128256": lambda ops, dev, a: bench_argmax(ops, dev, a.steps),
     "bulk_write_and_select_decode_70b": lambda ops, dev, a: bench_bulk_select(ops, dev, a.steps),
     "bulk_fp8_70b_tp_sharded_heads_compact_pool": lambda ops, dev, a: bench_bulk_tp_heads(ops, dev, a.steps),
 }

@@ -3,6 +3,7 @@
 //
 //   floor_lstm_traffic   the loads and stores of sum_lstm (nine 16-byte loads per lane from the rows of
 //                        states, z4 and prev_cell, two 16-byte stores), one workgroup per row, no arithmetic
+//   floor_row_read       the loads of the row-argmax kernel (one workgroup per row), nothing computed
 //   floor_node           an empty kernel, or one that makes a single memory round trip: the fixed cost of a node
 //   floor_valu_rate      chains of one vector-ALU operation, for its issue rate per SIMD
 //   floor_stream         load-only, store-only or a 2:1 load:store stream in 64 KiB pieces, the pieces dealt
@@ -135,6 +136,31 @@ extern "C" int floor_node(const void *in, void *out, int blocks, int threads, in
   if (blocks <= 0 || threads < 64 || threads > 1024) return 1;
   hipLaunchKernelGGL(node_floor_kernel, dim3((unsigned)blocks), dim3((unsigned)threads), 0, (hipStream_t)stream,
                      (const u32x4 *)in, (u32x4 *)out, touch);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+// The loads of the row-argmax kernel and nothing else: one workgroup per row, 16-byte streaming loads in batches of
+// four per lane, the words xor-ed together.
+__global__ __launch_bounds__(1024) void row_read_kernel(const char *in, int64_t row_bytes, unsigned *sink) {
+  const u32x4 *row = (const u32x4 *)(in + (int64_t)blockIdx.x * row_bytes);
+  const int chunks = (int)(row_bytes / 16);
+  unsigned acc = 0;
+  for (int c0 = threadIdx.x; c0 < chunks; c0 += 4 * blockDim.x) {
+    u32x4 raw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + u * (int)blockDim.x < chunks) raw[u] = __builtin_nontemporal_load(row + c0 + u * blockDim.x);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + u * (int)blockDim.x < chunks) acc ^= raw[u].x ^ raw[u].y ^ raw[u].z ^ raw[u].w;
+  }
+  if (acc == 0x12345677u) *sink = acc;
+}
+
+extern "C" int floor_row_read(const void *in, int64_t rows, int64_t row_bytes, int threads, void *sink, void *stream) {
+  if (rows <= 0 || row_bytes <= 0 || row_bytes % 16 != 0 || threads < 64 || threads > 1024 || !sink) return 1;
+  hipLaunchKernelGGL(row_read_kernel, dim3((unsigned)rows), dim3((unsigned)threads), 0, (hipStream_t)stream,
+                     (const char *)in, row_bytes, (unsigned *)sink);
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 

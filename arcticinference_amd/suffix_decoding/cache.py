@@ -53,6 +53,48 @@ def _extend(tree: SuffixTree, seq_id: int, tokens: Tokens) -> None:
         tree.extend(seq_id, tokens)
 
 
+class _ResponseSlots:
+    """Which sequence of the global tree holds which request's response.
+
+    Sequence numbers are 31-bit and handed out by a counter that wraps; ``by_request`` keeps the
+    responses in the order they were given a sequence, which is the order of eviction."""
+
+    def __init__(self, limit: int):
+        self.limit = limit                            # < 0: no limit
+        self.by_request: Dict[Hashable, int] = {}     # insertion order = age
+        self.holder: Dict[int, Hashable] = {}
+        self.counter = 0
+
+    def release(self, req_id: Hashable) -> int:
+        seq = self.by_request.pop(req_id)
+        del self.holder[seq]
+        return seq
+
+    def take(self, req_id: Hashable, is_active) -> List[int]:
+        """Give ``req_id`` the next sequence number that is free or whose holder has finished, then apply
+        the limit.  Returns the sequences whose responses have to leave the tree, in that order: a finished
+        holder of the number taken first, then the oldest responses beyond the limit (never the one just
+        added).  Reference cache.py:306-345."""
+        while True:
+            seq = self.counter
+            self.counter = (seq + 1) & _SEQ_ID_MASK
+            previous = self.holder.get(seq)
+            if previous is None or not is_active(previous):
+                break
+        leaving = []
+        if previous is not None:
+            leaving.append(self.release(previous))
+        self.by_request[req_id] = seq
+        self.holder[seq] = req_id
+        if self.limit >= 0:
+            assert self.limit != 0   # with a limit of 0 no response is ever given a sequence
+            excess = len(self.by_request) - self.limit
+            if excess > 0:
+                oldest = [r for r in self.by_request if r != req_id][:excess]
+                leaving.extend(self.release(r) for r in oldest)
+        return leaving
+
+
 class SuffixDecodingCache:
 
     def __init__(self, max_tree_depth: int = 64, max_cached_requests: int = -1):
@@ -63,12 +105,9 @@ class SuffixDecodingCache:
             raise ValueError("max_cached_requests must be at most 2^31")
         self._max_tree_depth = max_tree_depth
         self._max_cached_requests = max_cached_requests
-        self._global_tree = SuffixTree(max_tree_depth)
-        self._local_trees: Dict[Hashable, SuffixTree] = {}
-        # request id <-> sequence id in the global tree, for every cached response
-        self._req_to_seq_id: Dict[Hashable, int] = {}
-        self._seq_to_req_id: Dict[int, Hashable] = {}
-        self._next_seq_id = 0
+        self._global_tree = SuffixTree(max_tree_depth)   # the reference's simulator reads this attribute
+        self._prompt_trees: Dict[Hashable, SuffixTree] = {}
+        self._slots = _ResponseSlots(max_cached_requests)
 
     @property
     def max_tree_depth(self) -> int:
@@ -81,53 +120,56 @@ class SuffixDecodingCache:
     @property
     def active_requests(self) -> KeysView:
         """Requests between ``start_request`` and ``stop_request`` (their prompts are held)."""
-        return self._local_trees.keys()
+        return self._prompt_trees.keys()
 
     @property
     def cached_requests(self) -> KeysView:
         """Requests whose responses are in the global tree."""
-        return self._req_to_seq_id.keys()
+        return self._slots.by_request.keys()
+
+    def _active_tree(self, req_id: Hashable) -> SuffixTree:
+        try:
+            return self._prompt_trees[req_id]
+        except KeyError:
+            raise ValueError(f"Request '{req_id}' is not active") from None
 
     def start_request(self, req_id: Hashable, prompt_token_ids: Tokens):
         """Begin a request: its prompt goes into a tree of its own, and (unless the global tree is switched
-        off) a slot for its response is taken in the global tree, evicting the oldest response if the
+        off) a sequence for its response is taken in the global tree, evicting the oldest response if the
         limit is reached (reference cache.py:120-157)."""
-        if req_id in self._local_trees:
+        if req_id in self._prompt_trees:
             raise ValueError(f"Request '{req_id}' is already active")
-        prompt_token_ids = _validated(prompt_token_ids)
-        tree = SuffixTree(self._max_tree_depth)
-        self._local_trees[req_id] = tree
-        _extend(tree, 0, prompt_token_ids)
-        if self._max_cached_requests != 0:
-            if req_id in self._req_to_seq_id:
-                self.evict_cached_response(req_id)
-            self._generate_seq_id(req_id)
+        tokens = _validated(prompt_token_ids)
+        tree = self._prompt_trees[req_id] = SuffixTree(self._max_tree_depth)
+        _extend(tree, 0, tokens)
+        if self._max_cached_requests == 0:
+            return
+        if req_id in self._slots.by_request:     # an earlier response under the same id
+            self.evict_cached_response(req_id)
+        for seq in self._slots.take(req_id, self._prompt_trees.__contains__):
+            self._global_tree.remove(seq)
 
     def stop_request(self, req_id: Hashable):
         """End a request: its prompt tree is dropped; its response stays cached until evicted
         (reference cache.py:159-175)."""
-        if req_id not in self._local_trees:
-            raise ValueError(f"Request '{req_id}' is not active")
-        del self._local_trees[req_id]
+        self._active_tree(req_id)
+        del self._prompt_trees[req_id]
 
     def add_active_response(self, req_id: Hashable, token_ids: Tokens):
         """Append generated tokens to the request's own tree and to its response in the global tree
         (reference cache.py:177-207)."""
-        if req_id not in self._local_trees:
-            raise ValueError(f"Request '{req_id}' is not active")
-        token_ids = _validated(token_ids)
-        _extend(self._local_trees[req_id], 0, token_ids)
-        seq_id = self._req_to_seq_id.get(req_id)
-        if seq_id is not None:
-            _extend(self._global_tree, seq_id, token_ids)
+        own = self._active_tree(req_id)
+        tokens = _validated(token_ids)
+        _extend(own, 0, tokens)
+        seq = self._slots.by_request.get(req_id)
+        if seq is not None:
+            _extend(self._global_tree, seq, tokens)
 
     def evict_cached_response(self, req_id: Hashable):
         """Remove the request's response from the global tree (reference cache.py:209-226)."""
-        if req_id not in self._req_to_seq_id:
+        if req_id not in self._slots.by_request:
             raise ValueError(f"Request '{req_id}' is not cached")
-        seq_id = self._req_to_seq_id.pop(req_id)
-        self._seq_to_req_id.pop(seq_id)
-        self._global_tree.remove(seq_id)
+        self._global_tree.remove(self._slots.release(req_id))
 
     def speculate(self, req_id: Hashable, context: Tokens, max_spec_tokens: Optional[int] = None,
                   max_spec_factor: float = 1.0, max_spec_offset: float = 0.0, min_token_prob: float = 0.1,
@@ -137,47 +179,16 @@ class SuffixDecodingCache:
         depth) and at most ``max_spec_factor * match_len + max_spec_offset``, each with an estimated
         probability of at least ``min_token_prob`` (reference cache.py:228-304; a tie goes to the
         request's own tree)."""
-        if req_id not in self._local_trees:
-            raise ValueError(f"Request '{req_id}' is not active")
+        own_tree = self._active_tree(req_id)
         context = _validated(context)
-        if max_spec_tokens is None:
-            max_spec_tokens = self._max_tree_depth
-        if len(context) > self._max_tree_depth:
-            context = context[-self._max_tree_depth:]
-        drafts = []
-        for tree in (self._local_trees[req_id], self._global_tree):
-            if isinstance(context, np.ndarray):
-                drafts.append(tree.speculate_ndarray(np.ascontiguousarray(context), max_spec_tokens, max_spec_factor,
-                                                     max_spec_offset, min_token_prob, use_tree_spec))
-            else:
-                drafts.append(tree.speculate(context, max_spec_tokens, max_spec_factor, max_spec_offset,
-                                             min_token_prob, use_tree_spec))
-        own, shared = drafts
-        return SuffixDecodingDraft.from_native(own if own.score >= shared.score else shared)
-
-    def _generate_seq_id(self, req_id: Hashable) -> int:
-        # the next sequence id (mod 2^31) that is free or belongs to a response of a finished request,
-        # which is then evicted (reference cache.py:306-334)
-        while True:
-            seq_id = self._next_seq_id
-            self._next_seq_id = (self._next_seq_id + 1) & _SEQ_ID_MASK
-            holder = self._seq_to_req_id.get(seq_id)
-            if holder is None or holder not in self._local_trees:
-                break
-        if seq_id in self._seq_to_req_id:
-            del self._req_to_seq_id[self._seq_to_req_id[seq_id]]
-            del self._seq_to_req_id[seq_id]
-            self._global_tree.remove(seq_id)
-        self._req_to_seq_id[req_id] = seq_id
-        self._seq_to_req_id[seq_id] = req_id
-        self._maybe_evict_requests(seq_id)
-        return seq_id
-
-    def _maybe_evict_requests(self, new_seq_id: int):
-        # oldest first (dict order = order of insertion), never the slot just taken (reference cache.py:336-345)
-        if self._max_cached_requests < 0:
-            return
-        assert self._max_cached_requests != 0
-        while len(self._req_to_seq_id) > self._max_cached_requests:
-            victim = next(r for r, s in self._req_to_seq_id.items() if s != new_seq_id)
-            self.evict_cached_response(victim)
+        depth = self._max_tree_depth
+        budget = depth if max_spec_tokens is None else max_spec_tokens
+        if len(context) > depth:
+            context = context[-depth:]
+        limits = (budget, max_spec_factor, max_spec_offset, min_token_prob, use_tree_spec)
+        if isinstance(context, np.ndarray):
+            context = np.ascontiguousarray(context)
+            own, shared = (t.speculate_ndarray(context, *limits) for t in (own_tree, self._global_tree))
+        else:
+            own, shared = (t.speculate(context, *limits) for t in (own_tree, self._global_tree))
+        return SuffixDecodingDraft.from_native(shared if shared.score > own.score else own)

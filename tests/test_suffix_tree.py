@@ -252,6 +252,29 @@ def test_cache_eviction_is_first_in_first_out_and_limits():
     assert list(cache.cached_requests) == ["r1", "r2"] and cache._global_tree.num_seqs() == 1
 
 
+def test_cache_sequence_numbers_wrap_skip_active_holders_and_displace_finished_ones():
+    # reference cache.py:306-334: 31-bit numbers from a wrapping counter; a number whose holder is still active is
+    # passed over, a number whose holder has finished is taken and that response leaves the tree
+    cache = SuffixDecodingCache(max_tree_depth=4)
+    cache._slots.counter = 0x7FFFFFFE
+    for name in ("a", "b", "c"):                      # numbers 2^31-2, 2^31-1, 0
+        cache.start_request(name, [1])
+        cache.add_active_response(name, [20, 21, 22])
+    assert [cache._slots.by_request[n] for n in "abc"] == [0x7FFFFFFE, 0x7FFFFFFF, 0]
+    cache.stop_request("b")
+    cache._slots.counter = 0x7FFFFFFE                 # the counter comes round again
+    cache.start_request("d", [1])                     # a is active: passed over; b has finished: displaced
+    assert cache._slots.by_request["d"] == 0x7FFFFFFF and "b" not in cache.cached_requests
+    assert list(cache.cached_requests) == ["a", "c", "d"]
+    assert cache._global_tree.num_seqs() == 2             # a and c: b has left, d has no tokens yet
+    cache.start_request("e", [1])                     # c (number 0) is active: passed over as well
+    assert cache._slots.by_request["e"] == 1
+    cache.add_active_response("d", [30, 31])
+    assert cache._global_tree.num_seqs() == 3
+    assert cache.speculate("e", [1, 30], max_spec_tokens=1).token_ids == [31]
+    assert cache._global_tree.check_integrity() == ""
+
+
 def test_cache_validates_ndarrays_and_truncates_context():
     cache = SuffixDecodingCache(max_tree_depth=4)
     with pytest.raises(ValueError, match="dtype=int32"):

@@ -38,6 +38,17 @@ def test_random(ops, dtype, nhd, shape):
 
 
 @pytest.mark.parametrize("nhd", [True, False])
+@pytest.mark.parametrize("shape", [
+    (2050, 8, 128, 16, 130),   # thousands of tokens: a last workgroup that is partly idle
+    (2051, 3, 80, 4, 520),     # rows that are no multiple of a wave's 64 groups
+    (4096, 32, 128, 16, 256),  # rows wider than one workgroup
+])
+def test_many_tokens(ops, nhd, shape):
+    T, H, D, bs, NB = shape
+    run_both(ops, *make_case(T, H, D, bs, NB, torch.bfloat16, nhd, seed=31, pad=0.15))
+
+
+@pytest.mark.parametrize("nhd", [True, False])
 def test_slots_outside_the_cache_move_nothing(ops, nhd):
     key, value, kc, vc, ksc, vsc, slots = make_case(20, 4, 64, 8, 3, torch.bfloat16, nhd, seed=23)
     bad = [2, 11]

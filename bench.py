@@ -296,6 +296,7 @@ def load_floor_kernels():
     lib = ctypes.CDLL(path)
     vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
     lib.floor_lstm_traffic.argtypes = [vp, vp, vp, vp, vp, i64, i32, vp]
+    lib.floor_ln_traffic.argtypes = [vp, vp, i64, i32, vp]
     lib.floor_stream.argtypes = [vp, i32, vp, i32, i64, i32, vp, vp]
     lib.floor_valu_rate.argtypes = [i32, i32, i32, vp, vp]
     lib.floor_node.argtypes = [vp, vp, i32, i32, i32, vp]
@@ -372,6 +373,9 @@ def bench_speculator(ops, dev, steps, warmup):
             floor.floor_lstm_traffic(S[i % sets][k].data_ptr(), Z[i % sets][k].data_ptr(), C0[i % sets].data_ptr(),
                                      OS[0].data_ptr(), OS[1].data_ptr(), T, Hd, stream)
 
+    def ln_traffic_only(i):
+        floor.floor_ln_traffic(X[i % sets].data_ptr(), OS[0].data_ptr(), T, Hd, torch.cuda.current_stream().cuda_stream)
+
     cases = [("sum_lstm", lstm3, 22 * Hd * T, 3),
              ("sum_lstm_shared_z", lstm3_shared_z, 16 * Hd * T, 3),
              ("lookup_repeat_sum_lstm_as_three_ops", lstm3_lookup_repeat, 16 * Hd * T, 3),
@@ -381,6 +385,7 @@ def bench_speculator(ops, dev, steps, warmup):
              ("add_ln_gelu_as_three_ops", add_ln_gelu_separate, 6 * Hd * T, 1)]
     if floor is not None:
         cases.insert(1, ("sum_lstm_traffic_only_floor", lstm3_traffic_only, 22 * Hd * T, 3))
+        cases.append(("speculator_ln_traffic_only_floor", ln_traffic_only, 4 * Hd * T, 1))
     out = {}
     for name, fn, per_call, calls in cases:
         for i in range(warmup):
@@ -703,15 +708,18 @@ def bench_decode_mix(ops, dev, steps):
             gr.replay()
         torch.cuda.synchronize()
         counter = iter(range(10 ** 9))
-        us = event_times_us(lambda: graphs[next(counter) % sets].replay(), max(40, steps))
+        us = event_times_us(lambda: graphs[next(counter) % sets].replay(), max(200, steps))
         med = statistics.median(us)
         # the same graphs replayed back to back, one pair of events around all of them: per step, without the
         # idle gap in front of a lone replay
         def all_sets():
             for gr in graphs:
                 gr.replay()
-        b2b = statistics.median(event_times_us(all_sets, max(10, steps // 4))) / sets
-        out.update({f"us_per_step_graph{name}": round(med, 2), f"GBps{name}": round(nbytes / med / 1e3, 1),
+        b2b = statistics.median(event_times_us(all_sets, max(25, steps // 4))) / sets
+        us.sort()
+        out.update({f"us_per_step_graph{name}": round(med, 2),
+                    f"us_per_step_graph_p10_p90{name}": [round(us[len(us) // 10], 2), round(us[len(us) * 9 // 10], 2)],
+                    f"replays{name}": len(us), f"GBps{name}": round(nbytes / med / 1e3, 1),
                     f"hbm_frac{name}": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4),
                     f"us_per_step_graphs_back_to_back{name}": round(b2b, 2),
                     f"hbm_frac_back_to_back{name}": round(nbytes / b2b / 1e3 / HBM_PEAK_GBS, 4)})

@@ -3,6 +3,7 @@
 //
 //   floor_lstm_traffic   the loads and stores of sum_lstm (nine 16-byte loads per lane from the rows of
 //                        states, z4 and prev_cell, two 16-byte stores), one workgroup per row, no arithmetic
+//   floor_ln_traffic     the load and the store of speculator_ln (one 16-byte chunk per lane, one workgroup per row)
 //   floor_row_read       the loads of the row-argmax kernel (one workgroup per row), nothing computed
 //   floor_node           an empty kernel, or one that makes a single memory round trip: the fixed cost of a node
 //   floor_valu_rate      chains of one vector-ALU operation, for its issue rate per SIMD
@@ -31,6 +32,14 @@ __global__ void lstm_traffic_kernel(const char *s, const char *z, const char *pc
   const u32x4 a = v[0] ^ v[1] ^ v[2] ^ v[3] ^ v[8], b = v[4] ^ v[5] ^ v[6] ^ v[7];
   __builtin_nontemporal_store(a, (u32x4 *)(out_cell + row1) + c);
   __builtin_nontemporal_store(b, (u32x4 *)(out_state + row1) + c);
+}
+
+__global__ void ln_traffic_kernel(const char *x, char *out, int hidden) {
+  const int c = threadIdx.x;
+  if (c >= hidden / 8) return;
+  const size_t row = (size_t)blockIdx.x * hidden * 2;
+  const u32x4 v = __builtin_nontemporal_load((const u32x4 *)(x + row) + c);
+  __builtin_nontemporal_store(v, (u32x4 *)(out + row) + c);
 }
 
 struct Three {
@@ -162,6 +171,13 @@ extern "C" int floor_row_read(const void *in, int64_t rows, int64_t row_bytes, i
   hipLaunchKernelGGL(row_read_kernel, dim3((unsigned)rows), dim3((unsigned)threads), 0, (hipStream_t)stream,
                      (const char *)in, row_bytes, (unsigned *)sink);
   return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+extern "C" int floor_ln_traffic(const void *x, void *out, int64_t rows, int hidden, void *stream) {
+  if (hidden % 8 || hidden / 8 > 1024 || rows <= 0) return 1;
+  hipLaunchKernelGGL(ln_traffic_kernel, dim3((unsigned)rows), dim3((unsigned)((hidden / 8 + 63) & ~63)), 0,
+                     (hipStream_t)stream, (const char *)x, (char *)out, hidden);
+  return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
 extern "C" int floor_lstm_traffic(const void *s, const void *z, const void *pc, void *out_state, void *out_cell,

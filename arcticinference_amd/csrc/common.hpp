@@ -14,6 +14,15 @@ namespace arctic {
 int fail(int code, const char *fmt, ...);
 int check_launch(const char *what);
 
+// A row pitch (in elements) that `rows` rows of a tensor inside a 2^47-byte address space can have: not negative,
+// and the last row's byte offset stays inside that space, so that no product of the two formed later, on the host
+// or in a kernel, overflows 64 bits.
+inline bool pitch_ok(int64_t pitch_elems, int64_t rows, int elem_bytes) {
+  if (pitch_elems < 0) return false;
+  const int64_t limit = ((int64_t)1 << 47) / elem_bytes;
+  return pitch_elems <= limit / (rows > 1 ? rows - 1 : 1);
+}
+
 // ---- 16-bit floats ---------------------------------------------------------
 // Activation element types. to_float is exact; from_float rounds to nearest
 // even (what __float2bfloat16 / __float2half do in the reference,

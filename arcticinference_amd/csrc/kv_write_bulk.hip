@@ -570,10 +570,22 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
     return fail(ARCTIC_ERR_UNSUPPORTED, "%s: Unsupported data type of kv cache: %d", fn, kv_cache_dtype);
   if (!keys || !values || !slot_mapping || !key_cache_ptrs || !value_cache_ptrs)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
+  if (block_size > (1 << 20) || num_blocks > ((int64_t)1 << 40))
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: block_size beyond 2^20 or num_blocks beyond 2^40", fn);
+  {
+    const int src_bytes = src_dtype == ARCTIC_DTYPE_F32 ? 4 : 2;
+    const int64_t src_rows = sel_in.mode != kSelectNone && sel_in.indices ? std::max(num_tokens, sel_in.num_src_rows) : num_tokens;
+    if (!pitch_ok(key_stride, src_rows, src_bytes) || !pitch_ok(value_stride, src_rows, src_bytes) ||
+        !pitch_ok(block_stride, num_blocks, kv_cache_dtype == ARCTIC_KV_AUTO ? src_bytes : 1))
+      return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: row or block pitch out of range", fn);
+    if (sel_in.mode != kSelectNone && (!pitch_ok(sel_in.out_key_stride, sel_in.num_out_rows, src_bytes) ||
+                                       !pitch_ok(sel_in.out_value_stride, sel_in.num_out_rows, src_bytes)))
+      return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: negative number of output rows or row pitch out of range", fn);
+  }
   SelectArgs sel = sel_in;
   if (sel.mode != kSelectNone) {
-    if (sel.num_out_rows < 0 || sel.out_key_stride < 0 || sel.out_value_stride < 0)
-      return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: negative number of output rows or row pitch", fn);
+    if (sel.num_out_rows < 0 || sel.num_out_rows > 0x7fffffffLL || sel.out_key_stride < 0 || sel.out_value_stride < 0)
+      return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: negative number of output rows or row pitch, or 2^31 output rows or more", fn);
     if (sel.num_out_rows == 0) sel.mode = kSelectNone;   // no row to copy to: the plain write
   }
   if (sel.mode != kSelectNone) {

@@ -114,6 +114,14 @@ extern "C" int arctic_reshape_and_cache_flash_fp4(
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: sizes must be positive", fn);
   if (head_size % 16)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: head_size must be a multiple of 16 (one scale per 16 elements)", fn);
+  if (num_tokens > 0x7fffffffLL || (int64_t)num_heads * head_size > (1 << 24) || block_size > (1 << 20) ||
+      num_blocks < 0 || num_blocks > ((int64_t)1 << 40))
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: num_tokens beyond 2^31, num_heads*head_size beyond 2^24, block_size beyond "
+                "2^20 or num_blocks outside [0, 2^40]", fn);
+  if (!pitch_ok(key_stride, num_tokens, 2) || !pitch_ok(value_stride, num_tokens, 2) ||
+      !pitch_ok(block_stride, num_blocks, 1) || !pitch_ok(page_stride, block_size, 1) ||
+      !pitch_ok(head_stride, num_heads, 1))
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: row, block, page or head pitch out of range", fn);
   if (!key || !value || !key_cache || !value_cache || !key_scale_cache || !value_scale_cache || !slot_mapping)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
   if (((uintptr_t)key | (uintptr_t)value) & 15 || (num_tokens > 1 && ((key_stride | value_stride) & 7)))

@@ -262,6 +262,8 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
   if (rows == 0) return ARCTIC_OK;
   if (!out || !logits) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
   const int es = dtype == ARCTIC_DTYPE_F32 ? 4 : 2;
+  if (cols > (1 << 30) || !pitch_ok(row_stride, rows, es))
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: more than 2^30 columns, or a row pitch out of range", fn);
   const int64_t stride_bytes = row_stride * es;
   const bool vec = ((uintptr_t)logits % 16 == 0) && (stride_bytes % 16 == 0 || rows == 1);
   const int per_chunk = 16 / es;

@@ -129,6 +129,10 @@ extern "C" int arctic_gather_rows(int num_tensors, const void *const *src, void 
     if (row_bytes[t] < 0 || src_row_stride_bytes[t] < 0 || dst_row_stride_bytes[t] < 0)
       return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: tensor %d: negative size or pitch", fn, t);
     if (row_bytes[t] == 0) continue;
+    const int64_t most_rows = std::max(num_indices, num_indexed_rows);
+    if (row_bytes[t] > ((int64_t)1 << 40) || !pitch_ok(src_row_stride_bytes[t], most_rows, 1) ||
+        !pitch_ok(dst_row_stride_bytes[t], most_rows, 1))
+      return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: tensor %d: row size or pitch out of range", fn, t);
     if (!src[t] || !dst[t]) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: tensor %d: null pointer", fn, t);
     const int c = tab.count++;
     tab.src[c] = (const char *)src[t];

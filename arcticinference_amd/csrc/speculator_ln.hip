@@ -216,12 +216,15 @@ static int ln_entry(const char *fn, void *out, const void *in, const void *weigh
   if (dtype != ARCTIC_DTYPE_F16 && dtype != ARCTIC_DTYPE_BF16)
     return fail(ARCTIC_ERR_UNSUPPORTED, "%s: only fp16 and bf16 are supported.", fn);
   if (hidden <= 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: hidden size must be > 0", fn);
+  if (hidden > (1 << 30)) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: hidden size beyond 2^30", fn);
   if (rows < 0 || rows > 0x7fffffffLL) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: bad row count", fn);
   if (glue.activation != ARCTIC_ACT_NONE && glue.activation != ARCTIC_ACT_GELU &&
       glue.activation != ARCTIC_ACT_GELU_TANH)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: unknown activation %d", fn, glue.activation);
   if (rows == 0) return ARCTIC_OK;
   if (!out || !in) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
+  if (!pitch_ok(in_row_stride, rows, 2) || !pitch_ok(hidden, rows, 2))
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: row pitch out of range", fn);
   hipStream_t s = (hipStream_t)stream;
   if (dtype == ARCTIC_DTYPE_BF16)
     launch_ln<BF16>(out, in, weight, bias, rows, hidden, in_row_stride, eps, glue, s);
@@ -241,6 +244,8 @@ extern "C" int arctic_speculator_add_ln_act(void *out, const void *in, const voi
                                             const void *bias, int64_t rows, int hidden, int64_t in_row_stride,
                                             int64_t z_row_stride, float alpha, float eps, int activation,
                                             float out_scale, int dtype, void *stream) {
+  if (!pitch_ok(z_row_stride, rows, 2))
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "speculator_add_ln_act: row pitch of z out of range");
   const LnGlue glue = {(const char *)z, z_row_stride * 2, nullptr, 0, alpha, activation, out_scale};
   return ln_entry("speculator_add_ln_act", out, in, weight, bias, rows, hidden, in_row_stride, eps, glue, dtype,
                   stream);
@@ -254,6 +259,8 @@ extern "C" int arctic_speculator_embed_add_ln_act(void *out, const void *in, con
   const char *fn = "speculator_embed_add_ln_act";
   if (rows > 0 && (!emb_table || !token_ids)) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null embedding table or token ids", fn);
   if (rows > 0 && num_embeddings <= 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: the embedding table has no rows", fn);
+  if (!pitch_ok(emb_row_stride, num_embeddings, 2))
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: row pitch of the embedding table out of range", fn);
   const LnGlue glue = {(const char *)emb_table, emb_row_stride * 2, token_ids, num_embeddings, alpha, activation, out_scale};
   return ln_entry(fn, out, in, weight, bias, rows, hidden, in_row_stride, eps, glue, dtype, stream);
 }

@@ -463,6 +463,10 @@ static int sum_lstm_entry(const char *fn, bool shared_z, void *out_state, void *
   if (!out_state || !out_cell || !states || !z)   // prev_cell may be null: a cell of zeros
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null tensor pointer", fn);
   if (z_index && z_rows <= 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: the embedding table has no rows", fn);
+  if (D > (1 << 28)) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: D_gate beyond 2^28", fn);
+  if (!pitch_ok(s_stride, rows, 2) || !pitch_ok(z_stride, z_index ? z_rows : rows, 2) ||
+      !pitch_ok(pc_stride, rows, 2) || !pitch_ok(out_stride, rows, 2))
+    return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: row pitch out of range", fn);
   LstmParams p;
   p.z_index = z_index;
   p.z_rows = z_rows;

@@ -14,6 +14,13 @@
  * ARCTIC_ERR_* code on failure; arctic_last_error() then holds a message for the
  * calling thread.  The library keeps no reference to any argument after return.
  *
+ * Sizes are checked before anything is computed from them: row and token counts
+ * must be below 2^31, widths (hidden, D_gate, columns, num_heads * head_size) at
+ * most 2^30 / 2^28 / 2^30 / 2^24, block_size at most 2^20, num_blocks at most
+ * 2^40, and every pitch non-negative and small enough that its last row still
+ * starts inside a 2^47-byte address space.  A call outside these limits returns
+ * ARCTIC_ERR_INVALID_ARGUMENT and launches nothing.
+ *
  * Reference paths below are relative to the ArcticInference source tree.
  */
 #ifndef ARCTIC_MI355X_H

@@ -257,3 +257,26 @@ def test_no_previous_cell_equals_a_cell_of_zeros(ops, cfg, dtype, fast):
     if s3 is not None:
         g3 = ops.sum_lstm(s3, d["z4"].contiguous().view(rows, 1, 4 * D), None, *tail)
         assert g3[0].shape == (rows, 1, D) and torch.equal(g3[1].view(rows, D), ops.sum_lstm(d["states"], d["z4"], zeros, *tail)[1])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [512, 100])        # the 16-byte-lane kernel and the element-wise one
+def test_saturated_gates_zero_rows_and_extreme_magnitudes(ops, dtype, D):
+    """Finite inputs at the ends of the formats' ranges: gates driven to both ends of the sigmoid, rows of zeros
+    (the norm divides by sqrt(eps)), tiny values, and values whose squares overflow fp32 (the inverse RMS is then
+    0 and the normalised row 0).  The results stay finite and match the oracle."""
+    big = 6.0e4 if dtype == torch.float16 else 3.0e38
+    c = make_lstm_case(rows=8, D=D, dtype=dtype, seed=77)
+    s, z, pc = c["states"], c["z4"], c["prev_cell"]
+    f, i, o, g = (slice(k * D, (k + 1) * D) for k in range(4))   # any order covers every gate: all four are driven
+    s[0, f], s[0, i], s[0, o] = 80.0, -80.0, 80.0              # saturated gates, ordinary candidate
+    s[1, :], z[1, :] = 0.0, 0.0                                # a row of zeros
+    pc[1, :] = 0.0
+    s[2, :], z[2, :] = 1.0e-7 if dtype == torch.float16 else 1.0e-30, 0.0   # tiny
+    s[3, g], z[3, :] = big / 8, 0.0                            # squares overflow fp32 in one gate
+    s[4, :] = -80.0                                            # everything closed
+    pc[5, :] = big / 4                                         # a huge previous cell, kept by an open gate
+    s[5, f], s[5, i], s[5, o], s[5, g] = 80.0, 80.0, 80.0, 80.0
+    z[5, :] = 0.0
+    got_s, got_c, want_s, want_c = run(ops, c, alpha=1.0)
+    assert torch.isfinite(want_s.float()).all() and torch.isfinite(want_c.float()).all()

@@ -80,6 +80,7 @@ struct BulkParams {
   int select_mode;   // kSelectNone / kSelectByRowMap / kSelectByScan (the vector kernels take it as a template argument)
 #ifdef ARCTIC_TUNING
   int stores_before_loads;  // measurement build: a batch is converted and stored before the next one is requested
+  unsigned items;           // measurement build: not 0 = workgroups loop over this many items (ARCTIC_BULK_PERSISTENT)
 #endif
 };
 
@@ -201,14 +202,12 @@ __device__ __forceinline__ void select_leftover_rows(const BulkParams &p, unsign
 // are built: 512 x 2 (a workgroup moves two batches or more) and 256 x 4 (decode:
 // few tokens, a single batch per workgroup).
 template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll, int kSelect>
-__global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
-    const BulkParams p, const LayerTables tab) {
+__device__ __forceinline__ void bulk_item(const BulkParams &p, const LayerTables &tab, unsigned block) {
   constexpr bool kCopy = std::is_same<Dst, Copy>::value;
   constexpr int kDstElemBytes = kCopy ? Src::kBytes : 1;
 
   __shared__ RowDesc rows[2 * kLayersPerLaunch];
 
-  unsigned block = blockIdx.x;
   if constexpr (kSelect) {
     if (block < p.index_blocks) {  // uniform over the workgroup, before any barrier
       select_leftover_rows<Src, kPow2, kBulkThreads, kSelect>(p, block);
@@ -368,6 +367,21 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
   }
 }
 
+template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll, int kSelect>
+__global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
+    const BulkParams p, const LayerTables tab) {
+#ifdef ARCTIC_TUNING
+  if (p.items) {   // measurement build: a grid of fewer workgroups, each taking every gridDim.x-th item in turn
+    for (unsigned item = blockIdx.x; item < p.items; item += gridDim.x) {
+      bulk_item<Src, Dst, kPow2, kBulkThreads, kUnroll, kSelect>(p, tab, item);
+      __syncthreads();   // the next item rewrites the row descriptors
+    }
+    return;
+  }
+#endif
+  bulk_item<Src, Dst, kPow2, kBulkThreads, kUnroll, kSelect>(p, tab, blockIdx.x);
+}
+
 // Fallback for shapes or addresses that do not allow 16-byte accesses: one
 // element per lane per step, any alignment.  Same arithmetic, no vector access.
 template <typename SrcElem, typename Dst>
@@ -474,6 +488,22 @@ __global__ __launch_bounds__(kScalarThreads) void kv_write_bulk_scalar_kernel(
 template <typename Src, typename Dst, int kSelect>
 static void launch_vec_shape(const BulkParams &p, const LayerTables &tab, int64_t grid, bool wide, hipStream_t s) {
   const dim3 g((unsigned)grid);
+#ifdef ARCTIC_TUNING
+  // measurement build: ARCTIC_BULK_SHAPE = 1: 512 lanes x 4 chunks, 2: 1024 x 2, 3: 1024 x 4, 4: 1024 x 1
+  if constexpr (kSelect == kSelectNone) {
+    const char *e = getenv("ARCTIC_BULK_SHAPE");
+    const int shape = e ? atoi(e) : 0;
+    if (shape && p.chunk_shift >= 0) {
+      switch (shape) {
+        case 1: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 512, 4, kSelectNone>), g, dim3(512), 0, s, p, tab); break;
+        case 2: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 1024, 2, kSelectNone>), g, dim3(1024), 0, s, p, tab); break;
+        case 3: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 1024, 4, kSelectNone>), g, dim3(1024), 0, s, p, tab); break;
+        default: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 1024, 1, kSelectNone>), g, dim3(1024), 0, s, p, tab); break;
+      }
+      return;
+    }
+  }
+#endif
   if (p.chunk_shift >= 0) {
     if (wide)
       hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 512, 2, kSelect>), g, dim3(512), 0, s, p, tab);
@@ -695,6 +725,7 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
     if (const char *e = getenv("ARCTIC_BULK_WIDE")) wide = atoi(e) != 0;
     p.stores_before_loads = 0;
     if (const char *e = getenv("ARCTIC_BULK_STORES_FIRST")) p.stores_before_loads = atoi(e) != 0;
+    p.items = 0;
 #endif
     p.layers_per_group = (count + groups - 1) / groups;
     p.groups_per_token = (count + p.layers_per_group - 1) / p.layers_per_group;
@@ -705,10 +736,19 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
     if (grid > 0x7fffffffLL)
       return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: too many tokens (%lld)", fn, (long long)num_tokens);
 
+    int64_t workgroups = grid;
+#ifdef ARCTIC_TUNING
+    if (const char *e = getenv("ARCTIC_BULK_PERSISTENT")) {
+      if (atoi(e) > 0 && vec && !p.indices) {   // that many workgroups, each looping over the grid's items
+        p.items = (unsigned)grid;
+        workgroups = std::min<int64_t>(grid, atoi(e));
+      }
+    }
+#endif
     switch (kv_cache_dtype) {
-      case ARCTIC_KV_AUTO: dispatch_src<Copy>(vec, wide, src_dtype, p, tab, grid, s); break;
-      case ARCTIC_KV_FP8_E4M3: dispatch_src<E4M3>(vec, wide, src_dtype, p, tab, grid, s); break;
-      default: dispatch_src<E5M2>(vec, wide, src_dtype, p, tab, grid, s); break;
+      case ARCTIC_KV_AUTO: dispatch_src<Copy>(vec, wide, src_dtype, p, tab, workgroups, s); break;
+      case ARCTIC_KV_FP8_E4M3: dispatch_src<E4M3>(vec, wide, src_dtype, p, tab, workgroups, s); break;
+      default: dispatch_src<E5M2>(vec, wide, src_dtype, p, tab, workgroups, s); break;
     }
     const int rc = check_launch(fn);
     if (rc) return rc;

@@ -297,6 +297,7 @@ def load_floor_kernels():
     vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
     lib.floor_lstm_traffic.argtypes = [vp, vp, vp, vp, vp, i64, i32, vp]
     lib.floor_ln_traffic.argtypes = [vp, vp, i64, i32, vp]
+    lib.floor_stream_resident.argtypes = [vp, vp, i32, i64, i32, i32, vp]
     lib.floor_stream.argtypes = [vp, i32, vp, i32, i64, i32, vp, vp]
     lib.floor_valu_rate.argtypes = [i32, i32, i32, vp, vp]
     lib.floor_node.argtypes = [vp, vp, i32, i32, i32, vp]
@@ -982,6 +983,20 @@ def placement_sweep(ops, dev, steps):
                 "the same with 16-byte stores (a lane loads 32 adjacent bytes)": {
                     f"stores_to_{n}_regions": stream_GBps(4, 1, n, pieces * 98304) for n in (1, 2, 3)},
             }
+
+            # the scattered stream by resident workgroups of 1024 lanes (the best of four shapes): what the pattern
+            # costs when nothing but bandwidth shapes the kernel
+            def resident_GBps(ndst):
+                best = 0
+                for loads, groups in ((4, 256), (4, 768), (8, 256), (8, 512)):
+                    f = lambda: floor.floor_stream_resident(chunks[reps[0]].data_ptr(), high, ndst, 3 << 30, loads, groups, stream)
+                    for _ in range(2):
+                        assert f() == 0
+                    best = max(best, round((3 << 30) * 1.5 / statistics.median(event_times_us(f, steps)) / 1e3))
+                return best
+
+            out["bare_stream_GBps"]["scattered 2:1 stream by resident workgroups (1024 lanes, 4 or 8 loads per lane in flight)"] = {
+                f"stores_to_{n}_regions": resident_GBps(n) for n in (1, 2, 3)}
     return out
 
 
@@ -1089,20 +1104,44 @@ def bench_bulk_variants(dev, steps):
              ("256 lanes x 4 chunks", {"ARCTIC_BULK_WIDE": "0"}),
              ("one group of 40 layers per token", {"ARCTIC_BULK_GROUPS": "1"}),
              ("4 groups of 10 layers per token", {"ARCTIC_BULK_GROUPS": "4"}),
-             ("8 groups of 5 layers per token", {"ARCTIC_BULK_GROUPS": "8"})]
+             ("8 groups of 5 layers per token", {"ARCTIC_BULK_GROUPS": "8"}),
+             ("512 lanes x 4 chunks", {"ARCTIC_BULK_SHAPE": "1"}),
+             ("512 lanes x 4 chunks, one group of 40 layers", {"ARCTIC_BULK_SHAPE": "1", "ARCTIC_BULK_GROUPS": "1"}),
+             ("1024 lanes x 1 chunk", {"ARCTIC_BULK_SHAPE": "4"}),
+             ("1024 lanes x 2 chunks", {"ARCTIC_BULK_SHAPE": "2"}),
+             ("1024 lanes x 2 chunks, one group of 40 layers", {"ARCTIC_BULK_SHAPE": "2", "ARCTIC_BULK_GROUPS": "1"}),
+             ("1024 lanes x 4 chunks, one group of 40 layers", {"ARCTIC_BULK_SHAPE": "3", "ARCTIC_BULK_GROUPS": "1"}),
+             ("as shipped, 768 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "768"}),
+             ("as shipped, 1024 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "1024"}),
+             ("as shipped, 2048 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "2048"}),
+             ("1024 lanes x 2 chunks, 256 workgroups that loop", {"ARCTIC_BULK_SHAPE": "2", "ARCTIC_BULK_PERSISTENT": "256"}),
+             ("1024 lanes x 2 chunks, 512 workgroups that loop", {"ARCTIC_BULK_SHAPE": "2", "ARCTIC_BULK_PERSISTENT": "512"}),
+             ("1024 lanes x 4 chunks, one group of 40 layers, 256 workgroups that loop",
+              {"ARCTIC_BULK_SHAPE": "3", "ARCTIC_BULK_GROUPS": "1", "ARCTIC_BULK_PERSISTENT": "256"}),
+             ("1024 lanes x 4 chunks, one group of 40 layers, 512 workgroups that loop",
+              {"ARCTIC_BULK_SHAPE": "3", "ARCTIC_BULK_GROUPS": "1", "ARCTIC_BULK_PERSISTENT": "512"})]
     out = {name: [] for name, _ in cases}
+    written, same = {}, {}
     for _ in range(3):
         for name, env in cases:
-            for k in ("ARCTIC_BULK_STORES_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS"):
+            for k in ("ARCTIC_BULK_STORES_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT"):
                 os.environ.pop(k, None)
             os.environ.update(env)
+            # what the variant writes into the first and the last layer's caches, against the first variant's
+            probed = [w.key_caches[0], w.value_caches[0], w.key_caches[-1], w.value_caches[-1]]
+            for t in probed:
+                t.view(torch.int32).zero_()
             for _ in range(3):
                 launch()
+            sums = [int(t.view(torch.int32).sum(dtype=torch.int64)) for t in probed]
+            written.setdefault("first", sums)
+            same[name] = same.get(name, True) and sums == written["first"]
             out[name].append(round(statistics.mean(event_times_us(launch, max(10, steps // 4))), 1))
-    for k in ("ARCTIC_BULK_STORES_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS"):
+    for k in ("ARCTIC_BULK_STORES_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT"):
         os.environ.pop(k, None)
     return {name: {"kernel_us_rounds": v, "GBps": round(w.bytes / statistics.mean(v) / 1e3),
-                   "hbm_frac": round(w.bytes / statistics.mean(v) / 1e3 / HBM_PEAK_GBS, 4)} for name, v in out.items()}
+                   "hbm_frac": round(w.bytes / statistics.mean(v) / 1e3 / HBM_PEAK_GBS, 4),
+                   "writes_the_same_bytes": same[name]} for name, v in out.items()}
 
 
 def bench_argmax_variants(dev, steps):

@@ -10,6 +10,9 @@
 //   floor_stream         load-only, store-only or a 2:1 load:store stream in 64 KiB pieces, the pieces dealt
 //                        round robin over up to three buffers (which the caller places in different regions
 //                        of the HBM); the 2:1 stream also with its stores scattered as rows of 1 KiB
+//   floor_stream_resident the scattered 2:1 stream once more, shaped for bandwidth alone: as many workgroups of 1024
+//                        lanes as stay resident (one or two per CU), each looping over pieces with all of a piece's
+//                        loads (4 or 8 per lane) requested before the first store
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -85,6 +88,46 @@ __global__ void stream_kernel(Three src, int nsrc, Three dst, int ndst, int64_t 
     }
   }
   if (mode == 0 && acc == 0x12345677u) *sink = acc;
+}
+
+// The 2:1 stream with scattered 1 KiB rows (mode 3 of stream_kernel) by resident workgroups: a piece is kLoads x 16 KiB,
+// every lane requests its kLoads chunks of it at once, then stores the halves; the rows are dealt over `ndst` buffers.
+template <int kLoads>
+__global__ __launch_bounds__(1024) void resident_stream_kernel(const char *src, Three dst, int ndst, int64_t pieces,
+                                                                int scatter_bits) {
+  const unsigned rows_per_piece = kLoads * 8;
+  for (int64_t k = blockIdx.x; k < pieces; k += gridDim.x) {
+    const u32x4 *from = (const u32x4 *)(src + k * (int64_t)kLoads * 16384);
+    u32x4 v[kLoads];
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) v[u] = __builtin_nontemporal_load(from + u * 1024 + threadIdx.x);
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+      const u32x2 w = {v[u].x ^ v[u].z, v[u].y ^ v[u].w};
+      const unsigned i = u * 1024 + threadIdx.x;
+      const unsigned g = (unsigned)k * rows_per_piece + i / 128u, mask = (1u << scatter_bits) - 1u;
+      const unsigned row = (g & ~mask) | ((g * 40503u) & mask);
+      __builtin_nontemporal_store(w, (u32x2 *)(dst.p[row % ndst] + (int64_t)(row / ndst) * 1024) + i % 128);
+    }
+  }
+}
+
+// bytes_in of `src` (a multiple of loads x 16 KiB, at most 2^41) are read, half as many written, dealt over dst[0..ndst)
+extern "C" int floor_stream_resident(const void *src, void *const *dst, int ndst, int64_t bytes_in, int loads,
+                                     int workgroups, void *stream) {
+  if (!src || !dst || ndst < 1 || ndst > 3 || (loads != 4 && loads != 8) || workgroups < 1 || workgroups > 65535 ||
+      bytes_in <= 0 || bytes_in % ((int64_t)loads * 16384) || bytes_in > ((int64_t)1 << 41))
+    return 1;
+  Three d = {};
+  for (int i = 0; i < ndst; ++i) d.p[i] = (char *)dst[i];
+  const int64_t pieces = bytes_in / ((int64_t)loads * 16384);
+  const int scatter_bits = __builtin_ctzll((unsigned long long)(pieces * loads * 8));
+  hipStream_t s = (hipStream_t)stream;
+  if (loads == 4)
+    hipLaunchKernelGGL(resident_stream_kernel<4>, dim3(workgroups), dim3(1024), 0, s, (const char *)src, d, ndst, pieces, scatter_bits);
+  else
+    hipLaunchKernelGGL(resident_stream_kernel<8>, dim3(workgroups), dim3(1024), 0, s, (const char *)src, d, ndst, pieces, scatter_bits);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 
 // Issue rates of the vector ALU: every lane runs `iters` rounds of eight independent chains of one operation

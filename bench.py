@@ -297,7 +297,7 @@ def load_floor_kernels():
     vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
     lib.floor_lstm_traffic.argtypes = [vp, vp, vp, vp, vp, i64, i32, vp]
     lib.floor_ln_traffic.argtypes = [vp, vp, i64, i32, vp]
-    lib.floor_stream_resident.argtypes = [vp, vp, i32, i64, i32, i32, vp]
+    lib.floor_stream_resident.argtypes = [vp, vp, i32, i64, i32, i32, i32, i32, vp]
     lib.floor_stream.argtypes = [vp, i32, vp, i32, i64, i32, vp, vp]
     lib.floor_valu_rate.argtypes = [i32, i32, i32, vp, vp]
     lib.floor_node.argtypes = [vp, vp, i32, i32, i32, vp]
@@ -986,17 +986,25 @@ def placement_sweep(ops, dev, steps):
 
             # the scattered stream by resident workgroups of 1024 lanes (the best of four shapes): what the pattern
             # costs when nothing but bandwidth shapes the kernel
-            def resident_GBps(ndst):
+            def resident_GBps(ndst, slices=((0, 0),), shapes=((4, 256), (4, 768), (8, 256), (8, 512))):
                 best = 0
-                for loads, groups in ((4, 256), (4, 768), (8, 256), (8, 512)):
-                    f = lambda: floor.floor_stream_resident(chunks[reps[0]].data_ptr(), high, ndst, 3 << 30, loads, groups, stream)
-                    for _ in range(2):
-                        assert f() == 0
-                    best = max(best, round((3 << 30) * 1.5 / statistics.median(event_times_us(f, steps)) / 1e3))
+                for loads, groups in shapes:
+                    for period_us, read_share in slices:
+                        # a period in which every workgroup moves one piece at `period_us`'s assumed rate (bytes / us)
+                        period = int(groups * loads * 16384 * 1.5 / period_us * 100) if period_us else 0
+                        f = lambda: floor.floor_stream_resident(chunks[reps[0]].data_ptr(), high, ndst, 3 << 30, loads, groups,
+                                                                period, int(period * read_share), stream)
+                        for _ in range(2):
+                            assert f() == 0
+                        best = max(best, round((3 << 30) * 1.5 / statistics.median(event_times_us(f, max(5, steps // 10))) / 1e3))
                 return best
 
             out["bare_stream_GBps"]["scattered 2:1 stream by resident workgroups (1024 lanes, 4 or 8 loads per lane in flight)"] = {
                 f"stores_to_{n}_regions": resident_GBps(n) for n in (1, 2, 3)}
+            # ... with reads and writes in turns: periods sized for 5.0 to 6.5 TB/s, 50 to 70 % of a period for the loads
+            slices = [(rate, share) for rate in (5.0e6, 5.5e6, 6.0e6, 6.5e6) for share in (0.5, 0.6, 0.7)]
+            out["bare_stream_GBps"]["the same with all loads in one window of the shared clock and all stores in the other (best of 12 schedules)"] = {
+                "stores_to_1_regions": resident_GBps(1, slices, ((8, 256), (4, 512)))}
     return out
 
 

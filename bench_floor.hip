@@ -92,15 +92,24 @@ __global__ void stream_kernel(Three src, int nsrc, Three dst, int ndst, int64_t 
 
 // The 2:1 stream with scattered 1 KiB rows (mode 3 of stream_kernel) by resident workgroups: a piece is kLoads x 16 KiB,
 // every lane requests its kLoads chunks of it at once, then stores the halves; the rows are dealt over `ndst` buffers.
+// period > 0: time slices.  Every workgroup requests its loads only while the shared 100 MHz clock, modulo `period`
+// ticks, is below `read_ticks`, and stores only in the rest of the period, so that the memory system sees reads and
+// writes in turns instead of mixed.  (Both waits end by themselves: the clock runs on.)
 template <int kLoads>
 __global__ __launch_bounds__(1024) void resident_stream_kernel(const char *src, Three dst, int ndst, int64_t pieces,
-                                                                int scatter_bits) {
+                                                                int scatter_bits, int period, int read_ticks) {
   const unsigned rows_per_piece = kLoads * 8;
   for (int64_t k = blockIdx.x; k < pieces; k += gridDim.x) {
+    if (period > 0)
+      while ((int)(wall_clock64() % (unsigned long long)period) >= read_ticks) __builtin_amdgcn_s_sleep(4);
     const u32x4 *from = (const u32x4 *)(src + k * (int64_t)kLoads * 16384);
     u32x4 v[kLoads];
 #pragma unroll
     for (int u = 0; u < kLoads; ++u) v[u] = __builtin_nontemporal_load(from + u * 1024 + threadIdx.x);
+    if (period > 0) {
+      if (v[kLoads - 1].x == 0x9e3779b9u && v[0].y == 0x12345u) __builtin_amdgcn_s_sleep(1);   // the data has arrived
+      while ((int)(wall_clock64() % (unsigned long long)period) < read_ticks) __builtin_amdgcn_s_sleep(4);
+    }
 #pragma unroll
     for (int u = 0; u < kLoads; ++u) {
       const u32x2 w = {v[u].x ^ v[u].z, v[u].y ^ v[u].w};
@@ -112,21 +121,25 @@ __global__ __launch_bounds__(1024) void resident_stream_kernel(const char *src, 
   }
 }
 
-// bytes_in of `src` (a multiple of loads x 16 KiB, at most 2^41) are read, half as many written, dealt over dst[0..ndst)
+// bytes_in of `src` (a multiple of loads x 16 KiB, at most 2^41) are read, half as many written, dealt over dst[0..ndst);
+// period_ticks = 0: no time slices, else 0 < read_ticks < period_ticks (ticks of 10 ns)
 extern "C" int floor_stream_resident(const void *src, void *const *dst, int ndst, int64_t bytes_in, int loads,
-                                     int workgroups, void *stream) {
+                                     int workgroups, int period_ticks, int read_ticks, void *stream) {
   if (!src || !dst || ndst < 1 || ndst > 3 || (loads != 4 && loads != 8) || workgroups < 1 || workgroups > 65535 ||
       bytes_in <= 0 || bytes_in % ((int64_t)loads * 16384) || bytes_in > ((int64_t)1 << 41))
     return 1;
+  if (period_ticks < 0 || (period_ticks > 0 && (read_ticks <= 0 || read_ticks >= period_ticks))) return 1;
   Three d = {};
   for (int i = 0; i < ndst; ++i) d.p[i] = (char *)dst[i];
   const int64_t pieces = bytes_in / ((int64_t)loads * 16384);
   const int scatter_bits = __builtin_ctzll((unsigned long long)(pieces * loads * 8));
   hipStream_t s = (hipStream_t)stream;
   if (loads == 4)
-    hipLaunchKernelGGL(resident_stream_kernel<4>, dim3(workgroups), dim3(1024), 0, s, (const char *)src, d, ndst, pieces, scatter_bits);
+    hipLaunchKernelGGL(resident_stream_kernel<4>, dim3(workgroups), dim3(1024), 0, s, (const char *)src, d, ndst, pieces, scatter_bits,
+                       period_ticks, read_ticks);
   else
-    hipLaunchKernelGGL(resident_stream_kernel<8>, dim3(workgroups), dim3(1024), 0, s, (const char *)src, d, ndst, pieces, scatter_bits);
+    hipLaunchKernelGGL(resident_stream_kernel<8>, dim3(workgroups), dim3(1024), 0, s, (const char *)src, d, ndst, pieces, scatter_bits,
+                       period_ticks, read_ticks);
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 

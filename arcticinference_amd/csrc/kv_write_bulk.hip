@@ -382,6 +382,131 @@ __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
   bulk_item<Src, Dst, kPow2, kBulkThreads, kUnroll, kSelect>(p, tab, blockIdx.x);
 }
 
+#ifdef ARCTIC_TUNING
+// Measurement build only (ARCTIC_BULK_RESIDENT): measured slower than one workgroup per token and layer group.
+// The same write by resident workgroups, for launches of thousands of tokens whose per-workgroup share is a
+// whole number of batches.  The grid is a few workgroups per CU (a multiple of groups_per_token, so that a
+// workgroup keeps its layer group); each walks over every (gridDim.x / groups_per_token)-th token.  What depends
+// on the layers alone - cache pointer and reciprocal scale of each row - is put into LDS once, and so are the slots
+// of the workgroup's tokens; what depends on the token is then one number, the byte offset of its slot's row inside
+// a cache, which is uniform and lives in scalar registers.  So there is nothing to rebuild and no barrier between
+// tokens, and the stream of batches runs across token boundaries.  Every batch is straight-line code - kUnroll
+// loads of the next batch, kUnroll conversions and stores of the current one, no lane left out - so that the compiler
+// knows exactly how many requests are outstanding and waits for the oldest only: loads and stores of a workgroup
+// overlap.  Tokens without a slot are skipped while walking the slot list and cost no source traffic.
+constexpr int kResidentMaxTokens = 1024;   // tokens per workgroup whose slots fit the LDS list
+
+__device__ __forceinline__ int64_t uniform64(int64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+template <typename Src, typename Dst, int kBulkThreads, int kUnroll>
+__global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_resident_kernel(const BulkParams p, const LayerTables tab) {
+  constexpr bool kCopy = std::is_same<Dst, Copy>::value;
+  constexpr int kDstElemBytes = kCopy ? Src::kBytes : 1;
+  constexpr int kBatch = kBulkThreads * kUnroll;
+  __shared__ RowDesc rows[2 * kLayersPerLaunch];
+  __shared__ int64_t slots[kResidentMaxTokens];   // of this workgroup's tokens; -1: no row to write
+
+  const int group = blockIdx.x % (unsigned)p.groups_per_token;
+  const int step = gridDim.x / (unsigned)p.groups_per_token;
+  const int layer0 = group * p.layers_per_group;
+  const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
+  const int cpr = p.chunks_per_row;
+  const int total = 2 * nlayers * cpr;   // chunks of one token that this workgroup moves: a multiple of kBatch
+  const int64_t column0 = (int64_t)layer0 * p.n * Src::kBytes;
+  const int64_t token0 = blockIdx.x / (unsigned)p.groups_per_token;
+  const int ntok = (int)((p.num_tokens - token0 + step - 1) / step);   // <= kResidentMaxTokens (the host sees to it)
+
+  for (int r = threadIdx.x; r < 2 * nlayers; r += kBulkThreads) {
+    const int layer = layer0 + (r >> 1);
+    const bool is_v = r & 1;
+    RowDesc d;
+    d.dst = (char *)(is_v ? tab.value_cache[layer] : tab.key_cache[layer]);
+    d.inv = 0.0;
+    if constexpr (!kCopy) d.inv = 1.0 / (double)(*(is_v ? tab.v_scale[layer] : tab.k_scale[layer]));
+    rows[r] = d;
+  }
+  for (int k = threadIdx.x; k < ntok; k += kBulkThreads) {
+    const int64_t slot = p.slot_mapping[token0 + (int64_t)k * step];
+    slots[k] = (slot >= 0 && slot < p.num_slots) ? slot : -1;
+  }
+  __syncthreads();
+
+  auto next_with_row = [&](int k, int64_t &slot) {   // uniform: every lane reads the same LDS words
+    slot = -1;
+    while (k < ntok && (slot = uniform64(slots[k])) < 0) ++k;
+    return k;
+  };
+  auto row_offset = [&](int64_t slot) -> int64_t {   // bytes from a cache's base to the slot's row
+    int64_t blk, off;
+    if (slot < 0x7fffffffLL) {
+      const uint32_t s32 = (uint32_t)slot, bs = (uint32_t)p.block_size;
+      blk = s32 / bs;
+      off = s32 - (uint32_t)blk * bs;
+    } else {
+      blk = slot / p.block_size;
+      off = slot - blk * p.block_size;
+    }
+    return (blk * p.block_stride + off * (int64_t)p.n) * kDstElemBytes;
+  };
+  auto load_batch = [&](int64_t token, int first, uint4 (&v)[kUnroll]) {
+    const char *ksrc = p.keys + token * p.key_stride_bytes + column0;
+    const char *vsrc = p.values + token * p.value_stride_bytes + column0;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int c = first + (int)threadIdx.x + u * kBulkThreads;
+      const int r = c >> p.chunk_shift, col = c & (cpr - 1);
+      v[u] = load16_stream(((r & 1) ? vsrc : ksrc) + ((int64_t)(r >> 1) * cpr + col) * 16);
+    }
+  };
+
+  int64_t slot;
+  int k = next_with_row(0, slot);
+  if (k >= ntok) return;
+  int64_t token = token0 + (int64_t)k * step;
+  int64_t offset = row_offset(slot);
+  int first = 0;
+  // One batch: request the batch behind it into `nxt`, convert and store `cur`.  Called with the two register sets
+  // in turn, so that no batch is ever copied from one set to the other (a copy would wait for its loads).
+  auto batch = [&](uint4 (&cur)[kUnroll], uint4 (&nxt)[kUnroll]) -> bool {
+    // where the batch behind this one lies: further on in the token, or at the start of the next token with a row
+    int nfirst = first + kBatch;
+    int64_t ntoken = token, noffset = offset;
+    bool last = false;
+    if (nfirst >= total) {
+      nfirst = 0;
+      k = next_with_row(k + 1, slot);
+      if (k < ntok) {
+        ntoken = token0 + (int64_t)k * step;
+        noffset = row_offset(slot);
+      } else {
+        last = true;   // nothing behind it: the loads below fetch this token's first batch again and are dropped
+      }
+    }
+    load_batch(ntoken, nfirst, nxt);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int c = first + (int)threadIdx.x + u * kBulkThreads;
+      const int r = c >> p.chunk_shift, col = c & (cpr - 1);
+      RowDesc d = rows[r];
+      d.dst += offset;
+      emit_chunk<Src, Dst>(cur[u], d, col);
+    }
+    token = ntoken;
+    offset = noffset;
+    first = nfirst;
+    return !last;
+  };
+  uint4 even[kUnroll], odd[kUnroll];
+  load_batch(token, first, even);
+  while (batch(even, odd) && batch(odd, even)) {
+  }
+}
+#endif  // ARCTIC_TUNING
+
 // Fallback for shapes or addresses that do not allow 16-byte accesses: one
 // element per lane per step, any alignment.  Same arithmetic, no vector access.
 template <typename SrcElem, typename Dst>
@@ -489,7 +614,29 @@ template <typename Src, typename Dst, int kSelect>
 static void launch_vec_shape(const BulkParams &p, const LayerTables &tab, int64_t grid, bool wide, hipStream_t s) {
   const dim3 g((unsigned)grid);
 #ifdef ARCTIC_TUNING
-  // measurement build: ARCTIC_BULK_SHAPE = 1: 512 lanes x 4 chunks, 2: 1024 x 2, 3: 1024 x 4, 4: 1024 x 1
+  // measurement build: ARCTIC_BULK_RESIDENT = workgroups per CU of the resident kernel (x 10 + 1: four chunks per lane)
+  if constexpr (kSelect == kSelectNone) {
+    const char *e = getenv("ARCTIC_BULK_RESIDENT");
+    const int v = e ? atoi(e) : 0;
+    if (v && p.chunk_shift >= 0) {
+      const int per_cu = v >= 10 ? v / 10 : v;
+      unsigned wg = (unsigned)std::min<int64_t>(grid, 256LL * per_cu);
+      wg -= wg % (unsigned)p.groups_per_token;
+      const bool four = v >= 10 && v % 10 == 1;
+      const int64_t per_wg = 2LL * p.layers_per_group * p.chunks_per_row;   // chunks of a token per workgroup
+      const bool fits = wg >= (unsigned)p.groups_per_token && p.num_layers % p.layers_per_group == 0 &&
+                        per_wg % (512 * (four ? 4 : 2)) == 0 &&
+                        (p.num_tokens + wg / p.groups_per_token - 1) / (wg / p.groups_per_token) <= kResidentMaxTokens;
+      if (fits) {
+        if (four)
+          hipLaunchKernelGGL((kv_write_bulk_resident_kernel<Src, Dst, 512, 4>), dim3(wg), dim3(512), 0, s, p, tab);
+        else
+          hipLaunchKernelGGL((kv_write_bulk_resident_kernel<Src, Dst, 512, 2>), dim3(wg), dim3(512), 0, s, p, tab);
+        return;
+      }
+    }
+  }
+  // ARCTIC_BULK_SHAPE = 1: 512 lanes x 4 chunks, 2: 1024 x 2, 3: 1024 x 4, 4: 1024 x 1
   if constexpr (kSelect == kSelectNone) {
     const char *e = getenv("ARCTIC_BULK_SHAPE");
     const int shape = e ? atoi(e) : 0;

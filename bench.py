@@ -1054,8 +1054,9 @@ def bench_valu_rates(dev, steps):
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     iters = 4096
     names = {0: "v_mul_f32", 1: "v_fma_f32", 2: "v_rcp_f32", 3: "v_exp_f32",
-             4: "v_rcp_f32 + 3 dependent full-rate operations (per instruction)", 5: "v_lshlrev_b32"}
-    per_round = {0: 1, 1: 1, 2: 1, 3: 1, 4: 4, 5: 1}
+             4: "v_rcp_f32 + 3 dependent full-rate operations (per instruction)", 5: "v_lshlrev_b32",
+             6: "v_cvt_f64_f32 . v_mul_f64 . v_cvt_f32_f64 (per instruction)", 7: "v_med3_f32"}
+    per_round = {0: 1, 1: 1, 2: 1, 3: 1, 4: 4, 5: 1, 6: 3, 7: 1}
     out = {"compute_units": cus}
     for op, name in names.items():
         row = {}
@@ -1119,6 +1120,10 @@ def bench_bulk_variants(dev, steps):
              ("1024 lanes x 2 chunks", {"ARCTIC_BULK_SHAPE": "2"}),
              ("1024 lanes x 2 chunks, one group of 40 layers", {"ARCTIC_BULK_SHAPE": "2", "ARCTIC_BULK_GROUPS": "1"}),
              ("1024 lanes x 4 chunks, one group of 40 layers", {"ARCTIC_BULK_SHAPE": "3", "ARCTIC_BULK_GROUPS": "1"}),
+             ("resident workgroups that stream across tokens (slots and row descriptors in LDS, straight-line batches), 2 per CU",
+              {"ARCTIC_BULK_RESIDENT": "2"}),
+             ("resident workgroups that stream across tokens, 3 per CU", {"ARCTIC_BULK_RESIDENT": "3"}),
+             ("resident workgroups that stream across tokens, 4 per CU", {"ARCTIC_BULK_RESIDENT": "4"}),
              ("as shipped, 768 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "768"}),
              ("as shipped, 1024 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "1024"}),
              ("as shipped, 2048 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "2048"}),
@@ -1132,7 +1137,7 @@ def bench_bulk_variants(dev, steps):
     written, same = {}, {}
     for _ in range(3):
         for name, env in cases:
-            for k in ("ARCTIC_BULK_STORES_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT"):
+            for k in ("ARCTIC_BULK_STORES_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT", "ARCTIC_BULK_RESIDENT"):
                 os.environ.pop(k, None)
             os.environ.update(env)
             # what the variant writes into the first and the last layer's caches, against the first variant's
@@ -1145,7 +1150,7 @@ def bench_bulk_variants(dev, steps):
             written.setdefault("first", sums)
             same[name] = same.get(name, True) and sums == written["first"]
             out[name].append(round(statistics.mean(event_times_us(launch, max(10, steps // 4))), 1))
-    for k in ("ARCTIC_BULK_STORES_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT"):
+    for k in ("ARCTIC_BULK_STORES_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT", "ARCTIC_BULK_RESIDENT"):
         os.environ.pop(k, None)
     return {name: {"kernel_us_rounds": v, "GBps": round(w.bytes / statistics.mean(v) / 1e3),
                    "hbm_frac": round(w.bytes / statistics.mean(v) / 1e3 / HBM_PEAK_GBS, 4),

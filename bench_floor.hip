@@ -145,7 +145,8 @@ extern "C" int floor_stream_resident(const void *src, void *const *dst, int ndst
 
 // Issue rates of the vector ALU: every lane runs `iters` rounds of eight independent chains of one operation
 // (0 multiply, 1 fused multiply-add, 2 reciprocal, 3 exp2, 4 one reciprocal followed by three dependent full-rate
-// operations, 5 16-bit unpack by shift).  The host times it with 1, 2 and 4 waves per SIMD.
+// operations, 5 16-bit unpack by shift, 6 v_cvt_f64_f32 . v_mul_f64 . v_cvt_f32_f64, 7 v_med3_f32).  The host times
+// it with 1, 2 and 4 waves per SIMD.
 template <int OP>
 __global__ __launch_bounds__(256) void valu_rate_kernel(float *out, int iters, float seed) {
   float a[8];
@@ -165,6 +166,9 @@ __global__ __launch_bounds__(256) void valu_rate_kernel(float *out, int iters, f
         a[j] = a[j] * a[j];
       }
       if (OP == 5) a[j] = __uint_as_float(__float_as_uint(a[j]) << 1);
+      // the bulk write's exact division by the scale: widen, multiply in fp64, narrow (3 instructions per round)
+      if (OP == 6) a[j] = (float)((double)a[j] * 1.0000001);
+      if (OP == 7) a[j] = __builtin_amdgcn_fmed3f(a[j], -448.0f, 448.0f);
     }
   }
   float s = 0;
@@ -185,6 +189,8 @@ extern "C" int floor_valu_rate(int op, int blocks, int iters, void *out, void *s
     case 3: hipLaunchKernelGGL(valu_rate_kernel<3>, g, b, 0, s, (float *)out, iters, 1.5f); break;
     case 4: hipLaunchKernelGGL(valu_rate_kernel<4>, g, b, 0, s, (float *)out, iters, 1.5f); break;
     case 5: hipLaunchKernelGGL(valu_rate_kernel<5>, g, b, 0, s, (float *)out, iters, 1.5f); break;
+    case 6: hipLaunchKernelGGL(valu_rate_kernel<6>, g, b, 0, s, (float *)out, iters, 1.5f); break;
+    case 7: hipLaunchKernelGGL(valu_rate_kernel<7>, g, b, 0, s, (float *)out, iters, 1.5f); break;
     default: return 1;
   }
   return hipGetLastError() == hipSuccess ? 0 : 3;

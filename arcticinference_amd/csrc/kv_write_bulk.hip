@@ -79,7 +79,7 @@ struct BulkParams {
   int index_is_64;
   int select_mode;   // kSelectNone / kSelectByRowMap / kSelectByScan (the vector kernels take it as a template argument)
 #ifdef ARCTIC_TUNING
-  int stores_before_loads;  // measurement build: a batch is converted and stored before the next one is requested
+  int loads_before_stores;  // measurement build: the next batch is requested before this one is converted and stored
   unsigned items;           // measurement build: not 0 = workgroups loop over this many items (ARCTIC_BULK_PERSISTENT)
 #endif
 };
@@ -329,15 +329,18 @@ __device__ __forceinline__ void bulk_item(const BulkParams &p, const LayerTables
     vout = p.values_out + (int64_t)layer0 * p.n * Src::kBytes;
   }
 
-  // software-pipelined main loop: the next batch is in flight while this one
-  // is converted and stored
+  // Main loop: a batch is converted and stored, then the next one is requested.  (Requesting the next batch first,
+  // so that it is in flight during the conversion, measures the same within half a per cent at every size and
+  // placement: the other workgroups of the CU cover a workgroup's wait either way.)
+#ifdef ARCTIC_TUNING
+  const bool loads_first = p.loads_before_stores;
+#else
+  constexpr bool loads_first = false;
+#endif
   while (c < total) {
     const int cn = c + kUnroll * kBulkThreads;
     uint4 nxt[kUnroll];
-#ifdef ARCTIC_TUNING
-    if (!p.stores_before_loads)
-#endif
-    load_batch(cn, nxt);
+    if (loads_first) load_batch(cn, nxt);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int cu = c + u * kBulkThreads;
@@ -358,9 +361,7 @@ __device__ __forceinline__ void bulk_item(const BulkParams &p, const LayerTables
         }
       }
     }
-#ifdef ARCTIC_TUNING
-    if (p.stores_before_loads) load_batch(cn, nxt);
-#endif
+    if (!loads_first) load_batch(cn, nxt);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) cur[u] = nxt[u];
     c = cn;
@@ -845,23 +846,32 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
     p.chunk_shift = -1;
     if (vec && (p.chunks_per_row & (p.chunks_per_row - 1)) == 0) p.chunk_shift = __builtin_ctz(p.chunks_per_row);
 
-    // A token's layers are split over `groups` workgroups.  Measured best on gfx950: the 512-lane shape
-    // with 2-5 batches of 1024 chunks per workgroup (20 layers of 8 x 128 bf16 at most) and at least
-    // about 1024 workgroups; when so few tokens come that a workgroup would get less than two batches
-    // (decode), the 256-lane shape with about 2048 workgroups of at least one batch each.
+    // A token's layers are split over `groups` workgroups.  Measured best on gfx950 (sweeps over the group count and
+    // both shapes at 64 to 16384 tokens, 16 and 40 layers):
+    //  - above 8192 tokens, the 512-lane shape with up to five batches of 1024 chunks per workgroup (20 layers of
+    //    8 x 128 bf16) and at least about 1024 workgroups; a workgroup that would get less than two batches takes
+    //    the 256-lane shape instead;
+    //  - below that, the 256-lane shape with about two batches of 1024 chunks per workgroup (8 such layers), more
+    //    and smaller workgroups when fewer than about 1280 would exist otherwise, but never less than one batch each.
     int groups = 1;
     bool wide = false;
     if (vec) {
       const int64_t chunks_per_layer = 2LL * p.chunks_per_row;
-      int64_t g = std::max<int64_t>((1024 + num_tokens - 1) / num_tokens, (chunks_per_layer * count + 5119) / 5120);
-      g = std::max<int64_t>(1, std::min<int64_t>(g, count));
-      const int64_t layers_per_group = (count + g - 1) / g;
-      if (layers_per_group * chunks_per_layer >= 2048) {
-        wide = true;
-        groups = (int)g;
+      const int min_layers = (int)std::max<int64_t>(1, (1024 + chunks_per_layer - 1) / chunks_per_layer);
+      if (num_tokens > 8192) {
+        int64_t g = std::max<int64_t>((1024 + num_tokens - 1) / num_tokens, (chunks_per_layer * count + 5119) / 5120);
+        g = std::max<int64_t>(1, std::min<int64_t>(g, count));
+        const int64_t layers_per_group = (count + g - 1) / g;
+        if (layers_per_group * chunks_per_layer >= 2048) {
+          wide = true;
+          groups = (int)g;
+        } else {
+          const int64_t want = (2048 + num_tokens - 1) / num_tokens;
+          groups = (int)std::max<int64_t>(1, std::min<int64_t>(want, count / min_layers));
+        }
       } else {
-        const int min_layers = (int)std::max<int64_t>(1, (1024 + chunks_per_layer - 1) / chunks_per_layer);
-        const int64_t want = (2048 + num_tokens - 1) / num_tokens;
+        const int64_t two_batches = std::max<int64_t>(1, (2048 + chunks_per_layer - 1) / chunks_per_layer);   // layers
+        const int64_t want = std::max<int64_t>((count + two_batches - 1) / two_batches, (1280 + num_tokens - 1) / num_tokens);
         groups = (int)std::max<int64_t>(1, std::min<int64_t>(want, count / min_layers));
       }
     } else {
@@ -870,8 +880,8 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
 #ifdef ARCTIC_TUNING
     if (const char *e = getenv("ARCTIC_BULK_GROUPS")) groups = std::max(1, std::min(count, atoi(e)));
     if (const char *e = getenv("ARCTIC_BULK_WIDE")) wide = atoi(e) != 0;
-    p.stores_before_loads = 0;
-    if (const char *e = getenv("ARCTIC_BULK_STORES_FIRST")) p.stores_before_loads = atoi(e) != 0;
+    p.loads_before_stores = 0;
+    if (const char *e = getenv("ARCTIC_BULK_LOADS_FIRST")) p.loads_before_stores = atoi(e) != 0;
     p.items = 0;
 #endif
     p.layers_per_group = (count + groups - 1) / groups;

@@ -1108,8 +1108,8 @@ def bench_bulk_variants(dev, steps):
             w.slots.data_ptr(), w.T, w.L, w.H, w.D, w.bs, w.key_caches[0].stride(0), w.NB, 2, 1, stream)
         assert rc == 0
 
-    cases = [("as shipped (512 lanes x 2 chunks, 2 groups of 20 layers, next loads before this batch's stores)", {}),
-             ("this batch's stores before the next batch's loads", {"ARCTIC_BULK_STORES_FIRST": "1"}),
+    cases = [("as shipped (512 lanes x 2 chunks, 2 groups of 20 layers, a batch's stores before the next batch's loads)", {}),
+             ("the next batch's loads before this batch's stores", {"ARCTIC_BULK_LOADS_FIRST": "1"}),
              ("256 lanes x 4 chunks", {"ARCTIC_BULK_WIDE": "0"}),
              ("one group of 40 layers per token", {"ARCTIC_BULK_GROUPS": "1"}),
              ("4 groups of 10 layers per token", {"ARCTIC_BULK_GROUPS": "4"}),
@@ -1137,7 +1137,7 @@ def bench_bulk_variants(dev, steps):
     written, same = {}, {}
     for _ in range(3):
         for name, env in cases:
-            for k in ("ARCTIC_BULK_STORES_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT", "ARCTIC_BULK_RESIDENT"):
+            for k in ("ARCTIC_BULK_LOADS_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT", "ARCTIC_BULK_RESIDENT"):
                 os.environ.pop(k, None)
             os.environ.update(env)
             # what the variant writes into the first and the last layer's caches, against the first variant's
@@ -1150,7 +1150,7 @@ def bench_bulk_variants(dev, steps):
             written.setdefault("first", sums)
             same[name] = same.get(name, True) and sums == written["first"]
             out[name].append(round(statistics.mean(event_times_us(launch, max(10, steps // 4))), 1))
-    for k in ("ARCTIC_BULK_STORES_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT", "ARCTIC_BULK_RESIDENT"):
+    for k in ("ARCTIC_BULK_LOADS_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT", "ARCTIC_BULK_RESIDENT"):
         os.environ.pop(k, None)
     return {name: {"kernel_us_rounds": v, "GBps": round(w.bytes / statistics.mean(v) / 1e3),
                    "hbm_frac": round(w.bytes / statistics.mean(v) / 1e3 / HBM_PEAK_GBS, 4),

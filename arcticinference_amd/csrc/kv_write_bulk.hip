@@ -201,7 +201,7 @@ __device__ __forceinline__ void select_leftover_rows(const BulkParams &p, unsign
 // kBulkThreads x kUnroll 16-byte chunks form one batch of a workgroup.  Two shapes
 // are built: 512 x 2 (a workgroup moves two batches or more) and 256 x 4 (decode:
 // few tokens, a single batch per workgroup).
-template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll, int kSelect>
+template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll, int kSelect, bool kLoadsFirst = false>
 __device__ __forceinline__ void bulk_item(const BulkParams &p, const LayerTables &tab, unsigned block) {
   constexpr bool kCopy = std::is_same<Dst, Copy>::value;
   constexpr int kDstElemBytes = kCopy ? Src::kBytes : 1;
@@ -332,15 +332,10 @@ __device__ __forceinline__ void bulk_item(const BulkParams &p, const LayerTables
   // Main loop: a batch is converted and stored, then the next one is requested.  (Requesting the next batch first,
   // so that it is in flight during the conversion, measures the same within half a per cent at every size and
   // placement: the other workgroups of the CU cover a workgroup's wait either way.)
-#ifdef ARCTIC_TUNING
-  const bool loads_first = p.loads_before_stores;
-#else
-  constexpr bool loads_first = false;
-#endif
   while (c < total) {
     const int cn = c + kUnroll * kBulkThreads;
     uint4 nxt[kUnroll];
-    if (loads_first) load_batch(cn, nxt);
+    if constexpr (kLoadsFirst) load_batch(cn, nxt);   // (an instantiation of the measurement build only)
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int cu = c + u * kBulkThreads;
@@ -361,27 +356,30 @@ __device__ __forceinline__ void bulk_item(const BulkParams &p, const LayerTables
         }
       }
     }
-    if (!loads_first) load_batch(cn, nxt);
+    if constexpr (!kLoadsFirst) load_batch(cn, nxt);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) cur[u] = nxt[u];
     c = cn;
   }
 }
 
-template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll, int kSelect>
+template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll, int kSelect, bool kLoadsFirst = false>
 __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
     const BulkParams p, const LayerTables tab) {
-#ifdef ARCTIC_TUNING
-  if (p.items) {   // measurement build: a grid of fewer workgroups, each taking every gridDim.x-th item in turn
-    for (unsigned item = blockIdx.x; item < p.items; item += gridDim.x) {
-      bulk_item<Src, Dst, kPow2, kBulkThreads, kUnroll, kSelect>(p, tab, item);
-      __syncthreads();   // the next item rewrites the row descriptors
-    }
-    return;
-  }
-#endif
-  bulk_item<Src, Dst, kPow2, kBulkThreads, kUnroll, kSelect>(p, tab, blockIdx.x);
+  bulk_item<Src, Dst, kPow2, kBulkThreads, kUnroll, kSelect, kLoadsFirst>(p, tab, blockIdx.x);
 }
+
+#ifdef ARCTIC_TUNING
+// Measurement build only (ARCTIC_BULK_PERSISTENT): a grid of fewer workgroups, each taking every gridDim.x-th item
+// in turn.  A kernel of its own, so that the kernel above is compiled exactly as in the library.
+template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll>
+__global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_looping_kernel(const BulkParams p, const LayerTables tab) {
+  for (unsigned item = blockIdx.x; item < p.items; item += gridDim.x) {
+    bulk_item<Src, Dst, kPow2, kBulkThreads, kUnroll, kSelectNone>(p, tab, item);
+    __syncthreads();   // the next item rewrites the row descriptors
+  }
+}
+#endif
 
 #ifdef ARCTIC_TUNING
 // Measurement build only (ARCTIC_BULK_RESIDENT): measured slower than one workgroup per token and layer group.
@@ -637,6 +635,20 @@ static void launch_vec_shape(const BulkParams &p, const LayerTables &tab, int64_
       }
     }
   }
+  // ARCTIC_BULK_PERSISTENT: p.items is set and the grid cut down; ARCTIC_BULK_LOADS_FIRST: the other order in the loop
+  if constexpr (kSelect == kSelectNone) {
+    if (p.chunk_shift >= 0 && (p.items || p.loads_before_stores)) {
+      if (p.items && wide)
+        hipLaunchKernelGGL((kv_write_bulk_looping_kernel<Src, Dst, true, 512, 2>), g, dim3(512), 0, s, p, tab);
+      else if (p.items)
+        hipLaunchKernelGGL((kv_write_bulk_looping_kernel<Src, Dst, true, 256, 4>), g, dim3(256), 0, s, p, tab);
+      else if (wide)
+        hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 512, 2, kSelectNone, true>), g, dim3(512), 0, s, p, tab);
+      else
+        hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 256, 4, kSelectNone, true>), g, dim3(256), 0, s, p, tab);
+      return;
+    }
+  }
   // ARCTIC_BULK_SHAPE = 1: 512 lanes x 4 chunks, 2: 1024 x 2, 3: 1024 x 4, 4: 1024 x 1
   if constexpr (kSelect == kSelectNone) {
     const char *e = getenv("ARCTIC_BULK_SHAPE");
@@ -852,7 +864,7 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
     //    8 x 128 bf16) and at least about 1024 workgroups; a workgroup that would get less than two batches takes
     //    the 256-lane shape instead;
     //  - below that, the 256-lane shape with about two batches of 1024 chunks per workgroup (8 such layers), more
-    //    and smaller workgroups when fewer than about 1280 would exist otherwise, but never less than one batch each.
+    //    and smaller workgroups when fewer than about 2048 would exist otherwise, but never less than one batch each.
     int groups = 1;
     bool wide = false;
     if (vec) {
@@ -871,7 +883,7 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
         }
       } else {
         const int64_t two_batches = std::max<int64_t>(1, (2048 + chunks_per_layer - 1) / chunks_per_layer);   // layers
-        const int64_t want = std::max<int64_t>((count + two_batches - 1) / two_batches, (1280 + num_tokens - 1) / num_tokens);
+        const int64_t want = std::max<int64_t>((count + two_batches - 1) / two_batches, (2048 + num_tokens - 1) / num_tokens);
         groups = (int)std::max<int64_t>(1, std::min<int64_t>(want, count / min_layers));
       }
     } else {

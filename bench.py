@@ -1126,13 +1126,7 @@ def bench_bulk_variants(dev, steps):
              ("resident workgroups that stream across tokens, 4 per CU", {"ARCTIC_BULK_RESIDENT": "4"}),
              ("as shipped, 768 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "768"}),
              ("as shipped, 1024 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "1024"}),
-             ("as shipped, 2048 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "2048"}),
-             ("1024 lanes x 2 chunks, 256 workgroups that loop", {"ARCTIC_BULK_SHAPE": "2", "ARCTIC_BULK_PERSISTENT": "256"}),
-             ("1024 lanes x 2 chunks, 512 workgroups that loop", {"ARCTIC_BULK_SHAPE": "2", "ARCTIC_BULK_PERSISTENT": "512"}),
-             ("1024 lanes x 4 chunks, one group of 40 layers, 256 workgroups that loop",
-              {"ARCTIC_BULK_SHAPE": "3", "ARCTIC_BULK_GROUPS": "1", "ARCTIC_BULK_PERSISTENT": "256"}),
-             ("1024 lanes x 4 chunks, one group of 40 layers, 512 workgroups that loop",
-              {"ARCTIC_BULK_SHAPE": "3", "ARCTIC_BULK_GROUPS": "1", "ARCTIC_BULK_PERSISTENT": "512"})]
+             ("as shipped, 2048 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "2048"})]
     out = {name: [] for name, _ in cases}
     written, same = {}, {}
     for _ in range(3):

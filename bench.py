@@ -1089,15 +1089,21 @@ def load_tuning_library():
     return lib
 
 
-def bench_bulk_variants(dev, steps):
-    """A/B of launch variants of the bulk write in the compact placement (70B shape, fp8, 40 caches of 8192 blocks and
-    the source allocated first in this process: one HBM region on an idle GPU), through the tuning build: the order of
-    a batch's stores and the next batch's loads, the workgroup shape, and the number of layer groups per token."""
+def bench_bulk_variants(dev, steps, placement="compact"):
+    """A/B of launch variants of the bulk write (70B shape, fp8) through the tuning build: the order of a batch's
+    stores and the next batch's loads, the workgroup shape, and the number of layer groups per token.  `placement`:
+    "compact" = 40 caches of 8192 blocks and the source allocated first in this process (one HBM region on an idle
+    GPU); "serving" = the headline's memory map (66 GiB of weights, an 80-layer pool of 65536 blocks, layers 40-79
+    written), where only the shapes and group counts that are candidates for the launch rule are timed."""
     import ctypes
     tuning = load_tuning_library()
     if tuning is None:
         return "libarctic_tuning_mi355x.so is not built"
-    w = BulkWorkload("70B-SwiftKV-compact", 16384, 40, 8, 128, 16, 8192, "fp8", 0.10, 2, 1.5, dev)
+    if placement == "serving":
+        mem = ServingMemoryMap(dev, 66, 80, 40, 65536, 16, 8, 128, torch.uint8)
+        w = BulkWorkload("70B-SwiftKV", 16384, 40, 8, 128, 16, 65536, "fp8", 0.10, 2, 1.5, dev, bufs=mem.written_layers())
+    else:
+        w = BulkWorkload("70B-SwiftKV-compact", 16384, 40, 8, 128, 16, 8192, "fp8", 0.10, 2, 1.5, dev)
     tab = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
     kc, vc, ks, vs = tab(w.key_caches), tab(w.value_caches), tab(w.k_scales), tab(w.v_scales)
     stream = torch.cuda.current_stream().cuda_stream
@@ -1108,15 +1114,15 @@ def bench_bulk_variants(dev, steps):
             w.slots.data_ptr(), w.T, w.L, w.H, w.D, w.bs, w.key_caches[0].stride(0), w.NB, 2, 1, stream)
         assert rc == 0
 
-    cases = [("as shipped (512 lanes x 2 chunks, 2 groups of 20 layers, a batch's stores before the next batch's loads)", {}),
-             ("the next batch's loads before this batch's stores", {"ARCTIC_BULK_LOADS_FIRST": "1"}),
+    cases = [("as shipped (1024 lanes x 1 chunk, 2 groups of 20 layers, a batch's stores before the next batch's loads)", {}),
+             ("512 lanes x 2 chunks", {"ARCTIC_BULK_SHAPE": "5"}),
+             ("512 lanes x 2 chunks, the next batch's loads before this batch's stores", {"ARCTIC_BULK_LOADS_FIRST": "1"}),
              ("256 lanes x 4 chunks", {"ARCTIC_BULK_WIDE": "0"}),
              ("one group of 40 layers per token", {"ARCTIC_BULK_GROUPS": "1"}),
              ("4 groups of 10 layers per token", {"ARCTIC_BULK_GROUPS": "4"}),
              ("8 groups of 5 layers per token", {"ARCTIC_BULK_GROUPS": "8"}),
              ("512 lanes x 4 chunks", {"ARCTIC_BULK_SHAPE": "1"}),
              ("512 lanes x 4 chunks, one group of 40 layers", {"ARCTIC_BULK_SHAPE": "1", "ARCTIC_BULK_GROUPS": "1"}),
-             ("1024 lanes x 1 chunk", {"ARCTIC_BULK_SHAPE": "4"}),
              ("1024 lanes x 2 chunks", {"ARCTIC_BULK_SHAPE": "2"}),
              ("1024 lanes x 2 chunks, one group of 40 layers", {"ARCTIC_BULK_SHAPE": "2", "ARCTIC_BULK_GROUPS": "1"}),
              ("1024 lanes x 4 chunks, one group of 40 layers", {"ARCTIC_BULK_SHAPE": "3", "ARCTIC_BULK_GROUPS": "1"}),
@@ -1124,9 +1130,13 @@ def bench_bulk_variants(dev, steps):
               {"ARCTIC_BULK_RESIDENT": "2"}),
              ("resident workgroups that stream across tokens, 3 per CU", {"ARCTIC_BULK_RESIDENT": "3"}),
              ("resident workgroups that stream across tokens, 4 per CU", {"ARCTIC_BULK_RESIDENT": "4"}),
-             ("as shipped, 768 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "768"}),
-             ("as shipped, 1024 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "1024"}),
-             ("as shipped, 2048 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "2048"})]
+             ("512 lanes x 2 chunks, 768 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "768"}),
+             ("512 lanes x 2 chunks, 1024 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "1024"}),
+             ("512 lanes x 2 chunks, 2048 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "2048"})]
+    if placement == "serving":
+        cases = [c for c in cases if "loop over" not in c[0] and "resident" not in c[0] and "8 groups" not in c[0]]
+        cases += [("512 lanes x 2 chunks, 4 groups of 10 layers", {"ARCTIC_BULK_SHAPE": "5", "ARCTIC_BULK_GROUPS": "4"}),
+                  ("256 lanes x 4 chunks, 5 groups of 8 layers", {"ARCTIC_BULK_WIDE": "0", "ARCTIC_BULK_GROUPS": "5"})]
     out = {name: [] for name, _ in cases}
     written, same = {}, {}
     for _ in range(3):
@@ -1337,9 +1347,10 @@ def main():
                          "each other and against the traffic-only kernel; prints one JSON object")
     ap.add_argument("--argmax-variants", action="store_true",
                     help="instead of the benchmark, time loop shapes of the row-argmax kernel through the tuning build")
-    ap.add_argument("--bulk-variants", action="store_true",
-                    help="instead of the benchmark, time launch variants of the bulk write in the compact placement "
-                         "through the tuning build; prints one JSON object")
+    ap.add_argument("--bulk-variants", nargs="?", const="compact", default=None, choices=["compact", "serving"],
+                    help="instead of the benchmark, time launch variants of the bulk write through the tuning build, "
+                         "in the compact placement (default) or on the headline's serving memory map; prints one "
+                         "JSON object")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) so that a counter run of this "
                          "command can scale FETCH_SIZE / WRITE_SIZE")
@@ -1367,7 +1378,8 @@ def main():
         print(json.dumps({"row_argmax_variants": bench_argmax_variants(dev, args.steps)}), flush=True)
         return
     if args.bulk_variants:
-        print(json.dumps({"bulk_write_variants_compact_pool": bench_bulk_variants(dev, args.steps)}), flush=True)
+        name = "bulk_write_variants_compact_pool" if args.bulk_variants == "compact" else "bulk_write_variants_serving_map"
+        print(json.dumps({name: bench_bulk_variants(dev, args.steps, args.bulk_variants)}), flush=True)
         return
     if args.only:
         if args.calibrate_copy:

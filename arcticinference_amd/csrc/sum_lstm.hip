@@ -14,6 +14,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 #include "activations.hpp"
 #include "common.hpp"
@@ -42,6 +43,9 @@ struct LstmParams {
   float alpha;
   float eps_cell;
   float eps_state;
+#ifdef ARCTIC_TUNING
+  unsigned long long *trace;   // measurement build: time stamps of sum_lstm_staged_kernel<..., kTrace>, or nullptr
+#endif
 };
 
 // Loads are issued in the order in which the arithmetic needs them - cell gate,
@@ -61,13 +65,15 @@ struct LstmParams {
 // kVariant: bit 0: input gate loaded and consumed before the forget gate and the previous cell; bit 1: the
 // output gate's sigmoid ahead of the second row sum (what the library ships for rows of up to 4096: by then the
 // gate has arrived and the waves would otherwise idle at the barrier); bit 2: one reciprocal shared by the
-// sigmoids and the GELU of a phase.  Built for tuning, every combination can be selected at run time.
+// sigmoids and the GELU of a phase; bit 3: a workgroup barrier (no memory wait) between the groups of requests, so
+// that every wave of the row has requested a gate before any wave requests the next one.  Built for tuning, the
+// combinations that the benchmark times can be selected at run time.
 template <typename C, int K>
 struct LstmRow {
   C sc[K], zc[K], sf[K], zf[K], si[K], zi[K], pc[K], so[K], zo[K];
 };
 
-enum : int { kLstmInputGateFirst = 1, kLstmEarlyOutputGate = 2, kLstmSharedReciprocal = 4 };
+enum : int { kLstmInputGateFirst = 1, kLstmEarlyOutputGate = 2, kLstmSharedReciprocal = 4, kLstmLoadGroupBarriers = 8 };
 
 template <typename T, int E, int kChunksPerThread, bool kFastGelu, int kMaxThreads, bool kSharedZ, bool kAllVectors,
           int kRows, int kVariant, bool kZeroCell = false>
@@ -134,17 +140,26 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
     };
     // the groups must reach memory in this order (it returns loads in issue order); with more than one row per
     // workgroup the compiler would otherwise interleave the rows' loads
-    if constexpr (kRows > 1) __builtin_amdgcn_sched_barrier(0);
+    auto fence = [&]() {
+      if constexpr (kVariant & kLstmLoadGroupBarriers) {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();   // no memory wait: only the order in which the waves issue their requests
+        __builtin_amdgcn_sched_barrier(0);
+      } else if constexpr (kRows > 1) {
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    fence();
     if constexpr (kVariant & kLstmInputGateFirst) {
       input_gate();
-      if constexpr (kRows > 1) __builtin_amdgcn_sched_barrier(0);
+      fence();
       forget_and_cell();
     } else {
       forget_and_cell();
-      if constexpr (kRows > 1) __builtin_amdgcn_sched_barrier(0);
+      fence();
       input_gate();
     }
-    if constexpr (kRows > 1) __builtin_amdgcn_sched_barrier(0);
+    fence();
 #pragma unroll
     for (int k = 0; k < K; ++k) {
       r.so[k] = C::load_stream(s_row + 2 * gate_bytes + off[k]);
@@ -328,6 +343,186 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
     if (r == 0 || row0 + r < p.rows) compute(row0 + r, in[r], slots_cpre[r], slots_cnew[r]);
 }
 
+// The speculator's shape (every lane owns one 16-byte chunk of the row, all four scale / shift vectors given) with the
+// requests of a row issued in stages.  A CU accepts vector-memory requests only as fast as HBM answers them: a wave
+// that asks for its nine chunks at once sits in the ninth request for microseconds, long after the first chunks have
+// arrived and with nothing computed, and the younger workgroup of the CU does not get its first request in before
+// the older one's last (time stamps of the waves: bench.py --lstm-timeline).  Here a wave requests the first kAhead0
+// chunks (order: cell gate z, s; forget gate s, z; previous cell; input gate s, z; output gate s, z), starts on the
+// cell gate as soon as that is in, and requests the rest at four later points of its arithmetic: kAhead1 chunks are
+// out after the first sum of squares, kAhead2 after the candidate's GELU, kAhead3 after the forget gate's part of
+// the cell update, all nine once the new cell is stored.  Waves that are computing leave the request slots to the
+// others, so both rows of a CU arrive gate by gate and every stage's arithmetic runs while the next stage is in flight.
+// kVectors places the requests for the scale / shift vectors (the same for every row, cache resident): 0: all four
+// ahead of the row; 1: the cell norm's pair behind the first sum of squares, the state norm's behind the forget
+// gate's part; 2: the cell norm's pair right behind the first kAhead0 chunks, the state norm's behind the candidate's
+// GELU.  kStreamOutputs / kStreamCell: non-temporal stores of both outputs / load of the previous cell (a step's
+// outputs are read by the next launches of the step, but a launch boundary writes them back anyway, and stores that
+// stream leave earlier).
+template <int kAhead0_, int kAhead1_, int kAhead2_, int kAhead3_, bool kEarlyGate_, int kVectors_, bool kStreamOutputs_,
+          bool kStreamCell_>
+struct LstmSchedule {
+  static constexpr int kAhead0 = kAhead0_, kAhead1 = kAhead1_, kAhead2 = kAhead2_, kAhead3 = kAhead3_;
+  static constexpr bool kEarlyGate = kEarlyGate_, kStreamOutputs = kStreamOutputs_, kStreamCell = kStreamCell_;
+  static constexpr int kVectors = kVectors_;
+  static_assert(kAhead0 >= 2 && kAhead1 >= kAhead0 && kAhead2 >= 5 && kAhead2 >= kAhead1 && kAhead3 >= 7 &&
+                    kAhead3 >= kAhead2 && kAhead3 <= 9,
+                "a chunk must be requested before the arithmetic that reads it");
+};
+// measured best of a sweep over the request points (512 rows of 4096): the cell gate first, the forget gate's s
+// behind the first sum of squares, the rest of the forget gate, the previous cell and the input gate behind the
+// candidate's GELU, the output gate behind the forget gate's part; the output gate is consumed last
+using LstmShippedSchedule = LstmSchedule<2, 3, 7, 7, false, 2, true, true>;
+
+// Same arithmetic, operation for operation, as sum_lstm_vec_kernel: results are bit-identical.
+template <typename T, bool kFastGelu, bool kSharedZ, bool kZeroCell, typename S = LstmShippedSchedule, bool kTrace = false>
+__global__ __launch_bounds__(512) void sum_lstm_staged_kernel(const LstmParams p) {
+  __shared__ float slots_cpre[16];
+  __shared__ float slots_cnew[16];
+  constexpr int E = 8;
+  using C = Chunk<E>;
+  using std::integral_constant;
+  const int64_t row = blockIdx.x;
+  const int64_t off = (int64_t)threadIdx.x * C::kBytes;
+  const int64_t gate_bytes = (int64_t)p.D * 2;
+  // measurement build: the constant-rate clock (100 MHz) at eight points of a wave's life, written by its first lane
+  auto stamp = [&](int k) {
+#ifdef ARCTIC_TUNING
+    if constexpr (kTrace) {
+      __builtin_amdgcn_sched_barrier(0);
+      const unsigned long long t = __builtin_amdgcn_s_memrealtime();
+      if (p.trace && (threadIdx.x & 63) == 0) p.trace[((size_t)blockIdx.x * 8 + threadIdx.x / 64) * 8 + k] = t;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#endif
+  };
+  stamp(0);   // the wave has started
+  C wc, bc, ws, bs;
+  auto request_vectors = [&](int place) {
+    if (place == (S::kVectors == 0 ? 0 : S::kVectors == 1 ? 2 : 1)) {
+      wc = C::load(p.w_cell + off);
+      bc = C::load(p.b_cell + off);
+    }
+    if (place == (S::kVectors == 0 ? 0 : S::kVectors == 1 ? 4 : 3)) {
+      ws = C::load(p.w_state + off);
+      bs = C::load(p.b_state + off);
+    }
+  };
+  request_vectors(0);
+  const char *s_row = p.states + row * p.s_stride * 2 + off;
+  int64_t zr = row;
+  if (kSharedZ && p.z_index) zr = min(max(p.z_index[row], (int64_t)0), p.z_rows - 1);
+  const char *z_row = p.z4 + zr * p.z_stride * 2 + off;
+  const char *pc_row = kZeroCell ? s_row : p.prev_cell + row * p.pc_stride * 2 + off;
+  char *oc_row = p.out_cell + row * p.out_stride * 2 + off;
+  char *os_row = p.out_state + row * p.out_stride * 2 + off;
+
+  C in[9];   // zc sc sf zf pc si zi so zo; with kSharedZ the one z chunk stands for all four, with kZeroCell pc is unused
+  auto request = [&](auto from, auto to) {
+    constexpr int kFrom = decltype(from)::value, kTo = decltype(to)::value;
+    __builtin_amdgcn_sched_barrier(0);   // neither hoisted above the arithmetic in front nor sunk below what follows
+    if constexpr (kFrom <= 0 && 0 < kTo) in[0] = C::load_stream(z_row + (kSharedZ ? 0 : 3 * gate_bytes));
+    if constexpr (kFrom <= 1 && 1 < kTo) in[1] = C::load_stream(s_row + 3 * gate_bytes);
+    if constexpr (kFrom <= 2 && 2 < kTo) in[2] = C::load_stream(s_row);
+    if constexpr (kFrom <= 3 && 3 < kTo && !kSharedZ) in[3] = C::load_stream(z_row);
+    if constexpr (kFrom <= 4 && 4 < kTo && !kZeroCell) in[4] = S::kStreamCell ? C::load_stream(pc_row) : C::load(pc_row);
+    if constexpr (kFrom <= 5 && 5 < kTo) in[5] = C::load_stream(s_row + gate_bytes);
+    if constexpr (kFrom <= 6 && 6 < kTo && !kSharedZ) in[6] = C::load_stream(z_row + gate_bytes);
+    if constexpr (kFrom <= 7 && 7 < kTo) in[7] = C::load_stream(s_row + 2 * gate_bytes);
+    if constexpr (kFrom <= 8 && 8 < kTo && !kSharedZ) in[8] = C::load_stream(z_row + 2 * gate_bytes);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  request(integral_constant<int, 0>(), integral_constant<int, S::kAhead0>());
+  request_vectors(1);
+  stamp(1);   // the first requests are out
+
+  // phase 1: pre_c and its sum of squares (reference :65-82)
+  float cact[E], a[E], b[E], c[E];
+  float ss = 0.f;
+  in[1].template unpack<T>(a);
+  in[0].template unpack<T>(b);
+#pragma unroll
+  for (int j = 0; j < E; ++j) {
+    cact[j] = fmaf(p.alpha, b[j], a[j]);
+    ss = fmaf(cact[j], cact[j], ss);
+  }
+  stamp(2);   // the cell gate is in, its squares are summed
+  request_vectors(2);
+  request(integral_constant<int, S::kAhead0>(), integral_constant<int, S::kAhead1>());
+  const float inv_cpre = rsqrtf(block_sum(ss, slots_cpre) * p.inv_D + p.eps_cell);
+  stamp(3);   // first row sum known
+  {
+    float w[E], sh[E];
+    wc.template unpack<T>(w);
+    bc.template unpack<T>(sh);
+#pragma unroll
+    for (int j = 0; j < E; ++j) cact[j] = gelu<kFastGelu>(fmaf(cact[j] * inv_cpre, w[j], sh[j]));
+  }
+  request_vectors(3);
+  request(integral_constant<int, S::kAhead1>(), integral_constant<int, S::kAhead2>());
+
+  // phase 2: cell update; write out_cell (reference :104-140)
+  float cell[E];
+  in[2].template unpack<T>(a);
+  (kSharedZ ? in[0] : in[3]).template unpack<T>(b);
+  (kZeroCell ? C::zero() : in[4]).template unpack<T>(c);
+#pragma unroll
+  for (int j = 0; j < E; ++j) cell[j] = sigmoid_f(fmaf(p.alpha, b[j], a[j])) * c[j];
+  request_vectors(4);
+  request(integral_constant<int, S::kAhead2>(), integral_constant<int, S::kAhead3>());
+  in[5].template unpack<T>(a);
+  (kSharedZ ? in[0] : in[6]).template unpack<T>(b);
+  ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < E; ++j) {
+    const float cnew = fmaf(cact[j], sigmoid_f(fmaf(p.alpha, b[j], a[j])), cell[j]);
+    ss = fmaf(cnew, cnew, ss);  // unrounded, as in the reference (:136)
+    cell[j] = cnew;
+  }
+  {
+    const C packed = C::template pack<T>(cell);
+    if constexpr (S::kStreamOutputs) packed.store_stream(oc_row);
+    else packed.store(oc_row);
+    packed.template unpack<T>(cell);   // the state phase sees the rounded cell (:163,174)
+  }
+  stamp(4);   // forget gate, previous cell and input gate are in; the new cell is stored
+  request(integral_constant<int, S::kAhead3>(), integral_constant<int, 9>());
+  float og[E];
+  if constexpr (S::kEarlyGate) {
+    in[7].template unpack<T>(a);
+    (kSharedZ ? in[0] : in[8]).template unpack<T>(b);
+#pragma unroll
+    for (int j = 0; j < E; ++j) og[j] = sigmoid_f(fmaf(p.alpha, b[j], a[j]));
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  const float inv_cnew = rsqrtf(block_sum(ss, slots_cnew) * p.inv_D + p.eps_state);
+  stamp(5);   // second row sum known
+
+  // phase 3: state = gelu(rmsnorm(rounded cell)) * sigmoid(pre_o) (reference :160-190)
+  float st[E];
+  {
+    float w[E], sh[E];
+    ws.template unpack<T>(w);
+    bs.template unpack<T>(sh);
+#pragma unroll
+    for (int j = 0; j < E; ++j) st[j] = gelu<kFastGelu>(fmaf(cell[j] * inv_cnew, w[j], sh[j]));
+  }
+  stamp(6);   // state GELU done (with the late output gate: before the output gate is looked at)
+  if constexpr (S::kEarlyGate) {
+#pragma unroll
+    for (int j = 0; j < E; ++j) st[j] *= og[j];
+  } else {
+    __builtin_amdgcn_sched_barrier(0);   // the GELU above runs while the output gate is still on its way
+    in[7].template unpack<T>(a);
+    (kSharedZ ? in[0] : in[8]).template unpack<T>(b);
+#pragma unroll
+    for (int j = 0; j < E; ++j) st[j] *= sigmoid_f(fmaf(p.alpha, b[j], a[j]));
+  }
+  if constexpr (S::kStreamOutputs) C::template pack<T>(st).store_stream(os_row);
+  else C::template pack<T>(st).store(os_row);
+  stamp(7);   // state stored
+}
+
 // Any D, any alignment: element-wise, three passes like the reference's scalar
 // kernel (sum_lstm.cu:193-291).
 template <typename T, bool kFastGelu>
@@ -382,7 +577,8 @@ static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 #ifdef ARCTIC_TUNING
 // Measurement build only: ARCTIC_LSTM_VARIANT = variant bits (see sum_lstm_vec_kernel) + 8 for two rows per workgroup
 // + 16 for two chunks per lane (256 lanes per 4096-wide row), or + 32 for 8-byte chunks (1024 lanes per 4096-wide
-// row).  Read at every call.
+// row); 66 = variant 2 with barriers between the groups of requests.  ARCTIC_LSTM_STAGED selects a schedule of
+// sum_lstm_staged_kernel instead.  Read at every call.
 static int lstm_tuning_variant() {
   const char *e = getenv("ARCTIC_LSTM_VARIANT");
   return e ? atoi(e) : 0;
@@ -419,8 +615,39 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
     const bool all = p.w_cell && p.b_cell && p.w_state && p.b_state && threads * cpt == chunks;
 #ifdef ARCTIC_TUNING
     if (cpt == 1 && all && threads % 128 == 0 && p.prev_cell) {
+      if (const char *st = getenv("ARCTIC_LSTM_STAGED")) {
+        // the staged kernel's schedules that the benchmark times against each other; + 100 for the time stamps
+        LstmParams q = p;
+        const char *e = getenv("ARCTIC_LSTM_TRACE");   // address of rows x 8 waves x 8 words
+        q.trace = e ? (unsigned long long *)strtoull(e, nullptr, 0) : nullptr;
+        const int code = atoi(st);
+#define ARCTIC_STAGED(CODE, ...)                                                                                     \
+  if (code == CODE)                                                                                                  \
+    hipLaunchKernelGGL((sum_lstm_staged_kernel<T, kFastGelu, kSharedZ, false, LstmSchedule<__VA_ARGS__>>), grid,     \
+                       dim3(threads), 0, s, q);                                                                      \
+  if (code == 100 + CODE)                                                                                            \
+    hipLaunchKernelGGL((sum_lstm_staged_kernel<T, kFastGelu, kSharedZ, false, LstmSchedule<__VA_ARGS__>, true>),     \
+                       grid, dim3(threads), 0, s, q);
+        ARCTIC_STAGED(0, 9, 9, 9, 9, true, 0, false, false)    // everything requested at once, as sum_lstm_vec_kernel does
+        ARCTIC_STAGED(1, 2, 3, 7, 7, false, 0, false, false)   // staged requests
+        ARCTIC_STAGED(2, 2, 3, 7, 7, false, 2, false, false)   // + the vectors requested where they are needed
+        ARCTIC_STAGED(3, 2, 3, 7, 7, false, 2, true, false)    // + streaming stores
+        ARCTIC_STAGED(4, 2, 3, 7, 7, false, 2, true, true)     // + streaming load of the previous cell: as shipped
+        ARCTIC_STAGED(5, 2, 3, 7, 7, true, 2, true, true)      // as shipped with the early output gate
+        ARCTIC_STAGED(6, 2, 4, 7, 9, false, 2, true, true)     // other request points
+        ARCTIC_STAGED(7, 3, 4, 7, 7, false, 2, true, true)
+        ARCTIC_STAGED(8, 2, 3, 5, 7, false, 2, true, true)
+        ARCTIC_STAGED(9, 5, 7, 9, 9, false, 2, true, true)
+        ARCTIC_STAGED(10, 9, 9, 9, 9, true, 0, true, true)     // everything at once with the streaming accesses
+#undef ARCTIC_STAGED
+        return;
+      }
       const int v = lstm_tuning_variant();
       const int shape = (v >> 3) & 7;   // 4: 8-byte units, twice the lanes (rows of up to 4096)
+      if (v == 66) {   // variant 2 + a barrier between the groups of requests
+        launch_lstm_tuned<T, kFastGelu, kSharedZ, kLstmEarlyOutputGate | kLstmLoadGroupBarriers>(p, rows, 0, threads, s);
+        return;
+      }
       switch (v & 7) {
         case 0: launch_lstm_tuned<T, kFastGelu, kSharedZ, 0>(p, rows, shape, threads, s); break;
         case 1: launch_lstm_tuned<T, kFastGelu, kSharedZ, 1>(p, rows, shape, threads, s); break;
@@ -433,10 +660,10 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
     }
 #endif
     constexpr int kShipped = kLstmEarlyOutputGate;   // measured best of the variants that change no result bit
-    if (cpt == 1 && all && !p.prev_cell)
-      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, true, 1, kShipped, true>), grid, dim3(threads), 0, s, p);
+    if (cpt == 1 && all && !p.prev_cell)   // the speculator's shapes: requests in stages
+      hipLaunchKernelGGL((sum_lstm_staged_kernel<T, kFastGelu, kSharedZ, true>), grid, dim3(threads), 0, s, p);
     else if (cpt == 1 && all)
-      hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, true, 1, kShipped>), grid, dim3(threads), 0, s, p);
+      hipLaunchKernelGGL((sum_lstm_staged_kernel<T, kFastGelu, kSharedZ, false>), grid, dim3(threads), 0, s, p);
     else if (cpt == 1)
       hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, false, 1, kShipped>), grid, dim3(threads), 0, s, p);
     else
@@ -489,6 +716,9 @@ static int sum_lstm_entry(const char *fn, bool shared_z, void *out_state, void *
   p.alpha = alpha;
   p.eps_cell = eps_cell;
   p.eps_state = eps_state;
+#ifdef ARCTIC_TUNING
+  p.trace = nullptr;
+#endif
   hipStream_t s = (hipStream_t)stream;
 #define ARCTIC_LSTM_DISPATCH(TYPE)                                        \
   do {                                                                    \

@@ -402,10 +402,12 @@ def bench_speculator(ops, dev, steps, warmup):
         with torch.cuda.graph(graph):
             for i in range(reps):
                 fn(i)
-        for _ in range(3):
+        # the eager loop above leaves the GPU mostly idle (the host issues a launch slower than it runs), and the first
+        # milliseconds of back-to-back work behind that run a few per cent slower: warm up with replays, not with three
+        for _ in range(max(20, warmup)):
             graph.replay()
         torch.cuda.synchronize()
-        us = event_times_us(graph.replay, max(10, steps // 2))
+        us = event_times_us(graph.replay, max(100, steps))
         med = statistics.median(us) / (reps * calls)
         out[name].update({"us_per_call_graph": round(med, 2),
                           "GBps_graph": round(per_call / med / 1e3, 1),
@@ -1210,11 +1212,12 @@ def bench_argmax_variants(dev, steps):
 
 
 # ARCTIC_LSTM_VARIANT values of the tuning build (sum_lstm.hip): bits 0-2 = arithmetic / ordering variants,
-# bits 3-4 = launch shape
+# bits 3-5 = launch shape, 66 = variant 2 with barriers between the request groups; "S<n>" = schedule n of the
+# staged kernel (ARCTIC_LSTM_STAGED)
 LSTM_VARIANTS = [
     (0, "loads c f pc i o, one row per 512-lane workgroup, output gate after the second row sum"),
     (1, "input gate loaded and consumed before forget gate and previous cell (c i f pc o)"),
-    (2, "as shipped: output gate's sigmoid ahead of the second row sum"),
+    (2, "output gate's sigmoid ahead of the second row sum (what shipped before the staged kernel)"),
     (3, "input gate first + output gate's sigmoid ahead of the second row sum"),
     (4, "shared reciprocals: one for the forget and input gates, one for the state GELU and the output gate"),
     (8, "two rows per workgroup, second row's loads issued behind the first row's"),
@@ -1222,7 +1225,85 @@ LSTM_VARIANTS = [
     (16, "two 16-byte chunks per lane (256 lanes per row)"),
     (24, "two chunks per lane and two rows per workgroup"),
     (34, "8-byte chunks, 1024 lanes per row (twice the waves, half the work each), early output gate"),
+    (66, "the row's gates requested gate by gate: a workgroup barrier between the groups of requests"),
+    ("S0", "staged kernel, every chunk requested at once (the order and the accesses of the rows above)"),
+    ("S1", "staged kernel: cell gate first; forget gate's s behind the first sum of squares; rest of the forget gate, "
+           "previous cell and input gate behind the candidate's GELU; output gate behind the forget gate's part and "
+           "consumed last"),
+    ("S2", "the same + scale / shift vectors requested where they are needed, not ahead of the row"),
+    ("S3", "the same + streaming stores of both outputs"),
+    ("S4", "the same + streaming load of the previous cell (shipped)"),
+    ("S5", "as shipped with the output gate's sigmoid ahead of the second row sum"),
+    ("S6", "as shipped with other request points: 2 | 4 | 7 | 9 chunks out"),
+    ("S7", "as shipped with other request points: 3 | 4 | 7 | 7"),
+    ("S8", "as shipped with other request points: 2 | 3 | 5 | 7"),
+    ("S9", "as shipped with other request points: 5 | 7 | 9 | 9"),
+    ("S10", "every chunk requested at once, with the streaming stores and the streaming load of the previous cell"),
 ]
+
+
+def bench_lstm_timeline(dev, steps):
+    """When the waves of one sum_lstm launch reach eight points of their life, from time stamps (the GPU's constant
+    100 MHz clock) that the measurement build's staged kernel writes: the shipped schedule next to the same kernel
+    with every chunk requested at once.  512 x 4096 bf16, eight rotating sets x three chained steps in one HIP graph;
+    the stamps of the graph's last launch are read, in microseconds after its first wave's start.  The stamps slow
+    a launch down by about a microsecond, so they show the order of events, not the operator's speed."""
+    import numpy as np
+    tuning = load_tuning_library()
+    if tuning is None:
+        return "libarctic_tuning_mi355x.so is not built"
+    T, Hd, sets = 512, 4096, 8
+    g = torch.Generator(device=dev).manual_seed(3)
+    rn = lambda *s: torch.randn(*s, generator=g, device=dev).to(torch.bfloat16)
+    S = [[rn(T, 4 * Hd) for _ in range(3)] for _ in range(sets)]
+    Z = [[rn(T, 4 * Hd) for _ in range(3)] for _ in range(sets)]
+    C0 = [rn(T, Hd) for _ in range(sets)]
+    vec = lambda m: (m + 0.02 * torch.randn(Hd, generator=g, device=dev)).to(torch.bfloat16)
+    w_cell, b_cell, w_state, b_state = vec(1.0), vec(0.0), vec(1.0), vec(0.0)
+    ST = [[torch.empty(T, Hd, dtype=torch.bfloat16, device=dev) for _ in range(3)] for _ in range(sets)]
+    CE = [[torch.empty(T, Hd, dtype=torch.bfloat16, device=dev) for _ in range(3)] for _ in range(sets)]
+    trace = torch.zeros(T * 8 * 8, dtype=torch.int64, device=dev)
+    os.environ["ARCTIC_LSTM_TRACE"] = hex(trace.data_ptr())
+
+    def run_all():
+        stream = torch.cuda.current_stream().cuda_stream
+        for i in range(sets):
+            cell = C0[i]
+            for k in range(3):
+                rc = tuning.arctic_sum_lstm(ST[i][k].data_ptr(), CE[i][k].data_ptr(), S[i][k].data_ptr(), Z[i][k].data_ptr(),
+                                            cell.data_ptr(), w_cell.data_ptr(), b_cell.data_ptr(), w_state.data_ptr(),
+                                            b_state.data_ptr(), T, Hd, 4 * Hd, 4 * Hd, Hd, Hd, 1.0, 1e-6, 1e-6, 0, 2, stream)
+                assert rc == 0
+                cell = CE[i][k]
+
+    points = ["wave started", "first requests out", "cell gate in, squares summed", "first row sum known",
+              "forget gate, previous cell, input gate in; new cell stored", "second row sum known", "state GELU done",
+              "output gate in; state stored"]
+    out = {}
+    for code, what in ((100, "every chunk requested at once"), (104, "requests in stages (shipped schedule)")):
+        os.environ["ARCTIC_LSTM_STAGED"] = str(code)
+        run_all()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            run_all()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        us = statistics.mean(event_times_us(graph.replay, max(10, steps // 4))) / (sets * 3)
+        t = trace.cpu().numpy().reshape(T, 8, 8).astype(np.float64)
+        t = (t - t[:, :, 0].min()) * 0.01   # ticks of 10 ns -> us after the first wave's start
+        rows = {}
+        for k, name in enumerate(points):
+            lower, upper = t[:T // 2, :, k].ravel(), t[T // 2:, :, k].ravel()
+            rows[name] = {"older_workgroup_of_a_cu_median_p90": [round(float(np.median(lower)), 2), round(float(np.percentile(lower, 90)), 2)],
+                          "younger_workgroup_of_a_cu_median_p90": [round(float(np.median(upper)), 2), round(float(np.percentile(upper, 90)), 2)],
+                          "all_waves_max": round(float(t[:, :, k].max()), 2)}
+        out[what] = {"us_per_call_graph_with_stamps": round(us, 2), "us_after_first_wave_start": rows}
+        del graph
+    os.environ.pop("ARCTIC_LSTM_STAGED", None)
+    os.environ.pop("ARCTIC_LSTM_TRACE", None)
+    return out
 
 
 def bench_lstm_variants(dev, steps):
@@ -1262,7 +1343,11 @@ def bench_lstm_variants(dev, steps):
     rounds = 3   # every variant is timed in each round, so drift over the run shows up as spread, not as a ranking
     graphs = {}
     for code, what in LSTM_VARIANTS:
-        os.environ["ARCTIC_LSTM_VARIANT"] = str(code)
+        os.environ.pop("ARCTIC_LSTM_STAGED", None)
+        if str(code).startswith("S"):
+            os.environ["ARCTIC_LSTM_STAGED"] = str(code)[1:]
+        else:
+            os.environ["ARCTIC_LSTM_VARIANT"] = str(code)
         run_all()
         torch.cuda.synchronize()
         got = [t.clone() for i in range(sets) for t in (ST[i][2], CE[i][2])]
@@ -1276,6 +1361,7 @@ def bench_lstm_variants(dev, steps):
         graphs[code] = graph
         out[str(code)] = {"variant": what, "bit_identical_to_variant_0": round(same, 5), "max_abs_diff": worst, "us": []}
     os.environ.pop("ARCTIC_LSTM_VARIANT", None)
+    os.environ.pop("ARCTIC_LSTM_STAGED", None)
     if floor is not None:
         OS = [torch.empty(T, Hd, dtype=torch.bfloat16, device=dev) for _ in range(2)]
         graph = torch.cuda.CUDAGraph()
@@ -1345,6 +1431,9 @@ def main():
     ap.add_argument("--lstm-variants", action="store_true",
                     help="instead of the benchmark, time the sum_lstm kernel variants of the tuning build against "
                          "each other and against the traffic-only kernel; prints one JSON object")
+    ap.add_argument("--lstm-timeline", action="store_true",
+                    help="instead of the benchmark, print when the waves of a sum_lstm launch reach the stages of the "
+                         "kernel (time stamps written by the tuning build), with requests at once and in stages")
     ap.add_argument("--argmax-variants", action="store_true",
                     help="instead of the benchmark, time loop shapes of the row-argmax kernel through the tuning build")
     ap.add_argument("--bulk-variants", nargs="?", const="compact", default=None, choices=["compact", "serving"],
@@ -1373,6 +1462,9 @@ def main():
         return
     if args.lstm_variants:
         print(json.dumps({"sum_lstm_variants": bench_lstm_variants(dev, args.steps)}), flush=True)
+        return
+    if args.lstm_timeline:
+        print(json.dumps({"sum_lstm_wave_timeline": bench_lstm_timeline(dev, args.steps)}), flush=True)
         return
     if args.argmax_variants:
         print(json.dumps({"row_argmax_variants": bench_argmax_variants(dev, args.steps)}), flush=True)

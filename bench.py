@@ -296,6 +296,7 @@ def load_floor_kernels():
     lib = ctypes.CDLL(path)
     vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
     lib.floor_lstm_traffic.argtypes = [vp, vp, vp, vp, vp, i64, i32, vp]
+    lib.floor_lstm_traffic_staged.argtypes = [vp, vp, vp, vp, vp, i64, i32, vp]
     lib.floor_ln_traffic.argtypes = [vp, vp, i64, i32, vp]
     lib.floor_stream_resident.argtypes = [vp, vp, i32, i64, i32, i32, i32, i32, vp]
     lib.floor_stream.argtypes = [vp, i32, vp, i32, i64, i32, vp, vp]
@@ -374,6 +375,13 @@ def bench_speculator(ops, dev, steps, warmup):
             floor.floor_lstm_traffic(S[i % sets][k].data_ptr(), Z[i % sets][k].data_ptr(), C0[i % sets].data_ptr(),
                                      OS[0].data_ptr(), OS[1].data_ptr(), T, Hd, stream)
 
+    def lstm3_traffic_staged(i):
+        # the same bytes requested in the stages of the library's kernel (each stage waits for what it would read)
+        stream = torch.cuda.current_stream().cuda_stream
+        for k in range(3):
+            floor.floor_lstm_traffic_staged(S[i % sets][k].data_ptr(), Z[i % sets][k].data_ptr(), C0[i % sets].data_ptr(),
+                                            OS[0].data_ptr(), OS[1].data_ptr(), T, Hd, stream)
+
     def ln_traffic_only(i):
         floor.floor_ln_traffic(X[i % sets].data_ptr(), OS[0].data_ptr(), T, Hd, torch.cuda.current_stream().cuda_stream)
 
@@ -386,6 +394,7 @@ def bench_speculator(ops, dev, steps, warmup):
              ("add_ln_gelu_as_three_ops", add_ln_gelu_separate, 6 * Hd * T, 1)]
     if floor is not None:
         cases.insert(1, ("sum_lstm_traffic_only_floor", lstm3_traffic_only, 22 * Hd * T, 3))
+        cases.insert(2, ("sum_lstm_traffic_only_in_stages", lstm3_traffic_staged, 22 * Hd * T, 3))
         cases.append(("speculator_ln_traffic_only_floor", ln_traffic_only, 4 * Hd * T, 1))
     out = {}
     for name, fn, per_call, calls in cases:
@@ -1372,7 +1381,17 @@ def bench_lstm_variants(dev, steps):
                     floor.floor_lstm_traffic(S[i][k].data_ptr(), Z[i][k].data_ptr(), C0[i].data_ptr(), OS[0].data_ptr(),
                                              OS[1].data_ptr(), T, Hd, stream)
         graphs["floor"] = graph
-        out["floor"] = {"variant": "lstm_traffic_kernel: the same loads and stores, no arithmetic", "us": []}
+        out["floor"] = {"variant": "lstm_traffic_kernel: the same loads and stores requested at once, no arithmetic", "us": []}
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            stream = torch.cuda.current_stream().cuda_stream
+            for i in range(sets):
+                for k in range(3):
+                    floor.floor_lstm_traffic_staged(S[i][k].data_ptr(), Z[i][k].data_ptr(), C0[i].data_ptr(),
+                                                    OS[0].data_ptr(), OS[1].data_ptr(), T, Hd, stream)
+        graphs["floor_staged"] = graph
+        out["floor_staged"] = {"variant": "lstm_traffic_staged_kernel: the same loads and stores requested in the shipped "
+                                          "kernel's stages, no arithmetic", "us": []}
     for _ in range(rounds):
         for key, graph in graphs.items():
             for _ in range(3):

@@ -3,6 +3,8 @@
 //
 //   floor_lstm_traffic   the loads and stores of sum_lstm (nine 16-byte loads per lane from the rows of
 //                        states, z4 and prev_cell, two 16-byte stores), one workgroup per row, no arithmetic
+//   floor_lstm_traffic_staged  the same traffic requested in the stages of the library's staged kernel, each stage
+//                        waiting for what its arithmetic would read, no arithmetic
 //   floor_ln_traffic     the load and the store of speculator_ln (one 16-byte chunk per lane, one workgroup per row)
 //   floor_row_read       the loads of the row-argmax kernel (one workgroup per row), nothing computed
 //   floor_node           an empty kernel, or one that makes a single memory round trip: the fixed cost of a node
@@ -35,6 +37,35 @@ __global__ void lstm_traffic_kernel(const char *s, const char *z, const char *pc
   const u32x4 a = v[0] ^ v[1] ^ v[2] ^ v[3] ^ v[8], b = v[4] ^ v[5] ^ v[6] ^ v[7];
   __builtin_nontemporal_store(a, (u32x4 *)(out_cell + row1) + c);
   __builtin_nontemporal_store(b, (u32x4 *)(out_state + row1) + c);
+}
+
+// The same traffic requested the way the library's staged sum_lstm kernel requests it: cell gate; wait for it; forget
+// gate's s; barrier; rest of the forget gate, previous cell, input gate; wait for forget gate and cell; output gate;
+// wait for the input gate; store the cell; barrier; wait for the output gate; store the state.  No arithmetic: what
+// the stages and their waits cost by themselves.
+__global__ void lstm_traffic_staged_kernel(const char *s, const char *z, const char *pc, char *out_state,
+                                           char *out_cell, int D) {
+  const int c = threadIdx.x;   // the host launches D / 8 lanes, a multiple of 64
+  const size_t row4 = (size_t)blockIdx.x * 4 * D * 2, row1 = (size_t)blockIdx.x * D * 2, gate = (size_t)D * 2;
+  auto ld = [&](const char *p) { return __builtin_nontemporal_load((const u32x4 *)p + c); };
+  const u32x4 zc = ld(z + row4 + 3 * gate), sc = ld(s + row4 + 3 * gate);
+  __builtin_amdgcn_sched_barrier(0);
+  u32x4 acc = zc ^ sc;
+  __builtin_amdgcn_sched_barrier(0);
+  const u32x4 sf = ld(s + row4);
+  __builtin_amdgcn_sched_barrier(0);
+  __syncthreads();
+  const u32x4 zf = ld(z + row4), cell = ld(pc + row1), si = ld(s + row4 + gate), zi = ld(z + row4 + gate);
+  __builtin_amdgcn_sched_barrier(0);
+  acc ^= sf ^ zf ^ cell;
+  __builtin_amdgcn_sched_barrier(0);
+  const u32x4 so = ld(s + row4 + 2 * gate), zo = ld(z + row4 + 2 * gate);
+  __builtin_amdgcn_sched_barrier(0);
+  acc ^= si ^ zi;
+  __builtin_nontemporal_store(acc, (u32x4 *)(out_cell + row1) + c);
+  __builtin_amdgcn_sched_barrier(0);
+  __syncthreads();
+  __builtin_nontemporal_store(acc ^ so ^ zo, (u32x4 *)(out_state + row1) + c);
 }
 
 __global__ void ln_traffic_kernel(const char *x, char *out, int hidden) {
@@ -248,6 +279,14 @@ extern "C" int floor_lstm_traffic(const void *s, const void *z, const void *pc, 
   hipLaunchKernelGGL(lstm_traffic_kernel, dim3((unsigned)rows), dim3((unsigned)((D / 8 + 63) & ~63)), 0,
                      (hipStream_t)stream, (const char *)s, (const char *)z, (const char *)pc, (char *)out_state,
                      (char *)out_cell, D);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+extern "C" int floor_lstm_traffic_staged(const void *s, const void *z, const void *pc, void *out_state, void *out_cell,
+                                         int64_t rows, int D, void *stream) {
+  if (rows <= 0 || D <= 0 || D % 512 != 0 || D / 8 > 1024) return 1;
+  hipLaunchKernelGGL(lstm_traffic_staged_kernel, dim3((unsigned)rows), dim3((unsigned)(D / 8)), 0, (hipStream_t)stream,
+                     (const char *)s, (const char *)z, (const char *)pc, (char *)out_state, (char *)out_cell, D);
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 

@@ -11,6 +11,8 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include <cstdint>
 
 #include "common.hpp"
@@ -37,63 +39,81 @@ struct Fp4Params {
   int block_size;
 };
 
-template <typename T>
+// kGroups groups of 16 elements per lane, 256 groups apart, so that a wave's 64 lanes stay on 64 consecutive groups
+// (2 KiB of source, 512 bytes of packed cache) in each of them.  All of a lane's requests go out before the first
+// group is looked at.
+template <typename T, int kGroups>
 __global__ __launch_bounds__(256) void kv_write_fp4_kernel(const Fp4Params p) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= p.total_groups) return;
   const int groups_per_row = p.num_heads * p.groups_per_head;
-  const int64_t row = idx / groups_per_row;            // token * 2 + (0 = K, 1 = V)
-  const int in_row = (int)(idx - row * groups_per_row);
-  const int head = in_row / p.groups_per_head;
-  const int group = in_row - head * p.groups_per_head;
-  const int64_t token = row >> 1;
-  const bool is_v = row & 1;
-
-  const int64_t slot = p.slot_mapping[token];
-  if (slot < 0 || slot >= p.num_slots) return;  // padding token, or a slot outside the cache
-  const int64_t blk = slot / p.block_size;
-  const int64_t off = slot - blk * p.block_size;
-
-  const char *src = (is_v ? p.value + token * p.value_stride_bytes : p.key + token * p.key_stride_bytes) +
-                    (int64_t)in_row * 32;
-  const uint4 lo = load16_stream(src), hi = load16_stream(src + 16);
-  float x[16];
-  {
-    float a[8], b[8];
-    unpack8<T>(lo, a);
-    unpack8<T>(hi, b);
+  int64_t slot[kGroups];
+  uint4 lo[kGroups], hi[kGroups];
+  int64_t idx[kGroups];
+  // the slot is requested first and the group's 32 bytes right behind it: their address does not depend on the slot,
+  // so one round trip to memory serves both (a padding token throws its group away)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      x[j] = a[j];
-      x[8 + j] = b[j];
-    }
+  for (int u = 0; u < kGroups; ++u) {
+    idx[u] = ((int64_t)blockIdx.x * kGroups + u) * 256 + threadIdx.x;
+    const int64_t at = min(idx[u], p.total_groups - 1);   // lanes past the end read the last group and drop it
+    const int64_t row = at / groups_per_row;              // token * 2 + (0 = K, 1 = V)
+    const int in_row = (int)(at - row * groups_per_row);
+    const int64_t token = row >> 1;
+    slot[u] = p.slot_mapping[token];
+    const char *src = ((row & 1) ? p.value + token * p.value_stride_bytes : p.key + token * p.key_stride_bytes) +
+                      (int64_t)in_row * 32;
+    lo[u] = load16_stream(src);
+    hi[u] = load16_stream(src + 16);
   }
-  float amax = 0.f;
+  __builtin_amdgcn_sched_barrier(0);   // keeps the loads above the tests of the slots
 #pragma unroll
-  for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(x[j]));  // a NaN never becomes the maximum
+  for (int u = 0; u < kGroups; ++u) {
+    if (idx[u] >= p.total_groups) continue;
+    if (slot[u] < 0 || slot[u] >= p.num_slots) continue;  // padding token, or a slot outside the cache
+    const int64_t row = idx[u] / groups_per_row;
+    const int in_row = (int)(idx[u] - row * groups_per_row);
+    const int head = in_row / p.groups_per_head;
+    const int group = in_row - head * p.groups_per_head;
+    const bool is_v = row & 1;
+    const int64_t blk = slot[u] / p.block_size;
+    const int64_t off = slot[u] - blk * p.block_size;
 
-  // scale = e4m3(amax / 6), saturating; SF = the value that byte decodes to
-  const float sf = __builtin_amdgcn_fmed3f(amax * 0.16666667163372039794921875f, 0.0f, 448.0f);
-  const uint32_t code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(sf, 0.0f, 0, false) & 0xffu;
-  const float SF = __builtin_amdgcn_cvt_f32_fp8((int)code, 0);
-  const float inv = (SF != 0.0f) ? 1.0f / SF : 0.0f;
+    float x[16];
+    {
+      float a[8], b[8];
+      unpack8<T>(lo[u], a);
+      unpack8<T>(hi[u], b);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        x[j] = a[j];
+        x[8 + j] = b[j];
+      }
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(x[j]));  // a NaN never becomes the maximum
 
-  uint32_t w0 = 0, w1 = 0;
-  w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[0] * inv, x[1] * inv, 1.0f, 0);
-  w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[2] * inv, x[3] * inv, 1.0f, 1);
-  w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[4] * inv, x[5] * inv, 1.0f, 2);
-  w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[6] * inv, x[7] * inv, 1.0f, 3);
-  w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[8] * inv, x[9] * inv, 1.0f, 0);
-  w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[10] * inv, x[11] * inv, 1.0f, 1);
-  w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[12] * inv, x[13] * inv, 1.0f, 2);
-  w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[14] * inv, x[15] * inv, 1.0f, 3);
+    // scale = e4m3(amax / 6), saturating; SF = the value that byte decodes to
+    const float sf = __builtin_amdgcn_fmed3f(amax * 0.16666667163372039794921875f, 0.0f, 448.0f);
+    const uint32_t code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(sf, 0.0f, 0, false) & 0xffu;
+    const float SF = __builtin_amdgcn_cvt_f32_fp8((int)code, 0);
+    const float inv = (SF != 0.0f) ? 1.0f / SF : 0.0f;
 
-  uint8_t *cache = is_v ? p.value_cache : p.key_cache;
-  uint8_t *scales = is_v ? p.value_scale_cache : p.key_scale_cache;
-  const int64_t at = blk * p.block_stride + off * p.page_stride + (int64_t)head * p.head_stride;
-  const int64_t sat = blk * (p.block_stride / 8) + off * (p.page_stride / 8) + (int64_t)head * (p.head_stride / 8);
-  store8_stream(cache + at + (int64_t)group * 8, make_uint2(w0, w1));
-  ((ARCTIC_GLOBAL uint8_t *)scales)[sat + group] = (uint8_t)code;
+    uint32_t w0 = 0, w1 = 0;
+    w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[0] * inv, x[1] * inv, 1.0f, 0);
+    w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[2] * inv, x[3] * inv, 1.0f, 1);
+    w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[4] * inv, x[5] * inv, 1.0f, 2);
+    w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[6] * inv, x[7] * inv, 1.0f, 3);
+    w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[8] * inv, x[9] * inv, 1.0f, 0);
+    w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[10] * inv, x[11] * inv, 1.0f, 1);
+    w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[12] * inv, x[13] * inv, 1.0f, 2);
+    w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[14] * inv, x[15] * inv, 1.0f, 3);
+
+    uint8_t *cache = is_v ? p.value_cache : p.key_cache;
+    uint8_t *scales = is_v ? p.value_scale_cache : p.key_scale_cache;
+    const int64_t at = blk * p.block_stride + off * p.page_stride + (int64_t)head * p.head_stride;
+    const int64_t sat = blk * (p.block_stride / 8) + off * (p.page_stride / 8) + (int64_t)head * (p.head_stride / 8);
+    store8_stream(cache + at + (int64_t)group * 8, make_uint2(w0, w1));
+    ((ARCTIC_GLOBAL uint8_t *)scales)[sat + group] = (uint8_t)code;
+  }
 }
 
 }  // namespace arctic
@@ -147,12 +167,28 @@ extern "C" int arctic_reshape_and_cache_flash_fp4(
   p.block_size = block_size;
   p.total_groups = num_tokens * 2 * num_heads * p.groups_per_head;
   p.num_slots = num_blocks > 0 ? num_blocks * (int64_t)block_size : INT64_MAX;
-  const int64_t grid = (p.total_groups + 255) / 256;
-  if (grid > 0x7fffffffLL) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: too many tokens", fn);
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == ARCTIC_DTYPE_BF16)
-    hipLaunchKernelGGL((kv_write_fp4_kernel<BF16>), dim3((unsigned)grid), dim3(256), 0, s, p);
-  else
-    hipLaunchKernelGGL((kv_write_fp4_kernel<F16>), dim3((unsigned)grid), dim3(256), 0, s, p);
+  // groups per lane: ARCTIC_FP4_GROUPS in the measurement build
+  int per_lane = 1;
+#ifdef ARCTIC_TUNING
+  if (const char *e = getenv("ARCTIC_FP4_GROUPS")) per_lane = atoi(e);
+#endif
+  const int64_t grid = (p.total_groups + 256 * per_lane - 1) / (256 * per_lane);
+  if (grid > 0x7fffffffLL) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: too many tokens", fn);
+#define ARCTIC_FP4_LAUNCH(G)                                                                             \
+  do {                                                                                                   \
+    if (dtype == ARCTIC_DTYPE_BF16)                                                                      \
+      hipLaunchKernelGGL((kv_write_fp4_kernel<BF16, G>), dim3((unsigned)grid), dim3(256), 0, s, p);      \
+    else                                                                                                 \
+      hipLaunchKernelGGL((kv_write_fp4_kernel<F16, G>), dim3((unsigned)grid), dim3(256), 0, s, p);       \
+  } while (0)
+  switch (per_lane) {
+#ifdef ARCTIC_TUNING
+    case 2: ARCTIC_FP4_LAUNCH(2); break;
+    case 4: ARCTIC_FP4_LAUNCH(4); break;
+#endif
+    default: ARCTIC_FP4_LAUNCH(1); break;
+  }
+#undef ARCTIC_FP4_LAUNCH
   return check_launch(fn);
 }

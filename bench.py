@@ -413,10 +413,10 @@ def bench_speculator(ops, dev, steps, warmup):
                 fn(i)
         # the eager loop above leaves the GPU mostly idle (the host issues a launch slower than it runs), and the first
         # milliseconds of back-to-back work behind that run a few per cent slower: warm up with replays, not with three
-        for _ in range(max(20, warmup)):
+        for _ in range(max(3, warmup)):
             graph.replay()
         torch.cuda.synchronize()
-        us = event_times_us(graph.replay, max(100, steps))
+        us = event_times_us(graph.replay, max(10, steps))
         med = statistics.median(us) / (reps * calls)
         out[name].update({"us_per_call_graph": round(med, 2),
                           "GBps_graph": round(per_call / med / 1e3, 1),

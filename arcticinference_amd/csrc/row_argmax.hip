@@ -110,8 +110,12 @@ struct HalfElem {
 // kVec: rows are 16-byte aligned, so the body of a row is read in 16-byte chunks; the elements behind
 // the last whole chunk (and everything when !kVec) are read one by one.
 // kUnroll chunks per lane form a batch; kPipelined: the next batch is requested before the current one is looked at;
-// kStaggered: the odd waves take half a batch on its own first, so that neighbouring waves are half a batch apart.
-template <typename Elem, bool kVec, int kUnroll = 4, bool kPipelined = false, bool kStaggered = false>
+// kStaggered: the odd waves take half a batch on its own first, so that neighbouring waves are half a batch apart;
+// kLockstep: a workgroup barrier (no memory wait) behind every batch's requests, so that every wave of the row has
+// asked for batch k before any wave asks for batch k + 1 (a CU serves its oldest wave first: without the barrier the
+// oldest wave runs through all its batches before the youngest gets its first one in).
+template <typename Elem, bool kVec, int kUnroll = 4, bool kPipelined = false, bool kStaggered = false,
+          bool kLockstep = false>
 __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ out, const char *__restrict__ in,
                                                           int64_t row_stride_bytes, int cols, int64_t max_index) {
   __shared__ float wave_value[16];
@@ -179,6 +183,17 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) cur[u] = nxt[u];
         c0 += stride;
+      }
+    } else if constexpr (kLockstep) {
+      const int batches = (chunks + stride - 1) / stride;   // the same for every wave, as the barrier needs it
+      int c0 = threadIdx.x;
+      for (int b = 0; b < batches; ++b, c0 += stride) {
+        uint4 raw[kUnroll];
+        request(c0, raw);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        look_at(c0, raw);
       }
     } else {
       int c0 = threadIdx.x;
@@ -276,7 +291,7 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
   int variant = 0;
   if (const char *e = getenv("ARCTIC_ARGMAX_VARIANT")) variant = atoi(e);
   if (variant & 8) threads = std::max(64, threads / 2);
-  variant &= 7;
+  variant &= ~8;   // + 16: a barrier behind every batch's requests (batches of 4, 2 or 1: 16, 17, 18)
 #define ARCTIC_ARGMAX_VEC(ELEM)                                                                                          \
   do {                                                                                                                   \
     const dim3 b((unsigned)threads);                                                                                     \
@@ -287,6 +302,9 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
       case 4: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 2, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
       case 5: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 2, false>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
       case 6: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
+      case 16: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
+      case 17: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 2, false, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
+      case 18: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 1, false, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
       default: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
     }                                                                                                                    \
   } while (0)

@@ -1188,6 +1188,10 @@ def bench_argmax_variants(dev, steps):
              (2, "batches of 8"), (3, "batches of 8, next batch requested first"),
              (4, "batches of 2, next batch requested first"), (5, "batches of 2"),
              (6, "batches of 4, odd waves half a batch ahead of the even ones"),
+             (16, "batches of 4 with a workgroup barrier behind every batch's requests"),
+             (17, "batches of 2 with a workgroup barrier behind every batch's requests"),
+             (18, "batches of 1 with a workgroup barrier behind every batch's requests"),
+             (24, "512 lanes, batches of 4 with a workgroup barrier behind every batch's requests"),
              (9, "512 lanes, batches of 4, next batch first"),
              (11, "512 lanes, batches of 8, next batch first")]
 

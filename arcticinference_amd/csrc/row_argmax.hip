@@ -19,48 +19,44 @@
 
 namespace arctic {
 
-struct Winner {
-  float value;
-  int index;   // -1: nothing seen yet
-};
-
-// torch's GreaterOrNan with the index as tie break (aten/src/ATen/native/SharedReduceOps.h)
-__device__ __forceinline__ bool beats(float a, int ia, float b, int ib) {
-  if (ib < 0) return true;
-  if (ia < 0) return false;
-  const bool a_nan = a != a, b_nan = b != b;
-  if (a_nan) return b_nan ? ia < ib : true;
-  if (b_nan) return false;
-  return a == b ? ia < ib : a > b;
+// A candidate as one 64-bit key whose unsigned order is torch's order of winners (GreaterOrNan with the index as tie
+// break, aten/src/ATen/native/SharedReduceOps.h): the value's bits mapped monotonically to an unsigned number in the
+// upper half (-0 counts as +0, every NaN as the largest number of all), the complement of the index in the lower half
+// (among equal values the lowest index is the largest key).  0 = nothing seen: no element maps to upper half 0.
+// Merging two candidates is then one 64-bit unsigned maximum instead of a cascade of floating-point cases.
+__device__ __forceinline__ uint64_t winner_key(float value, int index) {
+  if (index < 0) return 0;
+  uint32_t b = __float_as_uint(value);
+  if (b == 0x80000000u) b = 0;   // -0 -> +0 (on the bits: no arithmetic that a denormal mode could touch)
+  uint32_t o = b ^ ((b & 0x80000000u) ? 0xffffffffu : 0x80000000u);
+  if (value != value) o = 0xffffffffu;
+  return ((uint64_t)o << 32) | (uint32_t)~(uint32_t)index;
 }
-
-__device__ __forceinline__ void offer(Winner &w, float v, int i) {
-  if (beats(v, i, w.value, w.index)) {
-    w.value = v;
-    w.index = i;
-  }
-}
+__device__ __forceinline__ int winner_index(uint64_t key) { return key ? (int)~(uint32_t)key : -1; }
 
 // The wave's winner in every lane.  Inside each row of 16 lanes the candidates meet through DPP lane exchanges
 // (vector-ALU moves, no LDS round trip): partners at distance 1 and 2 inside a quad, then the mirrored half and the
 // mirrored row, after which all 16 lanes of a row agree; the four row winners are read with v_readlane.
 template <int kCtrl>
-__device__ __forceinline__ void meet(Winner &w) {
-  const float ov = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(w.value), kCtrl, 0xf, 0xf, true));
-  const int oi = __builtin_amdgcn_update_dpp(0, w.index, kCtrl, 0xf, 0xf, true);
-  offer(w, ov, oi);
+__device__ __forceinline__ uint64_t meet(uint64_t k) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)k, kCtrl, 0xf, 0xf, true);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(k >> 32), kCtrl, 0xf, 0xf, true);
+  const uint64_t other = ((uint64_t)hi << 32) | lo;
+  return other > k ? other : k;
 }
 
-__device__ __forceinline__ Winner wave_winner(Winner w) {
-  meet<0xB1>(w);   // quad_perm [1,0,3,2]
-  meet<0x4E>(w);   // quad_perm [2,3,0,1]
-  meet<0x141>(w);  // row_half_mirror
-  meet<0x140>(w);  // row_mirror
-  const int vb = __float_as_int(w.value);
-  Winner r = {__int_as_float(__builtin_amdgcn_readlane(vb, 0)), __builtin_amdgcn_readlane(w.index, 0)};
+__device__ __forceinline__ uint64_t wave_winner(uint64_t k) {
+  k = meet<0xB1>(k);   // quad_perm [1,0,3,2]
+  k = meet<0x4E>(k);   // quad_perm [2,3,0,1]
+  k = meet<0x141>(k);  // row_half_mirror
+  k = meet<0x140>(k);  // row_mirror
+  uint64_t r = 0;
 #pragma unroll
-  for (int lane = 16; lane < 64; lane += 16)
-    offer(r, __int_as_float(__builtin_amdgcn_readlane(vb, lane)), __builtin_amdgcn_readlane(w.index, lane));
+  for (int lane = 0; lane < 64; lane += 16) {
+    const uint64_t row = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(k >> 32), lane) << 32) |
+                         (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)k, lane);
+    r = row > r ? row : r;
+  }
   return r;
 }
 
@@ -109,6 +105,12 @@ struct HalfElem {
 
 // kVec: rows are 16-byte aligned, so the body of a row is read in 16-byte chunks; the elements behind
 // the last whole chunk (and everything when !kVec) are read one by one.
+#ifdef ARCTIC_TUNING
+// measurement build: where the waves write the GPU's 100 MHz clock at eight points of their life (ARCTIC_ARGMAX_TRACE
+// holds the address of rows x 16 waves x 8 words), or nullptr
+__device__ unsigned long long *g_argmax_trace = nullptr;
+#endif
+
 // kUnroll chunks per lane form a batch; kPipelined: the next batch is requested before the current one is looked at;
 // kStaggered: the odd waves take half a batch on its own first, so that neighbouring waves are half a batch apart;
 // kLockstep: a workgroup barrier (no memory wait) behind every batch's requests, so that every wave of the row has
@@ -118,8 +120,19 @@ template <typename Elem, bool kVec, int kUnroll = 4, bool kPipelined = false, bo
           bool kLockstep = false>
 __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ out, const char *__restrict__ in,
                                                           int64_t row_stride_bytes, int cols, int64_t max_index) {
-  __shared__ float wave_value[16];
-  __shared__ int wave_index[16];
+  __shared__ uint64_t wave_key[16];
+  auto stamp = [&](int k) {
+#ifdef ARCTIC_TUNING
+    unsigned long long *trace = g_argmax_trace;
+    if (trace) {
+      __builtin_amdgcn_sched_barrier(0);
+      const unsigned long long t = __builtin_amdgcn_s_memrealtime();
+      if ((threadIdx.x & 63) == 0) trace[((size_t)blockIdx.x * 16 + threadIdx.x / 64) * 8 + k] = t;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#endif
+  };
+  stamp(0);
   const char *row = in + (int64_t)blockIdx.x * row_stride_bytes;
   // Per lane: the largest number seen, the chunk it was first seen in and that chunk's words (a strict ">" keeps the
   // earlier of equal values, the lane's chunk indices only grow); which of the chunk's elements it was is worked out
@@ -214,10 +227,11 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
           c0 += kLead * (int)blockDim.x;
         }
       }
-      for (; c0 < chunks; c0 += stride) {
+      for (int batch = 0; c0 < chunks; c0 += stride, ++batch) {
         uint4 raw[kUnroll];
         request(c0, raw);
         look_at(c0, raw);
+        stamp(1 + min(batch, 3));   // batch looked at
       }
     }
     done = chunks * P;
@@ -241,22 +255,21 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
     number(v, i);
     if (v != v) nan_at = min(nan_at, i);
   }
-  Winner w = nan_at != 0x7fffffff ? Winner{__builtin_nanf(""), nan_at} : Winner{best, best_at};
+  uint64_t w = nan_at != 0x7fffffff ? winner_key(__builtin_nanf(""), nan_at) : winner_key(best, best_at);
+  stamp(5);   // the lane's winner is known
 
   w = wave_winner(w);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  if (lane == 0) {
-    wave_value[wave] = w.value;
-    wave_index[wave] = w.index;
-  }
+  if (lane == 0) wave_key[wave] = w;
   __syncthreads();
+  stamp(6);   // every wave's winner is in LDS
   if (wave == 0) {
     const int waves = blockDim.x >> 6;
-    Winner x = {0.f, -1};
-    if (lane < waves) x = Winner{wave_value[lane], wave_index[lane]};
+    uint64_t x = lane < waves ? wave_key[lane] : 0;
     x = wave_winner(x);
     if (lane == 0) {
-      int64_t idx = x.index < 0 ? 0 : x.index;
+      const int found = winner_index(x);
+      int64_t idx = found < 0 ? 0 : found;
       out[blockIdx.x] = idx > max_index ? max_index : idx;
     }
   }
@@ -287,9 +300,18 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
   const dim3 grid((unsigned)rows), block((unsigned)threads);
 #ifdef ARCTIC_TUNING
   // measurement build: ARCTIC_ARGMAX_VARIANT = 1 pipelined batches of 4, 2 batches of 8, 3 pipelined batches of 8,
-  // 4 pipelined batches of 2, 5 batches of 2, 6 batches of 4 with the odd waves half a batch ahead; + 8: half the lanes
+  // 4 pipelined batches of 2, 5 batches of 2, 6 batches of 4 with the odd waves half a batch ahead, 7 batches of 1; + 8: half the lanes
   int variant = 0;
   if (const char *e = getenv("ARCTIC_ARGMAX_VARIANT")) variant = atoi(e);
+  {
+    const char *e = getenv("ARCTIC_ARGMAX_TRACE");
+    unsigned long long *trace = e ? (unsigned long long *)strtoull(e, nullptr, 0) : nullptr;
+    static unsigned long long *current = nullptr;
+    if (trace != current) {
+      (void)hipMemcpyToSymbol(HIP_SYMBOL(g_argmax_trace), &trace, sizeof(trace));
+      current = trace;
+    }
+  }
   if (variant & 8) threads = std::max(64, threads / 2);
   variant &= ~8;   // + 16: a barrier behind every batch's requests (batches of 4, 2 or 1: 16, 17, 18)
 #define ARCTIC_ARGMAX_VEC(ELEM)                                                                                          \
@@ -302,6 +324,7 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
       case 4: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 2, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
       case 5: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 2, false>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
       case 6: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
+      case 7: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 1, false>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
       case 16: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
       case 17: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 2, false, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
       case 18: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 1, false, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
@@ -309,9 +332,20 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
     }                                                                                                                    \
   } while (0)
 #else
-#define ARCTIC_ARGMAX_VEC(ELEM)                                                                             \
-  hipLaunchKernelGGL((row_argmax_kernel<ELEM, true>), grid, block, 0, s, out, (const char *)logits, stride_bytes, cols, \
-                     max_index)
+  // Launches of about one and a half to three workgroups per CU (the 256 CUs of this GPU; a decode batch of a few
+  // hundred rows) keep their waves in step, a chunk at a time: the two workgroups of a CU then finish together with
+  // little left to do, 5 % faster at 384 and 512 rows.  With fewer rows a wave needs four chunks in flight to cover
+  // the latency, with more the generations of workgroups overlap by themselves (measured 16 to 4096 rows).
+  const bool lockstep = rows > 256 && rows <= 768;
+#define ARCTIC_ARGMAX_VEC(ELEM)                                                                                   \
+  do {                                                                                                            \
+    if (lockstep)                                                                                                 \
+      hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 1, false, false, true>), grid, block, 0, s, out,          \
+                         (const char *)logits, stride_bytes, cols, max_index);                                    \
+    else                                                                                                          \
+      hipLaunchKernelGGL((row_argmax_kernel<ELEM, true>), grid, block, 0, s, out, (const char *)logits,           \
+                         stride_bytes, cols, max_index);                                                          \
+  } while (0)
 #endif
 #define ARCTIC_ARGMAX_LAUNCH(ELEM)                                                                          \
   do {                                                                                                      \

@@ -105,12 +105,6 @@ struct HalfElem {
 
 // kVec: rows are 16-byte aligned, so the body of a row is read in 16-byte chunks; the elements behind
 // the last whole chunk (and everything when !kVec) are read one by one.
-#ifdef ARCTIC_TUNING
-// measurement build: where the waves write the GPU's 100 MHz clock at eight points of their life (ARCTIC_ARGMAX_TRACE
-// holds the address of rows x 16 waves x 8 words), or nullptr
-__device__ unsigned long long *g_argmax_trace = nullptr;
-#endif
-
 // kUnroll chunks per lane form a batch; kPipelined: the next batch is requested before the current one is looked at;
 // kStaggered: the odd waves take half a batch on its own first, so that neighbouring waves are half a batch apart;
 // kLockstep: a workgroup barrier (no memory wait) behind every batch's requests, so that every wave of the row has
@@ -121,18 +115,6 @@ template <typename Elem, bool kVec, int kUnroll = 4, bool kPipelined = false, bo
 __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ out, const char *__restrict__ in,
                                                           int64_t row_stride_bytes, int cols, int64_t max_index) {
   __shared__ uint64_t wave_key[16];
-  auto stamp = [&](int k) {
-#ifdef ARCTIC_TUNING
-    unsigned long long *trace = g_argmax_trace;
-    if (trace) {
-      __builtin_amdgcn_sched_barrier(0);
-      const unsigned long long t = __builtin_amdgcn_s_memrealtime();
-      if ((threadIdx.x & 63) == 0) trace[((size_t)blockIdx.x * 16 + threadIdx.x / 64) * 8 + k] = t;
-      __builtin_amdgcn_sched_barrier(0);
-    }
-#endif
-  };
-  stamp(0);
   const char *row = in + (int64_t)blockIdx.x * row_stride_bytes;
   // Per lane: the largest number seen, the chunk it was first seen in and that chunk's words (a strict ">" keeps the
   // earlier of equal values, the lane's chunk indices only grow); which of the chunk's elements it was is worked out
@@ -227,11 +209,10 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
           c0 += kLead * (int)blockDim.x;
         }
       }
-      for (int batch = 0; c0 < chunks; c0 += stride, ++batch) {
+      for (; c0 < chunks; c0 += stride) {
         uint4 raw[kUnroll];
         request(c0, raw);
         look_at(c0, raw);
-        stamp(1 + min(batch, 3));   // batch looked at
       }
     }
     done = chunks * P;
@@ -256,13 +237,11 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
     if (v != v) nan_at = min(nan_at, i);
   }
   uint64_t w = nan_at != 0x7fffffff ? winner_key(__builtin_nanf(""), nan_at) : winner_key(best, best_at);
-  stamp(5);   // the lane's winner is known
 
   w = wave_winner(w);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   if (lane == 0) wave_key[wave] = w;
   __syncthreads();
-  stamp(6);   // every wave's winner is in LDS
   if (wave == 0) {
     const int waves = blockDim.x >> 6;
     uint64_t x = lane < waves ? wave_key[lane] : 0;
@@ -303,15 +282,6 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
   // 4 pipelined batches of 2, 5 batches of 2, 6 batches of 4 with the odd waves half a batch ahead, 7 batches of 1; + 8: half the lanes
   int variant = 0;
   if (const char *e = getenv("ARCTIC_ARGMAX_VARIANT")) variant = atoi(e);
-  {
-    const char *e = getenv("ARCTIC_ARGMAX_TRACE");
-    unsigned long long *trace = e ? (unsigned long long *)strtoull(e, nullptr, 0) : nullptr;
-    static unsigned long long *current = nullptr;
-    if (trace != current) {
-      (void)hipMemcpyToSymbol(HIP_SYMBOL(g_argmax_trace), &trace, sizeof(trace));
-      current = trace;
-    }
-  }
   if (variant & 8) threads = std::max(64, threads / 2);
   variant &= ~8;   // + 16: a barrier behind every batch's requests (batches of 4, 2 or 1: 16, 17, 18)
 #define ARCTIC_ARGMAX_VEC(ELEM)                                                                                          \

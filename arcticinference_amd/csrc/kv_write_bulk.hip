@@ -81,6 +81,7 @@ struct BulkParams {
 #ifdef ARCTIC_TUNING
   int loads_before_stores;  // measurement build: the next batch is requested before this one is converted and stored
   unsigned items;           // measurement build: not 0 = workgroups loop over this many items (ARCTIC_BULK_PERSISTENT)
+  int lockstep;             // measurement build: a barrier behind every batch's requests (ARCTIC_BULK_LOCKSTEP)
 #endif
 };
 
@@ -357,6 +358,15 @@ __device__ __forceinline__ void bulk_item(const BulkParams &p, const LayerTables
       }
     }
     if constexpr (!kLoadsFirst) load_batch(cn, nxt);
+#ifdef ARCTIC_TUNING
+    // measurement build (ARCTIC_BULK_LOCKSTEP, whole batches only): the waves of a workgroup request batch k + 1
+    // together, behind a barrier that waits for no memory
+    if (p.lockstep) {
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#endif
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) cur[u] = nxt[u];
     c = cn;
@@ -901,9 +911,15 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
     p.loads_before_stores = 0;
     if (const char *e = getenv("ARCTIC_BULK_LOADS_FIRST")) p.loads_before_stores = atoi(e) != 0;
     p.items = 0;
+    p.lockstep = 0;
 #endif
     p.layers_per_group = (count + groups - 1) / groups;
     p.groups_per_token = (count + p.layers_per_group - 1) / p.layers_per_group;
+#ifdef ARCTIC_TUNING
+    if (const char *e = getenv("ARCTIC_BULK_LOCKSTEP"))   // only where every lane of a workgroup runs the same number of batches
+      p.lockstep = atoi(e) != 0 && vec && count % p.layers_per_group == 0 &&
+                   (2LL * p.layers_per_group * p.chunks_per_row) % 1024 == 0 && !p.indices;
+#endif
     const int lanes = !vec ? kScalarThreads : (wide && p.chunk_shift >= 0) ? 512 : 256;   // of the shape launched below
     const int64_t index_blocks = p.indices ? (p.num_out_rows + lanes - 1) / lanes : 0;
     const int64_t grid = num_tokens * p.groups_per_token + index_blocks;

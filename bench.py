@@ -1124,6 +1124,7 @@ def bench_bulk_variants(dev, steps, placement="compact"):
         assert rc == 0
 
     cases = [("as shipped (1024 lanes x 1 chunk, 2 groups of 20 layers, a batch's stores before the next batch's loads)", {}),
+             ("as shipped + a workgroup barrier (no memory wait) behind every batch's requests", {"ARCTIC_BULK_LOCKSTEP": "1"}),
              ("512 lanes x 2 chunks", {"ARCTIC_BULK_SHAPE": "5"}),
              ("512 lanes x 2 chunks, the next batch's loads before this batch's stores", {"ARCTIC_BULK_LOADS_FIRST": "1"}),
              ("256 lanes x 4 chunks", {"ARCTIC_BULK_WIDE": "0"}),
@@ -1150,7 +1151,7 @@ def bench_bulk_variants(dev, steps, placement="compact"):
     written, same = {}, {}
     for _ in range(3):
         for name, env in cases:
-            for k in ("ARCTIC_BULK_LOADS_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT", "ARCTIC_BULK_RESIDENT"):
+            for k in ("ARCTIC_BULK_LOADS_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT", "ARCTIC_BULK_RESIDENT", "ARCTIC_BULK_LOCKSTEP"):
                 os.environ.pop(k, None)
             os.environ.update(env)
             # what the variant writes into the first and the last layer's caches, against the first variant's
@@ -1163,7 +1164,7 @@ def bench_bulk_variants(dev, steps, placement="compact"):
             written.setdefault("first", sums)
             same[name] = same.get(name, True) and sums == written["first"]
             out[name].append(round(statistics.mean(event_times_us(launch, max(10, steps // 4))), 1))
-    for k in ("ARCTIC_BULK_LOADS_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT", "ARCTIC_BULK_RESIDENT"):
+    for k in ("ARCTIC_BULK_LOADS_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT", "ARCTIC_BULK_RESIDENT", "ARCTIC_BULK_LOCKSTEP"):
         os.environ.pop(k, None)
     return {name: {"kernel_us_rounds": v, "GBps": round(w.bytes / statistics.mean(v) / 1e3),
                    "hbm_frac": round(w.bytes / statistics.mean(v) / 1e3 / HBM_PEAK_GBS, 4),

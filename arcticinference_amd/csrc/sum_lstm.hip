@@ -353,15 +353,18 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
 // out after the first sum of squares, kAhead2 after the candidate's GELU, kAhead3 after the forget gate's part of
 // the cell update, all nine once the new cell is stored.  Waves that are computing leave the request slots to the
 // others, so both rows of a CU arrive gate by gate and every stage's arithmetic runs while the next stage is in flight.
-// kVectors places the requests for the scale / shift vectors (the same for every row, cache resident): 0: all four
+// kBarriers: bit k = a workgroup barrier that waits for no memory behind the requests of point k (0: the first
+// chunks, 2: after the candidate's GELU, 3: after the forget gate's part; point 1 is followed by the first row sum's
+// barrier anyway).  kVectors places the requests for the scale / shift vectors (the same for every row, cache resident): 0: all four
 // ahead of the row; 1: the cell norm's pair behind the first sum of squares, the state norm's behind the forget
 // gate's part; 2: the cell norm's pair right behind the first kAhead0 chunks, the state norm's behind the candidate's
 // GELU.  kStreamOutputs / kStreamCell: non-temporal stores of both outputs / load of the previous cell (a step's
 // outputs are read by the next launches of the step, but a launch boundary writes them back anyway, and stores that
 // stream leave earlier).
 template <int kAhead0_, int kAhead1_, int kAhead2_, int kAhead3_, bool kEarlyGate_, int kVectors_, bool kStreamOutputs_,
-          bool kStreamCell_>
+          bool kStreamCell_, int kBarriers_ = 0>
 struct LstmSchedule {
+  static constexpr int kBarriers = kBarriers_;   // bit k: a workgroup barrier (no memory wait) behind the requests of point k
   static constexpr int kAhead0 = kAhead0_, kAhead1 = kAhead1_, kAhead2 = kAhead2_, kAhead3 = kAhead3_;
   static constexpr bool kEarlyGate = kEarlyGate_, kStreamOutputs = kStreamOutputs_, kStreamCell = kStreamCell_;
   static constexpr int kVectors = kVectors_;
@@ -371,8 +374,10 @@ struct LstmSchedule {
 };
 // measured best of a sweep over the request points (512 rows of 4096): the cell gate first, the forget gate's s
 // behind the first sum of squares, the rest of the forget gate, the previous cell and the input gate behind the
-// candidate's GELU, the output gate behind the forget gate's part; the output gate is consumed last
-using LstmShippedSchedule = LstmSchedule<2, 3, 7, 7, false, 2, true, true>;
+// candidate's GELU, with a workgroup barrier (no memory wait) behind them, so that every wave of the row has made
+// these requests before any wave makes the next ones; the output gate behind the forget gate's part; the output gate
+// is consumed last
+using LstmShippedSchedule = LstmSchedule<2, 3, 7, 7, false, 2, true, true, 4>;
 
 // Same arithmetic, operation for operation, as sum_lstm_vec_kernel: results are bit-identical.
 template <typename T, bool kFastGelu, bool kSharedZ, bool kZeroCell, typename S = LstmShippedSchedule, bool kTrace = false>
@@ -432,7 +437,14 @@ __global__ __launch_bounds__(512) void sum_lstm_staged_kernel(const LstmParams p
     if constexpr (kFrom <= 8 && 8 < kTo && !kSharedZ) in[8] = C::load_stream(z_row + 2 * gate_bytes);
     __builtin_amdgcn_sched_barrier(0);
   };
+  auto in_step = [&](int point) {
+    if ((S::kBarriers >> point) & 1) {
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
   request(integral_constant<int, 0>(), integral_constant<int, S::kAhead0>());
+  in_step(0);
   request_vectors(1);
   stamp(1);   // the first requests are out
 
@@ -460,6 +472,7 @@ __global__ __launch_bounds__(512) void sum_lstm_staged_kernel(const LstmParams p
   }
   request_vectors(3);
   request(integral_constant<int, S::kAhead1>(), integral_constant<int, S::kAhead2>());
+  in_step(2);
 
   // phase 2: cell update; write out_cell (reference :104-140)
   float cell[E];
@@ -470,6 +483,7 @@ __global__ __launch_bounds__(512) void sum_lstm_staged_kernel(const LstmParams p
   for (int j = 0; j < E; ++j) cell[j] = sigmoid_f(fmaf(p.alpha, b[j], a[j])) * c[j];
   request_vectors(4);
   request(integral_constant<int, S::kAhead2>(), integral_constant<int, S::kAhead3>());
+  in_step(3);
   in[5].template unpack<T>(a);
   (kSharedZ ? in[0] : in[6]).template unpack<T>(b);
   ss = 0.f;
@@ -632,13 +646,18 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
         ARCTIC_STAGED(1, 2, 3, 7, 7, false, 0, false, false)   // staged requests
         ARCTIC_STAGED(2, 2, 3, 7, 7, false, 2, false, false)   // + the vectors requested where they are needed
         ARCTIC_STAGED(3, 2, 3, 7, 7, false, 2, true, false)    // + streaming stores
-        ARCTIC_STAGED(4, 2, 3, 7, 7, false, 2, true, true)     // + streaming load of the previous cell: as shipped
-        ARCTIC_STAGED(5, 2, 3, 7, 7, true, 2, true, true)      // as shipped with the early output gate
+        ARCTIC_STAGED(4, 2, 3, 7, 7, false, 2, true, true)     // + streaming load of the previous cell
+        ARCTIC_STAGED(5, 2, 3, 7, 7, true, 2, true, true)      // the same with the early output gate
         ARCTIC_STAGED(6, 2, 4, 7, 9, false, 2, true, true)     // other request points
         ARCTIC_STAGED(7, 3, 4, 7, 7, false, 2, true, true)
         ARCTIC_STAGED(8, 2, 3, 5, 7, false, 2, true, true)
         ARCTIC_STAGED(9, 5, 7, 9, 9, false, 2, true, true)
         ARCTIC_STAGED(10, 9, 9, 9, 9, true, 0, true, true)     // everything at once with the streaming accesses
+        ARCTIC_STAGED(11, 2, 3, 7, 7, false, 2, true, true, 1)    // 4 + a barrier behind the first requests
+        ARCTIC_STAGED(12, 2, 3, 7, 7, false, 2, true, true, 4)    // ... behind the requests after the candidate's GELU: as shipped
+        ARCTIC_STAGED(13, 2, 3, 7, 7, false, 2, true, true, 8)    // ... behind the output gate's requests
+        ARCTIC_STAGED(14, 2, 3, 7, 7, false, 2, true, true, 13)   // ... behind all three
+        ARCTIC_STAGED(15, 2, 3, 7, 7, false, 2, true, true, 12)   // ... behind the last two
 #undef ARCTIC_STAGED
         return;
       }

@@ -1243,12 +1243,18 @@ LSTM_VARIANTS = [
            "consumed last"),
     ("S2", "the same + scale / shift vectors requested where they are needed, not ahead of the row"),
     ("S3", "the same + streaming stores of both outputs"),
-    ("S4", "the same + streaming load of the previous cell (shipped)"),
-    ("S5", "as shipped with the output gate's sigmoid ahead of the second row sum"),
-    ("S6", "as shipped with other request points: 2 | 4 | 7 | 9 chunks out"),
-    ("S7", "as shipped with other request points: 3 | 4 | 7 | 7"),
-    ("S8", "as shipped with other request points: 2 | 3 | 5 | 7"),
-    ("S9", "as shipped with other request points: 5 | 7 | 9 | 9"),
+    ("S4", "the same + streaming load of the previous cell"),
+    ("S12", "the same + a workgroup barrier (no memory wait) behind the requests that follow the candidate's GELU "
+            "(shipped)"),
+    ("S11", "S4 + that barrier behind the first requests instead"),
+    ("S13", "S4 + that barrier behind the output gate's requests instead"),
+    ("S14", "S4 + all three barriers"),
+    ("S15", "S4 + the barriers behind the last two groups of requests"),
+    ("S5", "S4 with the output gate's sigmoid ahead of the second row sum"),
+    ("S6", "S4 with other request points: 2 | 4 | 7 | 9 chunks out"),
+    ("S7", "S4 with other request points: 3 | 4 | 7 | 7"),
+    ("S8", "S4 with other request points: 2 | 3 | 5 | 7"),
+    ("S9", "S4 with other request points: 5 | 7 | 9 | 9"),
     ("S10", "every chunk requested at once, with the streaming stores and the streaming load of the previous cell"),
 ]
 
@@ -1291,7 +1297,7 @@ def bench_lstm_timeline(dev, steps):
               "forget gate, previous cell, input gate in; new cell stored", "second row sum known", "state GELU done",
               "output gate in; state stored"]
     out = {}
-    for code, what in ((100, "every chunk requested at once"), (104, "requests in stages (shipped schedule)")):
+    for code, what in ((100, "every chunk requested at once"), (112, "requests in stages (shipped schedule)")):
         os.environ["ARCTIC_LSTM_STAGED"] = str(code)
         run_all()
         torch.cuda.synchronize()

@@ -3,12 +3,16 @@
 // Replaces sum_lstm_cuda and its kernels
 // (csrc/custom_ops/sum_lstm.cu:14-473 in the reference).
 //
-// One workgroup per row.  On the vector path each lane owns 16-byte chunks
+// One workgroup per row.  On the vector paths each lane owns 16-byte chunks
 // (8 elements) at the same column of all four gates of `states` and `z4` and of
-// `prev_cell`: nine 16-byte loads per chunk, issued together.  The row then
-// stays in registers across both RMS reductions, so HBM sees 9*D elements read
-// and 2*D written per row (the reference re-reads the cell gate and reads
-// out_cell back: 12*D).  Sums are DPP wave reductions plus an LDS combine.
+// `prev_cell`: nine 16-byte loads per chunk.  The row then stays in registers
+// across both RMS reductions, so HBM sees 9*D elements read and 2*D written per
+// row (the reference re-reads the cell gate and reads out_cell back: 12*D).
+// Sums are DPP wave reductions plus an LDS combine.  Three kernels:
+// sum_lstm_staged_kernel (the speculator's shapes: the nine loads are requested
+// in stages, between the stages of the arithmetic), sum_lstm_vec_kernel (every
+// other shape with 16-byte accesses: the loads are requested together) and
+// sum_lstm_scalar_kernel (any size and alignment, element by element).
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 

@@ -128,11 +128,11 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
         r.sf[k] = C::load_stream(s_row + off[k]);
         r.zf[k] = kSharedZ ? r.zc[k] : C::load_stream(z_row + off[k]);
       }
-      // the cell comes straight from the previous step's launch and both outputs are read by the next
-      // kernels of the step, so these three accesses stay in the caches; the gates are touched once and stream
+      // (the previous cell and both outputs stream like the gates: a launch boundary writes the outputs back anyway,
+      // and streaming stores leave the CU earlier - measured on the staged kernel below)
       if constexpr (!kZeroCell) {
 #pragma unroll
-        for (int k = 0; k < K; ++k) r.pc[k] = C::load(pc_row + off[k]);
+        for (int k = 0; k < K; ++k) r.pc[k] = C::load_stream(pc_row + off[k]);
       }
     };
     auto input_gate = [&]() {
@@ -278,7 +278,7 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
         }
       }
       const C packed = C::template pack<T>(cell[k]);
-      if (live[k]) packed.store(oc_row + off[k]);
+      if (live[k]) packed.store_stream(oc_row + off[k]);
       packed.template unpack<T>(cell[k]);
     }
     float og[K][E];
@@ -318,7 +318,7 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
           const float rcp = __builtin_amdgcn_rcpf(u * v);
           st[j] = gelu_erf_given_t(x, rcp * v) * (rcp * u);
         }
-        if (live[k]) C::template pack<T>(st).store(os_row + off[k]);
+        if (live[k]) C::template pack<T>(st).store_stream(os_row + off[k]);
         continue;
       }
 #pragma unroll
@@ -333,7 +333,7 @@ __global__ __launch_bounds__(kMaxThreads) void sum_lstm_vec_kernel(const LstmPar
 #pragma unroll
         for (int j = 0; j < E; ++j) st[j] *= sigmoid_f(fmaf(p.alpha, g[j], a[j]));
       }
-      if (live[k]) C::template pack<T>(st).store(os_row + off[k]);
+      if (live[k]) C::template pack<T>(st).store_stream(os_row + off[k]);
     }
   };
 

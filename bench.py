@@ -1228,7 +1228,7 @@ def bench_argmax_variants(dev, steps):
 LSTM_VARIANTS = [
     (0, "loads c f pc i o, one row per 512-lane workgroup, output gate after the second row sum"),
     (1, "input gate loaded and consumed before forget gate and previous cell (c i f pc o)"),
-    (2, "output gate's sigmoid ahead of the second row sum (what shipped before the staged kernel)"),
+    (2, "output gate's sigmoid ahead of the second row sum (what the shapes outside the staged kernel take)"),
     (3, "input gate first + output gate's sigmoid ahead of the second row sum"),
     (4, "shared reciprocals: one for the forget and input gates, one for the state GELU and the output gate"),
     (8, "two rows per workgroup, second row's loads issued behind the first row's"),
@@ -1237,7 +1237,7 @@ LSTM_VARIANTS = [
     (24, "two chunks per lane and two rows per workgroup"),
     (34, "8-byte chunks, 1024 lanes per row (twice the waves, half the work each), early output gate"),
     (66, "the row's gates requested gate by gate: a workgroup barrier between the groups of requests"),
-    ("S0", "staged kernel, every chunk requested at once (the order and the accesses of the rows above)"),
+    ("S0", "staged kernel, every chunk requested at once, outputs and previous cell through the caches"),
     ("S1", "staged kernel: cell gate first; forget gate's s behind the first sum of squares; rest of the forget gate, "
            "previous cell and input gate behind the candidate's GELU; output gate behind the forget gate's part and "
            "consumed last"),

@@ -96,3 +96,22 @@ def test_random_configurations(ops):
         got = ops.speculator_argmax(base.to(DEV)[:, off:off + cols], vocab)
         want = torch.argmax(logits.float(), dim=-1).clamp_(0, vocab - 1)
         assert torch.equal(got.cpu(), want), f"configuration {it}: {dtype}, {rows} x {cols}, pad {pad}, offset {off}"
+
+
+@pytest.mark.parametrize("rows", [257, 300, 768, 769])   # 257-768 rows take the kernel whose waves move in step
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_row_counts_around_the_in_step_kernel(ops, rows, dtype):
+    """Launches of 257 to 768 rows keep the waves of a row in step, a 16-byte chunk at a time, behind a barrier whose
+    trip count has to be the same for every wave whatever the row length: rows shorter than one chunk per lane, rows
+    with a ragged last batch and an element-wise tail, ties everywhere, NaN and infinities, pitched rows."""
+    g = torch.Generator().manual_seed(900 + rows)
+    for cols, pad in ((8, 0), (1000, 8), (4100, 0), (8200, 24), (33001, 7)):
+        base = (torch.randint(0, 7, (rows, cols + pad), generator=g).float() - 3)
+        base[rows // 2, cols // 2] = float("nan")
+        base[rows - 1, 0] = float("inf")
+        base[0, cols - 1] = float("inf")
+        base[1] = -float("inf")
+        base = base.to(dtype)
+        got = ops.speculator_argmax(base.to(DEV)[:, :cols], cols)
+        want = torch.argmax(base[:, :cols].float(), dim=-1)
+        assert torch.equal(got.cpu(), want), f"{rows} x {cols} (+{pad}), {dtype}"

@@ -39,11 +39,11 @@ struct Fp4Params {
   int block_size;
 };
 
-// kGroups groups of 16 elements per lane, 256 groups apart, so that a wave's 64 lanes stay on 64 consecutive groups
+// kGroups groups of 16 elements per lane, kThreads groups apart, so that a wave's 64 lanes stay on 64 consecutive groups
 // (2 KiB of source, 512 bytes of packed cache) in each of them.  All of a lane's requests go out before the first
 // group is looked at.
-template <typename T, int kGroups>
-__global__ __launch_bounds__(256) void kv_write_fp4_kernel(const Fp4Params p) {
+template <typename T, int kGroups, int kThreads>
+__global__ __launch_bounds__(kThreads) void kv_write_fp4_kernel(const Fp4Params p) {
   const int groups_per_row = p.num_heads * p.groups_per_head;
   int64_t slot[kGroups];
   uint4 lo[kGroups], hi[kGroups];
@@ -52,7 +52,7 @@ __global__ __launch_bounds__(256) void kv_write_fp4_kernel(const Fp4Params p) {
   // so one round trip to memory serves both (a padding token throws its group away)
 #pragma unroll
   for (int u = 0; u < kGroups; ++u) {
-    idx[u] = ((int64_t)blockIdx.x * kGroups + u) * 256 + threadIdx.x;
+    idx[u] = ((int64_t)blockIdx.x * kGroups + u) * kThreads + threadIdx.x;
     const int64_t at = min(idx[u], p.total_groups - 1);   // lanes past the end read the last group and drop it
     const int64_t row = at / groups_per_row;              // token * 2 + (0 = K, 1 = V)
     const int in_row = (int)(at - row * groups_per_row);
@@ -168,26 +168,40 @@ extern "C" int arctic_reshape_and_cache_flash_fp4(
   p.total_groups = num_tokens * 2 * num_heads * p.groups_per_head;
   p.num_slots = num_blocks > 0 ? num_blocks * (int64_t)block_size : INT64_MAX;
   hipStream_t s = (hipStream_t)stream;
-  // groups per lane: ARCTIC_FP4_GROUPS in the measurement build
-  int per_lane = 1;
+  // One group per lane in workgroups of one wave: nothing is shared between lanes, and at 8192 tokens and beyond
+  // single-wave workgroups ran 1 to 1.5 % faster than 256-lane ones (equal below).  The measurement build also has
+  // other workgroup sizes (ARCTIC_FP4_LANES) and 2 or 4 groups per lane (ARCTIC_FP4_GROUPS); all measured slower.
+  int per_lane = 1, lanes = 64;
 #ifdef ARCTIC_TUNING
   if (const char *e = getenv("ARCTIC_FP4_GROUPS")) per_lane = atoi(e);
+  if (const char *e = getenv("ARCTIC_FP4_LANES")) lanes = atoi(e);
+  if (per_lane != 1) lanes = 256;
 #endif
-  const int64_t grid = (p.total_groups + 256 * per_lane - 1) / (256 * per_lane);
+  const int64_t per_workgroup = (int64_t)lanes * per_lane;
+  const int64_t grid = (p.total_groups + per_workgroup - 1) / per_workgroup;
   if (grid > 0x7fffffffLL) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: too many tokens", fn);
-#define ARCTIC_FP4_LAUNCH(G)                                                                             \
-  do {                                                                                                   \
-    if (dtype == ARCTIC_DTYPE_BF16)                                                                      \
-      hipLaunchKernelGGL((kv_write_fp4_kernel<BF16, G>), dim3((unsigned)grid), dim3(256), 0, s, p);      \
-    else                                                                                                 \
-      hipLaunchKernelGGL((kv_write_fp4_kernel<F16, G>), dim3((unsigned)grid), dim3(256), 0, s, p);       \
+#define ARCTIC_FP4_LAUNCH(G, LANES)                                                                          \
+  do {                                                                                                       \
+    if (dtype == ARCTIC_DTYPE_BF16)                                                                          \
+      hipLaunchKernelGGL((kv_write_fp4_kernel<BF16, G, LANES>), dim3((unsigned)grid), dim3(LANES), 0, s, p); \
+    else                                                                                                     \
+      hipLaunchKernelGGL((kv_write_fp4_kernel<F16, G, LANES>), dim3((unsigned)grid), dim3(LANES), 0, s, p);  \
   } while (0)
-  switch (per_lane) {
+  switch (per_workgroup) {
 #ifdef ARCTIC_TUNING
-    case 2: ARCTIC_FP4_LAUNCH(2); break;
-    case 4: ARCTIC_FP4_LAUNCH(4); break;
+    case 128: ARCTIC_FP4_LAUNCH(1, 128); break;
+    case 256: ARCTIC_FP4_LAUNCH(1, 256); break;
+    case 512:
+      if (per_lane == 2) ARCTIC_FP4_LAUNCH(2, 256);
+      else ARCTIC_FP4_LAUNCH(1, 512);
+      break;
+    case 1024:
+      if (per_lane == 4) ARCTIC_FP4_LAUNCH(4, 256);
+      else ARCTIC_FP4_LAUNCH(1, 1024);
+      break;
 #endif
-    default: ARCTIC_FP4_LAUNCH(1); break;
+    case 64: ARCTIC_FP4_LAUNCH(1, 64); break;
+    default: return fail(ARCTIC_ERR_UNSUPPORTED, "%s: no kernel built for %d lanes x %d groups", fn, lanes, per_lane);
   }
 #undef ARCTIC_FP4_LAUNCH
   return check_launch(fn);

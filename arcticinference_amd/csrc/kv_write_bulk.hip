@@ -659,7 +659,8 @@ static void launch_vec_shape(const BulkParams &p, const LayerTables &tab, int64_
       return;
     }
   }
-  // ARCTIC_BULK_SHAPE = 1: 512 lanes x 4 chunks, 2: 1024 x 2, 3: 1024 x 4, 4: 1024 x 1, 5: 512 x 2, 6: 256 x 2, 7: 256 x 1, 8: 512 x 1
+  // ARCTIC_BULK_SHAPE = 1: 512 lanes x 4 chunks, 2: 1024 x 2, 3: 1024 x 4, 4: 1024 x 1, 5: 512 x 2, 6: 256 x 2, 7: 256 x 1, 8: 512 x 1,
+  // 9: 64 x 4, 10: 64 x 8, 11: 128 x 4, 12: 128 x 8 (one- and two-wave workgroups: 2 to 25 % slower at 512 tokens)
   if constexpr (kSelect == kSelectNone) {
     const char *e = getenv("ARCTIC_BULK_SHAPE");
     const int shape = e ? atoi(e) : 0;
@@ -672,6 +673,10 @@ static void launch_vec_shape(const BulkParams &p, const LayerTables &tab, int64_
         case 6: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 256, 2, kSelectNone>), g, dim3(256), 0, s, p, tab); break;
         case 7: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 256, 1, kSelectNone>), g, dim3(256), 0, s, p, tab); break;
         case 8: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 512, 1, kSelectNone>), g, dim3(512), 0, s, p, tab); break;
+        case 9: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 64, 4, kSelectNone>), g, dim3(64), 0, s, p, tab); break;
+        case 10: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 64, 8, kSelectNone>), g, dim3(64), 0, s, p, tab); break;
+        case 11: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 128, 4, kSelectNone>), g, dim3(128), 0, s, p, tab); break;
+        case 12: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 128, 8, kSelectNone>), g, dim3(128), 0, s, p, tab); break;
         default: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 1024, 1, kSelectNone>), g, dim3(1024), 0, s, p, tab); break;
       }
       return;

@@ -311,6 +311,7 @@ def load_floor_kernels():
     lib.floor_lstm_traffic.argtypes = [vp, vp, vp, vp, vp, i64, i32, vp]
     lib.floor_lstm_traffic_staged.argtypes = [vp, vp, vp, vp, vp, i64, i32, vp]
     lib.floor_ln_traffic.argtypes = [vp, vp, i64, i32, vp]
+    lib.floor_fp4_traffic.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i32, vp]
     lib.floor_stream_resident.argtypes = [vp, vp, i32, i64, i32, i32, i32, i32, vp]
     lib.floor_stream.argtypes = [vp, i32, vp, i32, i64, i32, vp, vp]
     lib.floor_valu_rate.argtypes = [i32, i32, i32, vp, vp]
@@ -452,16 +453,29 @@ def bench_fp4(ops, dev, steps):
         for l in range(L):
             ops.reshape_and_cache_flash_fp4(keys[l], values[l], kc[l], vc[l], ks[l], vs[l], slots, "fp4", z, z)
 
-    for _ in range(3):
-        step()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        step()
-    warm_replays(graph.replay)
-    med = statistics.median(event_times_us(graph.replay, max(10, steps // 2))) / L
+    def per_layer(fn):
+        for _ in range(3):
+            fn()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fn()
+        warm_replays(graph.replay)
+        return statistics.median(event_times_us(graph.replay, max(10, steps // 2))) / L
+
+    med = per_layer(step)
     nbytes = T * (4 * H * D + 2 * (H * D // 2 + H * D // 16))
-    return {"us_per_layer_graph": round(med, 2), "bytes_per_layer": nbytes, "GBps": round(nbytes / med / 1e3, 1),
-            "hbm_frac": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
+    out = {"us_per_layer_graph": round(med, 2), "bytes_per_layer": nbytes, "GBps": round(nbytes / med / 1e3, 1),
+           "hbm_frac": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
+    floor = load_floor_kernels()
+    if floor is not None:   # the same loads and stores (both caches contiguous), nothing computed
+        def traffic():
+            st = torch.cuda.current_stream().cuda_stream
+            for l in range(L):
+                rc = floor.floor_fp4_traffic(keys[l].data_ptr(), values[l].data_ptr(), kc[l].data_ptr(), vc[l].data_ptr(),
+                                             ks[l].data_ptr(), vs[l].data_ptr(), slots.data_ptr(), T, H * D // 16, st)
+                assert rc == 0, rc
+        out["traffic_only_us_per_layer_graph"] = round(per_layer(traffic), 2)
+    return out
 
 
 def bench_row_gather(ops, dev, steps):

@@ -154,6 +154,30 @@ __global__ __launch_bounds__(1024) void resident_stream_kernel(const char *src, 
 
 // bytes_in of `src` (a multiple of loads x 16 KiB, at most 2^41) are read, half as many written, dealt over dst[0..ndst);
 // period_ticks = 0: no time slices, else 0 < read_ticks < period_ticks (ticks of 10 ns)
+// The traffic of the fp4 cache write and nothing else: one lane per group of 16 bf16 elements (the slot and two
+// 16-byte loads requested together, then 8 bytes of packed values and one scale byte stored at the slot's row of
+// contiguous caches).  `row_groups` = groups per token row (heads x head_size / 16); lanes walk a token's K row, then
+// its V row.
+__global__ __launch_bounds__(64) void fp4_traffic_kernel(const char *key, const char *value, char *key_cache,
+                                                         char *value_cache, char *key_scales, char *value_scales,
+                                                         const long long *slots, long long total_groups, int row_groups) {
+  const long long idx = (long long)blockIdx.x * 64 + threadIdx.x;
+  const long long at = idx < total_groups ? idx : total_groups - 1;
+  const long long row = at / row_groups;
+  const int in_row = (int)(at - row * row_groups);
+  const long long token = row >> 1;
+  const long long slot = slots[token];
+  const char *src = ((row & 1) ? value : key) + (token * row_groups + in_row) * 32;
+  const u32x4 lo = __builtin_nontemporal_load((const u32x4 *)src);
+  const u32x4 hi = __builtin_nontemporal_load((const u32x4 *)(src + 16));
+  __builtin_amdgcn_sched_barrier(0);
+  if (idx >= total_groups || slot < 0) return;
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  const u32x2 packed = {lo.x ^ hi.x ^ lo.z ^ hi.z, lo.y ^ hi.y ^ lo.w ^ hi.w};
+  __builtin_nontemporal_store(packed, (u32x2 *)(((row & 1) ? value_cache : key_cache) + (slot * row_groups + in_row) * 8));
+  ((row & 1) ? value_scales : key_scales)[slot * row_groups + in_row] = (char)(packed.x >> 7);
+}
+
 extern "C" int floor_stream_resident(const void *src, void *const *dst, int ndst, int64_t bytes_in, int loads,
                                      int workgroups, int period_ticks, int read_ticks, void *stream) {
   if (!src || !dst || ndst < 1 || ndst > 3 || (loads != 4 && loads != 8) || workgroups < 1 || workgroups > 65535 ||
@@ -279,6 +303,17 @@ extern "C" int floor_lstm_traffic(const void *s, const void *z, const void *pc, 
   hipLaunchKernelGGL(lstm_traffic_kernel, dim3((unsigned)rows), dim3((unsigned)((D / 8 + 63) & ~63)), 0,
                      (hipStream_t)stream, (const char *)s, (const char *)z, (const char *)pc, (char *)out_state,
                      (char *)out_cell, D);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+extern "C" int floor_fp4_traffic(const void *key, const void *value, void *key_cache, void *value_cache, void *key_scales,
+                                 void *value_scales, const void *slots, long long num_tokens, int row_groups, void *stream) {
+  if (num_tokens <= 0 || row_groups <= 0) return 1;
+  const long long total = num_tokens * 2 * row_groups;
+  if ((total + 63) / 64 > 0x7fffffffLL) return 1;
+  hipLaunchKernelGGL(fp4_traffic_kernel, dim3((unsigned)((total + 63) / 64)), dim3(64), 0, (hipStream_t)stream,
+                     (const char *)key, (const char *)value, (char *)key_cache, (char *)value_cache, (char *)key_scales,
+                     (char *)value_scales, (const long long *)slots, total, row_groups);
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 

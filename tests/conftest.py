@@ -10,6 +10,18 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # ARCTIC_TEST_SEED_SHIFT=k moves every `random.Random(seed)` of the tests to seed + k, so that the seeded sweeps
+    # (`-k random_configurations`) can be run over other configurations than the committed ones
+    shift = int(os.environ.get("ARCTIC_TEST_SEED_SHIFT", "0"))
+    if shift:
+        import random
+        base = random.Random
+
+        class Shifted(base):
+            def __init__(self, seed=None):
+                super().__init__(None if seed is None else seed + shift)
+
+        random.Random = Shifted
 
 
 @pytest.fixture(scope="session")

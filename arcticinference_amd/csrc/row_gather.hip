@@ -23,8 +23,8 @@
 namespace arctic {
 
 constexpr int kMaxGatherTensors = 8;
-// Lanes per workgroup.  Measured on swiftkv_select's five tensors (208 KiB per row): 512 rows 41.8 / 41.2 / 40.5 /
-// 40.9 / 43.3 us with 64 / 128 / 256 / 512 / 1024 lanes, 2048 rows 153.7 / 151.0 / 147.8 / 145.8 / 156.2 us.
+// Lanes per workgroup.  Measured on swiftkv_select's five tensors (208 KiB per row): 512 rows 39.0 / 38.7 / 38.5 /
+// 39.6 / 42.1 us with 64 / 128 / 256 / 512 / 1024 lanes, 2048 rows 140.2 / 140.5 / 140.5 / 139.3 / 153.2 us.
 constexpr int kGatherLanes = 256;
 constexpr int kGatherUnroll = 4;
 
@@ -33,7 +33,11 @@ struct GatherTable {
   char *dst[kMaxGatherTensors];
   int64_t src_stride[kMaxGatherTensors];   // bytes between rows
   int64_t dst_stride[kMaxGatherTensors];
-  int64_t first_unit[kMaxGatherTensors + 1];   // position of the tensor's first unit in the run
+  // Position of the tensor's first unit in the run and one past its last.  A tensor starts at a multiple of 8 units,
+  // so that workgroup boundaries inside wide rows fall on 128-byte lines of the row (a one-unit tensor such as the
+  // positions would otherwise shift every boundary behind it into the middle of a line).
+  int64_t first_unit[kMaxGatherTensors];
+  int64_t end_unit[kMaxGatherTensors];
   int unit_shift[kMaxGatherTensors];           // log2 of the unit size in bytes
   int count;
 };
@@ -84,7 +88,7 @@ __global__ __launch_bounds__(kGatherThreads) void row_gather_kernel(GatherTable 
     const int64_t dst_row = scatter ? idx : row;
     for (int t = 0; t < tab.count; ++t) {
       const int64_t lo = std::max(begin, tab.first_unit[t]);
-      const int64_t hi = std::min(end, tab.first_unit[t + 1]);
+      const int64_t hi = std::min(end, tab.end_unit[t]);
       if (lo >= hi) continue;
       const char *src = tab.src[t] + src_row * tab.src_stride[t];
       char *dst = tab.dst[t] + dst_row * tab.dst_stride[t];
@@ -148,10 +152,11 @@ extern "C" int arctic_gather_rows(int num_tensors, const void *const *src, void 
     shift = std::min(shift, alignment_shift((uint64_t)src_row_stride_bytes[t]));
     shift = std::min(shift, alignment_shift((uint64_t)dst_row_stride_bytes[t]));
     tab.unit_shift[c] = shift;
+    units = (units + 7) & ~(int64_t)7;
     tab.first_unit[c] = units;
     units += row_bytes[t] >> shift;
+    tab.end_unit[c] = units;
   }
-  tab.first_unit[tab.count] = units;
   if (units == 0) return ARCTIC_OK;
   int lanes = kGatherLanes;
 #ifdef ARCTIC_TUNING

@@ -1446,6 +1446,7 @@ ONLY = {
     "speculator_argmax_512x128256": lambda ops, dev, a: bench_argmax(ops, dev, a.steps),
     "fp4_write_8b_layer": lambda ops, dev, a: bench_fp4(ops, dev, a.steps),
     "bulk_write_and_select_decode_70b": lambda ops, dev, a: bench_bulk_select(ops, dev, a.steps),
+    "swiftkv_select_decode_70b": lambda ops, dev, a: bench_row_gather(ops, dev, a.steps),
     "bulk_fp8_70b_tp_sharded_heads_compact_pool": lambda ops, dev, a: bench_bulk_tp_heads(ops, dev, a.steps),
 }
 

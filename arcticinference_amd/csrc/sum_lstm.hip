@@ -9,8 +9,9 @@
 // across both RMS reductions, so HBM sees 9*D elements read and 2*D written per
 // row (the reference re-reads the cell gate and reads out_cell back: 12*D).
 // Sums are DPP wave reductions plus an LDS combine.  Three kernels:
-// sum_lstm_staged_kernel (the speculator's shapes: the nine loads are requested
-// in stages, between the stages of the arithmetic), sum_lstm_vec_kernel (every
+// sum_lstm_staged_kernel (the speculator's shapes, rows of a multiple of 512 up to
+// 8192 elements with all four vectors: the nine loads are requested in stages,
+// between the stages of the arithmetic, one chunk per lane), sum_lstm_vec_kernel (every
 // other shape with 16-byte accesses: the loads are requested together) and
 // sum_lstm_scalar_kernel (any size and alignment, element by element).
 #include <hip/hip_fp16.h>
@@ -384,8 +385,10 @@ struct LstmSchedule {
 using LstmShippedSchedule = LstmSchedule<2, 3, 7, 7, false, 2, true, true, 4>;
 
 // Same arithmetic, operation for operation, as sum_lstm_vec_kernel: results are bit-identical.
-template <typename T, bool kFastGelu, bool kSharedZ, bool kZeroCell, typename S = LstmShippedSchedule, bool kTrace = false>
-__global__ __launch_bounds__(512) void sum_lstm_staged_kernel(const LstmParams p) {
+// kMaxLanes: 512 for rows of up to 4096 elements, 1024 (half the registers per lane) for rows of up to 8192.
+template <typename T, bool kFastGelu, bool kSharedZ, bool kZeroCell, typename S = LstmShippedSchedule, bool kTrace = false,
+          int kMaxLanes = 512>
+__global__ __launch_bounds__(kMaxLanes) void sum_lstm_staged_kernel(const LstmParams p) {
   __shared__ float slots_cpre[16];
   __shared__ float slots_cnew[16];
   constexpr int E = 8;
@@ -683,7 +686,16 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
     }
 #endif
     constexpr int kShipped = kLstmEarlyOutputGate;   // measured best of the variants that change no result bit
-    if (cpt == 1 && all && !p.prev_cell)   // the speculator's shapes: requests in stages
+    const bool wide = chunks > 512 && chunks <= 1024 && chunks % 64 == 0 && p.w_cell && p.b_cell && p.w_state && p.b_state;
+    // rows of 4096 to 8192 elements: the staged kernel with one chunk per lane of up to 1024 (512 rows: 12.0 / 13.9 /
+    // 17.9 us at 5120 / 6144 / 8192 elements against 17.6 / 19.9 / 22.5 us with two chunks per lane in the kernel below)
+    if (wide && !p.prev_cell)
+      hipLaunchKernelGGL((sum_lstm_staged_kernel<T, kFastGelu, kSharedZ, true, LstmShippedSchedule, false, 1024>), grid,
+                         dim3(chunks), 0, s, p);
+    else if (wide)
+      hipLaunchKernelGGL((sum_lstm_staged_kernel<T, kFastGelu, kSharedZ, false, LstmShippedSchedule, false, 1024>), grid,
+                         dim3(chunks), 0, s, p);
+    else if (cpt == 1 && all && !p.prev_cell)   // the speculator's shapes: requests in stages
       hipLaunchKernelGGL((sum_lstm_staged_kernel<T, kFastGelu, kSharedZ, true>), grid, dim3(threads), 0, s, p);
     else if (cpt == 1 && all)
       hipLaunchKernelGGL((sum_lstm_staged_kernel<T, kFastGelu, kSharedZ, false>), grid, dim3(threads), 0, s, p);

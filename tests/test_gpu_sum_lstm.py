@@ -282,14 +282,16 @@ def test_saturated_gates_zero_rows_and_extreme_magnitudes(ops, dtype, D):
     assert torch.isfinite(want_s.float()).all() and torch.isfinite(want_c.float()).all()
 
 
-@pytest.mark.parametrize("D", [512, 1024, 1536, 2048, 3072, 4096])
+@pytest.mark.parametrize("D", [512, 1024, 1536, 2048, 3072, 4096, 4608, 5120, 6144, 8192])
 @pytest.mark.parametrize("rows", [1, 5, 300])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_staged_kernel_shapes(ops, D, rows, dtype):
-    """Rows of a multiple of 512 elements with all four vectors take the kernel that requests a row in stages
-    (every lane owns one 16-byte chunk): against the oracle with and without a previous cell, with pitched rows and
-    the tanh GELU, and bit for bit against the general kernel, which the same row takes as soon as one vector is
-    missing (an absent scale acts as 1, an absent shift as 0, so ones and zeros in their place change no bit)."""
+    """Rows of a multiple of 512 elements, up to 8192, with all four vectors take the kernel that requests a row in
+    stages (every lane owns one 16-byte chunk): against the oracle with and without a previous cell, with pitched rows
+    and the tanh GELU, and bit for bit against the general kernel, which the same row takes as soon as one vector is
+    missing (an absent scale acts as 1, an absent shift as 0, so ones and zeros in their place change no bit).  Beyond
+    4096 elements the general kernel gives a lane two chunks, so its row sums add up in another order: there the two
+    are compared within the tolerance."""
     pad = 8 if rows > 1 else 0   # pitches stay multiples of 16 bytes
     c = make_lstm_case(rows=rows, D=D, dtype=dtype, seed=900 + D // 512 + rows, pad4=pad, padD=pad)
     for fast in (False, True):
@@ -298,10 +300,17 @@ def test_staged_kernel_shapes(ops, D, rows, dtype):
     ones, zeros = torch.ones(D, dtype=dtype, device=DEV), torch.zeros(D, dtype=dtype, device=DEV)
     tail = (0.35, 1e-6, 1e-5, False)
     for cell in (d["prev_cell"], None):
+        def same(a, b):
+            for x, y in zip(a, b):
+                if D <= 4096:
+                    assert torch.equal(x, y)
+                else:
+                    assert_close(x, y, RTOL, ATOL, "staged against general")
+
         staged = ops.sum_lstm(d["states"], d["z4"], cell, ones, zeros, d["w_state"], d["b_state"], *tail)
         general = ops.sum_lstm(d["states"], d["z4"], cell, None, None, d["w_state"], d["b_state"], *tail)
-        assert torch.equal(staged[0], general[0]) and torch.equal(staged[1], general[1])
+        same(staged, general)
         z = d["z4"][:, :D].contiguous()
         staged = ops.sum_lstm_shared_z(d["states"], z, cell, d["w_cell"], d["b_cell"], ones, zeros, *tail)
         general = ops.sum_lstm_shared_z(d["states"], z, cell, d["w_cell"], d["b_cell"], None, None, *tail)
-        assert torch.equal(staged[0], general[0]) and torch.equal(staged[1], general[1])
+        same(staged, general)

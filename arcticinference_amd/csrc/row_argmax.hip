@@ -103,8 +103,9 @@ struct HalfElem {
   }
 };
 
-// kVec: rows are 16-byte aligned, so the body of a row is read in 16-byte chunks; the elements behind
-// the last whole chunk (and everything when !kVec) are read one by one.
+// kVec: the body of a row, from its first 16-byte boundary on, is read in 16-byte chunks; the elements in front of
+// that boundary (a row pitch that is no multiple of 16 bytes puts every row somewhere else), those behind the last
+// whole chunk, and everything when !kVec (a pointer that is not even element-aligned) are read one by one.
 // kUnroll chunks per lane form a batch; kPipelined: the next batch is requested before the current one is looked at;
 // kStaggered: the odd waves take half a batch on its own first, so that neighbouring waves are half a batch apart;
 // kLockstep: a workgroup barrier (no memory wait) behind every batch's requests, so that every wave of the row has
@@ -121,7 +122,9 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
   // once, after the loop.  Apart from that the first NaN: a chunk's sum is NaN only if the chunk holds a NaN (or
   // infinities of both signs), so the per-element NaN test runs almost never.
   constexpr int P = Elem::kPerChunk;
-  const int chunks = kVec ? cols / P : 0;
+  const int head = kVec ? min(cols, (int)((0 - (uintptr_t)row) & 15) / (16 / P)) : 0;   // elements in front of the body
+  const int chunks = kVec ? (cols - head) / P : 0;
+  const char *body = row + (int64_t)head * (16 / P);
   float best = -__builtin_inff();
   int best_at = -1;
   int nan_at = 0x7fffffff;
@@ -131,6 +134,13 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
       best_at = i;
     }
   };
+  // a lane's candidates come in the order of their indices (head, chunks, tail), so that ">" keeps the first of equals
+  if ((int)threadIdx.x < head) {
+    const float v = Elem::one(row, threadIdx.x);
+    best_at = threadIdx.x;   // stands for the lane even when it is -inf: a row of -inf must answer 0
+    best = v == v ? v : best;
+    if (v != v) nan_at = threadIdx.x;
+  }
   int done = 0;
   if (kVec) {
     int best_chunk = -1;
@@ -140,7 +150,7 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         const int c = c0 + u * blockDim.x;
-        if (c < chunks) raw[u] = load16_stream(row + (int64_t)c * 16);
+        if (c < chunks) raw[u] = load16_stream(body + (int64_t)c * 16);
       }
     };
     auto look_at_chunk = [&](int c, const uint4 &words) {
@@ -158,7 +168,7 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
       if (sum != sum) {
 #pragma unroll
         for (int j = 0; j < P; ++j)
-          if (f[j] != f[j]) nan_at = min(nan_at, c * P + j);
+          if (f[j] != f[j]) nan_at = min(nan_at, head + c * P + j);
       }
     };
     auto look_at = [&](int c0, const uint4 (&raw)[kUnroll]) {
@@ -199,7 +209,7 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
 #pragma unroll
           for (int u = 0; u < kLead; ++u) {
             const int c = c0 + u * (int)blockDim.x;
-            if (c < chunks) lead[u] = load16_stream(row + (int64_t)c * 16);
+            if (c < chunks) lead[u] = load16_stream(body + (int64_t)c * 16);
           }
 #pragma unroll
           for (int u = 0; u < kLead; ++u) {
@@ -215,7 +225,7 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
         look_at(c0, raw);
       }
     }
-    done = chunks * P;
+    done = head + chunks * P;
     if (best_chunk >= 0) {
       // the first element of that chunk that equals the lane's maximum
       float f[8];
@@ -224,9 +234,9 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
 #pragma unroll
       for (int k = P - 2; k >= 0; --k)
         if (f[k] == best) j = k;
-      best_at = best_chunk * P + j;
-    } else if ((int)threadIdx.x < chunks) {
-      best_at = (int)threadIdx.x * P;   // nothing above -inf here: the lane's first element stands for its chunks
+      best_at = head + best_chunk * P + j;
+    } else if (best_at < 0 && (int)threadIdx.x < chunks) {
+      best_at = head + (int)threadIdx.x * P;   // nothing above -inf here: the lane's first element stands for its chunks
     }
   }
   // (a lane without chunks takes its first tail element, if it has one, the same way: a row of -inf must answer 0)
@@ -272,7 +282,7 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
   if (cols > (1 << 30) || !pitch_ok(row_stride, rows, es))
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: more than 2^30 columns, or a row pitch out of range", fn);
   const int64_t stride_bytes = row_stride * es;
-  const bool vec = ((uintptr_t)logits % 16 == 0) && (stride_bytes % 16 == 0 || rows == 1);
+  const bool vec = (uintptr_t)logits % es == 0;   // rows may start anywhere between two 16-byte boundaries
   const int per_chunk = 16 / es;
   int threads = (int)std::min<int64_t>(1024, std::max<int64_t>(64, ((cols / per_chunk / 4 + 63) / 64) * 64));
   hipStream_t s = (hipStream_t)stream;

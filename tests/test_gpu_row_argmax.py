@@ -63,6 +63,32 @@ def test_clamp_and_row_pitch(ops):
     assert ops.speculator_argmax(padded, 1000).tolist() == [999] * 4
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_rows_that_start_between_16_byte_boundaries(ops, dtype):
+    """A contiguous [rows, vocab] with an odd vocabulary (GPT-2's 50257) puts every row at another offset from a
+    16-byte boundary: the elements in front of the first boundary, the 16-byte chunks and the elements behind the
+    last chunk are three stretches of one row, and the lowest index among equal values may lie in any of them."""
+    rows, cols = 24, 50257
+    g = torch.Generator().manual_seed(8)
+    x = (torch.randint(0, 9, (rows, cols), generator=g).float() - 4).to(dtype)      # ties everywhere
+    x[1, :] = -float("inf")                        # answers 0, which lies in front of row 1's first boundary
+    x[2, 0] = 50.0                                 # the very first element wins
+    x[3, 1], x[3, 9000] = 50.0, 50.0               # equal values in front of the boundary and in a chunk
+    x[4, cols - 1], x[4, 30000] = 50.0, 50.0       # ... in a chunk and behind the last chunk
+    x[5, cols - 1] = 50.0                          # the very last element wins
+    x[6, 2], x[6, 40000] = float("nan"), float("nan")   # the first NaN lies in front of the boundary
+    x[7, 3], x[7, 4] = float("inf"), float("nan")
+    d = x.to(DEV)
+    assert d.data_ptr() % 16 == 0 and (cols * x.element_size()) % 16 != 0
+    got = ops.speculator_argmax(d, cols)
+    assert torch.equal(got.cpu(), reference(x, cols))
+    assert got[[1, 2, 3, 4, 5, 6, 7]].tolist() == [0, 0, 1, 30000, cols - 1, 2, 4]
+    # a view that starts one element into such a buffer, and one row alone
+    view = d[:, 1:]
+    assert torch.equal(ops.speculator_argmax(view, cols - 1).cpu(), reference(x[:, 1:], cols - 1))
+    assert torch.equal(ops.speculator_argmax(d[5:6, 3:], cols).cpu(), reference(x[5:6, 3:], cols))
+
+
 def test_empty_and_errors(ops):
     assert ops.speculator_argmax(torch.empty(0, 64, device=DEV), 64).shape == (0,)
     with pytest.raises(RuntimeError, match="non-empty last dimension"):
@@ -75,7 +101,7 @@ def test_empty_and_errors(ops):
 
 def test_random_configurations(ops):
     """Seeded sweep over types, row counts, row lengths around the chunk and workgroup sizes, row pitches, start
-    offsets (unaligned rows take the element-wise path), value ranges with many ties, and sprinkled NaN / inf."""
+    offsets (rows that start between two 16-byte boundaries read their first elements one by one), value ranges with many ties, and sprinkled NaN / inf."""
     import random
     rnd = random.Random(13)
     for it in range(60):

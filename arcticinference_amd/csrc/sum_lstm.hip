@@ -9,9 +9,9 @@
 // across both RMS reductions, so HBM sees 9*D elements read and 2*D written per
 // row (the reference re-reads the cell gate and reads out_cell back: 12*D).
 // Sums are DPP wave reductions plus an LDS combine.  Three kernels:
-// sum_lstm_staged_kernel (the speculator's shapes, rows of a multiple of 512 up to
-// 8192 elements with all four vectors: the nine loads are requested in stages,
-// between the stages of the arithmetic, one chunk per lane), sum_lstm_vec_kernel (every
+// sum_lstm_staged_kernel (the speculator's shapes, rows of up to 8192 elements
+// with all four vectors: the nine loads are requested in stages, between the
+// stages of the arithmetic, one chunk per lane), sum_lstm_vec_kernel (every
 // other shape with 16-byte accesses: the loads are requested together) and
 // sum_lstm_scalar_kernel (any size and alignment, element by element).
 #include <hip/hip_fp16.h>
@@ -386,8 +386,10 @@ using LstmShippedSchedule = LstmSchedule<2, 3, 7, 7, false, 2, true, true, 4>;
 
 // Same arithmetic, operation for operation, as sum_lstm_vec_kernel: results are bit-identical.
 // kMaxLanes: 512 for rows of up to 4096 elements, 1024 (half the registers per lane) for rows of up to 8192.
+// kRagged: the row's chunks do not fill the last wave; the lanes behind the last chunk run along on that chunk (the
+// barriers need every wave), add nothing to the row sums and store nothing.
 template <typename T, bool kFastGelu, bool kSharedZ, bool kZeroCell, typename S = LstmShippedSchedule, bool kTrace = false,
-          int kMaxLanes = 512>
+          int kMaxLanes = 512, bool kRagged = false>
 __global__ __launch_bounds__(kMaxLanes) void sum_lstm_staged_kernel(const LstmParams p) {
   __shared__ float slots_cpre[16];
   __shared__ float slots_cnew[16];
@@ -395,7 +397,8 @@ __global__ __launch_bounds__(kMaxLanes) void sum_lstm_staged_kernel(const LstmPa
   using C = Chunk<E>;
   using std::integral_constant;
   const int64_t row = blockIdx.x;
-  const int64_t off = (int64_t)threadIdx.x * C::kBytes;
+  const bool active = !kRagged || (int)threadIdx.x < p.D / E;
+  const int64_t off = (int64_t)(kRagged ? min((int)threadIdx.x, p.D / E - 1) : (int)threadIdx.x) * C::kBytes;
   const int64_t gate_bytes = (int64_t)p.D * 2;
   // measurement build: the constant-rate clock (100 MHz) at eight points of a wave's life, written by its first lane
   auto stamp = [&](int k) {
@@ -468,7 +471,7 @@ __global__ __launch_bounds__(kMaxLanes) void sum_lstm_staged_kernel(const LstmPa
   stamp(2);   // the cell gate is in, its squares are summed
   request_vectors(2);
   request(integral_constant<int, S::kAhead0>(), integral_constant<int, S::kAhead1>());
-  const float inv_cpre = rsqrtf(block_sum(ss, slots_cpre) * p.inv_D + p.eps_cell);
+  const float inv_cpre = rsqrtf(block_sum(active ? ss : 0.f, slots_cpre) * p.inv_D + p.eps_cell);
   stamp(3);   // first row sum known
   {
     float w[E], sh[E];
@@ -502,8 +505,10 @@ __global__ __launch_bounds__(kMaxLanes) void sum_lstm_staged_kernel(const LstmPa
   }
   {
     const C packed = C::template pack<T>(cell);
-    if constexpr (S::kStreamOutputs) packed.store_stream(oc_row);
-    else packed.store(oc_row);
+    if (active) {
+      if constexpr (S::kStreamOutputs) packed.store_stream(oc_row);
+      else packed.store(oc_row);
+    }
     packed.template unpack<T>(cell);   // the state phase sees the rounded cell (:163,174)
   }
   stamp(4);   // forget gate, previous cell and input gate are in; the new cell is stored
@@ -516,7 +521,7 @@ __global__ __launch_bounds__(kMaxLanes) void sum_lstm_staged_kernel(const LstmPa
     for (int j = 0; j < E; ++j) og[j] = sigmoid_f(fmaf(p.alpha, b[j], a[j]));
     __builtin_amdgcn_sched_barrier(0);
   }
-  const float inv_cnew = rsqrtf(block_sum(ss, slots_cnew) * p.inv_D + p.eps_state);
+  const float inv_cnew = rsqrtf(block_sum(active ? ss : 0.f, slots_cnew) * p.inv_D + p.eps_state);
   stamp(5);   // second row sum known
 
   // phase 3: state = gelu(rmsnorm(rounded cell)) * sigmoid(pre_o) (reference :160-190)
@@ -539,8 +544,10 @@ __global__ __launch_bounds__(kMaxLanes) void sum_lstm_staged_kernel(const LstmPa
 #pragma unroll
     for (int j = 0; j < E; ++j) st[j] *= sigmoid_f(fmaf(p.alpha, b[j], a[j]));
   }
-  if constexpr (S::kStreamOutputs) C::template pack<T>(st).store_stream(os_row);
-  else C::template pack<T>(st).store(os_row);
+  if (active) {
+    if constexpr (S::kStreamOutputs) C::template pack<T>(st).store_stream(os_row);
+    else C::template pack<T>(st).store(os_row);
+  }
   stamp(7);   // state stored
 }
 
@@ -634,6 +641,7 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
     int threads = (chunks + cpt - 1) / cpt;
     threads = std::max(64, (threads + 63) & ~63);
     const bool all = p.w_cell && p.b_cell && p.w_state && p.b_state && threads * cpt == chunks;
+    (void)all;   // (the measurement build's variants below ask for it)
 #ifdef ARCTIC_TUNING
     if (cpt == 1 && all && threads % 128 == 0 && p.prev_cell) {
       if (const char *st = getenv("ARCTIC_LSTM_STAGED")) {
@@ -686,19 +694,29 @@ static void launch_lstm(const LstmParams &p, int64_t rows, hipStream_t s) {
     }
 #endif
     constexpr int kShipped = kLstmEarlyOutputGate;   // measured best of the variants that change no result bit
-    const bool wide = chunks > 512 && chunks <= 1024 && chunks % 64 == 0 && p.w_cell && p.b_cell && p.w_state && p.b_state;
-    // rows of 4096 to 8192 elements: the staged kernel with one chunk per lane of up to 1024 (512 rows: 12.0 / 13.9 /
-    // 17.9 us at 5120 / 6144 / 8192 elements against 17.6 / 19.9 / 22.5 us with two chunks per lane in the kernel below)
-    if (wide && !p.prev_cell)
-      hipLaunchKernelGGL((sum_lstm_staged_kernel<T, kFastGelu, kSharedZ, true, LstmShippedSchedule, false, 1024>), grid,
-                         dim3(chunks), 0, s, p);
-    else if (wide)
-      hipLaunchKernelGGL((sum_lstm_staged_kernel<T, kFastGelu, kSharedZ, false, LstmShippedSchedule, false, 1024>), grid,
-                         dim3(chunks), 0, s, p);
-    else if (cpt == 1 && all && !p.prev_cell)   // the speculator's shapes: requests in stages
-      hipLaunchKernelGGL((sum_lstm_staged_kernel<T, kFastGelu, kSharedZ, true>), grid, dim3(threads), 0, s, p);
-    else if (cpt == 1 && all)
-      hipLaunchKernelGGL((sum_lstm_staged_kernel<T, kFastGelu, kSharedZ, false>), grid, dim3(threads), 0, s, p);
+    // All four vectors given and a row of up to 8192 elements: the staged kernel, one chunk per lane (512 rows of
+    // 5120 / 6144 / 8192 elements: 12.0 / 13.9 / 17.9 us against 17.6 / 19.9 / 22.5 us with two chunks per lane in the
+    // kernel below), with idle lanes in the last wave when the row is no multiple of 512 elements.
+    const bool staged = chunks <= 1024 && p.w_cell && p.b_cell && p.w_state && p.b_state;
+    const int lanes = (chunks + 63) & ~63;
+#define ARCTIC_LSTM_STAGED_LAUNCH(ZERO, MAX_LANES, RAGGED)                                                           \
+  hipLaunchKernelGGL((sum_lstm_staged_kernel<T, kFastGelu, kSharedZ, ZERO, LstmShippedSchedule, false, MAX_LANES, RAGGED>), \
+                     grid, dim3(lanes), 0, s, p)
+    if (staged) {
+      const bool zero = !p.prev_cell, ragged = lanes != chunks;
+      if (chunks <= 512) {
+        if (zero && ragged) ARCTIC_LSTM_STAGED_LAUNCH(true, 512, true);
+        else if (zero) ARCTIC_LSTM_STAGED_LAUNCH(true, 512, false);
+        else if (ragged) ARCTIC_LSTM_STAGED_LAUNCH(false, 512, true);
+        else ARCTIC_LSTM_STAGED_LAUNCH(false, 512, false);
+      } else {
+        if (zero && ragged) ARCTIC_LSTM_STAGED_LAUNCH(true, 1024, true);
+        else if (zero) ARCTIC_LSTM_STAGED_LAUNCH(true, 1024, false);
+        else if (ragged) ARCTIC_LSTM_STAGED_LAUNCH(false, 1024, true);
+        else ARCTIC_LSTM_STAGED_LAUNCH(false, 1024, false);
+      }
+    }
+#undef ARCTIC_LSTM_STAGED_LAUNCH
     else if (cpt == 1)
       hipLaunchKernelGGL((sum_lstm_vec_kernel<T, 8, 1, kFastGelu, 512, kSharedZ, false, 1, kShipped>), grid, dim3(threads), 0, s, p);
     else

@@ -282,18 +282,18 @@ def test_saturated_gates_zero_rows_and_extreme_magnitudes(ops, dtype, D):
     assert torch.isfinite(want_s.float()).all() and torch.isfinite(want_c.float()).all()
 
 
-@pytest.mark.parametrize("D", [512, 1024, 1536, 2048, 3072, 4096, 4608, 5120, 6144, 8192])
+@pytest.mark.parametrize("D", [512, 1000, 1024, 1536, 2048, 2880, 3072, 4000, 4096, 4608, 5000, 5120, 6144, 8192])
 @pytest.mark.parametrize("rows", [1, 5, 300])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_staged_kernel_shapes(ops, D, rows, dtype):
-    """Rows of a multiple of 512 elements, up to 8192, with all four vectors take the kernel that requests a row in
-    stages (every lane owns one 16-byte chunk): against the oracle with and without a previous cell, with pitched rows
-    and the tanh GELU, and bit for bit against the general kernel, which the same row takes as soon as one vector is
-    missing (an absent scale acts as 1, an absent shift as 0, so ones and zeros in their place change no bit).  Beyond
-    4096 elements the general kernel gives a lane two chunks, so its row sums add up in another order: there the two
-    are compared within the tolerance."""
+    """Rows of up to 8192 elements with all four vectors take the kernel that requests a row in stages (one 16-byte
+    chunk per lane; rows that are no multiple of 512 elements leave lanes of the last wave idle): against the oracle
+    with and without a previous cell, with pitched rows and the tanh GELU, and bit for bit against the general kernel,
+    which the same row takes as soon as one vector is missing (an absent scale acts as 1, an absent shift as 0, so
+    ones and zeros in their place change no bit).  Beyond 4096 elements the general kernel gives a lane two chunks, so
+    its row sums add up in another order: there the two are compared within the tolerance."""
     pad = 8 if rows > 1 else 0   # pitches stay multiples of 16 bytes
-    c = make_lstm_case(rows=rows, D=D, dtype=dtype, seed=900 + D // 512 + rows, pad4=pad, padD=pad)
+    c = make_lstm_case(rows=rows, D=D, dtype=dtype, seed=900 + D // 8 + rows, pad4=pad, padD=pad)
     for fast in (False, True):
         run(ops, c, alpha=0.35, fast=fast)
     d = {k: dev(v) for k, v in c.items()}

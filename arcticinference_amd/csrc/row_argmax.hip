@@ -111,8 +111,9 @@ struct HalfElem {
 // kLockstep: a workgroup barrier (no memory wait) behind every batch's requests, so that every wave of the row has
 // asked for batch k before any wave asks for batch k + 1 (a CU serves its oldest wave first: without the barrier the
 // oldest wave runs through all its batches before the youngest gets its first one in).
+// kHead: rows may start between two 16-byte boundaries (without it the host has checked that none does).
 template <typename Elem, bool kVec, int kUnroll = 4, bool kPipelined = false, bool kStaggered = false,
-          bool kLockstep = false>
+          bool kLockstep = false, bool kHead = false>
 __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ out, const char *__restrict__ in,
                                                           int64_t row_stride_bytes, int cols, int64_t max_index) {
   __shared__ uint64_t wave_key[16];
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
   // once, after the loop.  Apart from that the first NaN: a chunk's sum is NaN only if the chunk holds a NaN (or
   // infinities of both signs), so the per-element NaN test runs almost never.
   constexpr int P = Elem::kPerChunk;
-  const int head = kVec ? min(cols, (int)((0 - (uintptr_t)row) & 15) / (16 / P)) : 0;   // elements in front of the body
+  const int head = kVec && kHead ? min(cols, (int)((0 - (uintptr_t)row) & 15) / (16 / P)) : 0;   // elements in front of the body
   const int chunks = kVec ? (cols - head) / P : 0;
   const char *body = row + (int64_t)head * (16 / P);
   float best = -__builtin_inff();
@@ -283,6 +284,7 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: more than 2^30 columns, or a row pitch out of range", fn);
   const int64_t stride_bytes = row_stride * es;
   const bool vec = (uintptr_t)logits % es == 0;   // rows may start anywhere between two 16-byte boundaries
+  const bool aligned_rows = (uintptr_t)logits % 16 == 0 && (stride_bytes % 16 == 0 || rows == 1);
   const int per_chunk = 16 / es;
   int threads = (int)std::min<int64_t>(1024, std::max<int64_t>(64, ((cols / per_chunk / 4 + 63) / 64) * 64));
   hipStream_t s = (hipStream_t)stream;
@@ -297,6 +299,10 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
 #define ARCTIC_ARGMAX_VEC(ELEM)                                                                                          \
   do {                                                                                                                   \
     const dim3 b((unsigned)threads);                                                                                     \
+    if (!aligned_rows) { /* the variants are built for aligned rows */                                                   \
+      hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false, false, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); \
+      break;                                                                                                             \
+    }                                                                                                                    \
     switch (variant) {                                                                                                   \
       case 1: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
       case 2: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 8, false>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
@@ -319,7 +325,13 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
   const bool lockstep = rows > 256 && rows <= 768;
 #define ARCTIC_ARGMAX_VEC(ELEM)                                                                                   \
   do {                                                                                                            \
-    if (lockstep)                                                                                                 \
+    if (!aligned_rows && lockstep)                                                                                \
+      hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 1, false, false, true, true>), grid, block, 0, s, out,    \
+                         (const char *)logits, stride_bytes, cols, max_index);                                    \
+    else if (!aligned_rows)                                                                                       \
+      hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false, false, false, true>), grid, block, 0, s, out,   \
+                         (const char *)logits, stride_bytes, cols, max_index);                                    \
+    else if (lockstep)                                                                                            \
       hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 1, false, false, true>), grid, block, 0, s, out,          \
                          (const char *)logits, stride_bytes, cols, max_index);                                    \
     else                                                                                                          \

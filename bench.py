@@ -855,6 +855,63 @@ def bench_lstm_rows(ops, dev, steps):
     return out
 
 
+def bench_lstm_widths(ops, dev, steps):
+    """sum_lstm at 512 rows against the row width: the kernel that requests a row in stages (all four scale / shift
+    vectors given, rows of up to 8192 elements, spare lanes in the last wave when the width is no multiple of 512)
+    next to the general kernel, which the same call takes when a vector is missing (here: the cell norm's pair)."""
+    T = 512
+    g = torch.Generator(device=dev).manual_seed(9)
+    rn = lambda *s: torch.randn(*s, generator=g, device=dev).to(torch.bfloat16)
+    out = {}
+    for Hd in (2048, 2880, 4000, 4096, 5120, 6144, 8192, 12288):
+        per_call = 22 * Hd * T
+        sets = max(8, -(-300 * 2 ** 20 // per_call))
+        S, Z, C = [rn(T, 4 * Hd) for _ in range(sets)], [rn(T, 4 * Hd) for _ in range(sets)], [rn(T, Hd) for _ in range(sets)]
+        w = [rn(Hd) for _ in range(4)]
+        row = {}
+        for name, cell_pair in (("all_four_vectors", (w[0], w[1])), ("without_the_cell_norm_vectors", (None, None))):
+            def run():
+                for i in range(sets):
+                    ops.sum_lstm(S[i], Z[i], C[i], cell_pair[0], cell_pair[1], w[2], w[3], 23.07, 1e-6, 1e-6, False)
+            run()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                run()
+            warm_replays(graph.replay)
+            us = statistics.median(event_times_us(graph.replay, max(10, steps // 2))) / sets
+            row[name] = {"us_per_call_graph": round(us, 2), "hbm_frac": round(per_call / us / 1e3 / HBM_PEAK_GBS, 4)}
+            del graph
+        out[f"{Hd}_wide"] = row
+        del S, Z, C
+    return out
+
+
+def bench_argmax_shapes(ops, dev, steps):
+    """speculator_argmax over vocabulary sizes (512 rows; 50257 and 128257 put every row at another offset from a
+    16-byte boundary) and over small batches (128256 logits per row), bf16, enough rotating sets to read from HBM."""
+    g = torch.Generator(device=dev).manual_seed(10)
+    out = {}
+    for T, V in ((512, 32000), (512, 50257), (512, 65536), (512, 128257), (512, 151936), (512, 262144),
+                 (1, 128256), (8, 128256), (64, 128256), (128, 128256), (256, 128256)):
+        sets = max(3, min(64, (400 << 20) // (T * V * 2) + 1))
+        logits = [torch.randn(T, V, generator=g, device=dev).to(torch.bfloat16) for _ in range(sets)]
+
+        def run():
+            for x in logits:
+                ops.speculator_argmax(x, V)
+        run()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            run()
+        warm_replays(graph.replay)
+        us = statistics.median(event_times_us(graph.replay, max(10, steps // 2))) / sets
+        out[f"{T}_rows_x_{V}"] = {"us_per_call_graph": round(us, 2), "hbm_frac": round(2 * T * V / us / 1e3 / HBM_PEAK_GBS, 4)}
+        del logits, graph
+    return out
+
+
 def bench_speculator_round_glue(ops, dev, steps):
     """Everything but the matrix products of one proposal round of the LSTM speculator (three heads, 512 rows,
     width 4096, 128256-entry vocabulary; arctic_speculator.py:733-862): ln0 / sqrt 2, then per head the embedding
@@ -1442,6 +1499,8 @@ ONLY = {
     "decode_mix": lambda ops, dev, a: bench_decode_mix(ops, dev, a.steps),
     "speculator": lambda ops, dev, a: bench_speculator(ops, dev, a.steps, a.warmup),
     "sum_lstm_rows_sweep": lambda ops, dev, a: bench_lstm_rows(ops, dev, a.steps),
+    "sum_lstm_width_sweep": lambda ops, dev, a: bench_lstm_widths(ops, dev, a.steps),
+    "speculator_argmax_shapes": lambda ops, dev, a: bench_argmax_shapes(ops, dev, a.steps),
     "bulk_auto_bf16_cache": lambda ops, dev, a: bench_bulk_auto(ops, dev, a.steps),
     "speculator_argmax_512x128256": lambda ops, dev, a: bench_argmax(ops, dev, a.steps),
     "fp4_write_8b_layer": lambda ops, dev, a: bench_fp4(ops, dev, a.steps),

@@ -1,4 +1,5 @@
-"""The speculator operators, the argmax, the row gather and the fp4 cache write on tensors of more than 2^32 bytes:
+"""The speculator operators, the argmax, the row gather, the fp4 cache write and the bulk write's source on tensors of
+more than 2^32 bytes:
 row offsets that no 32-bit product holds (the reference indexes rows with int64 throughout, e.g.
 csrc/custom_ops/sum_lstm.cu:100-116, csrc/custom_ops/speculator_ln.cu:44-60).  The buffers are too large to bring to
 the host whole, so the exact operators (argmax, gather) are compared with torch's own on the GPU, and the
@@ -136,3 +137,40 @@ def test_fp4_write_source_beyond_four_gib(ops):
     for c in (kc, ks):
         clean = (c.view(NB * bs, -1) == 0xA5).all(dim=1)
         assert torch.equal(clean.cpu(), ~written)
+
+
+def test_bulk_write_source_beyond_four_gib(ops):
+    """keys / values of 4.6 GB each (70 000 tokens x 32 layers x 1024): token rows whose byte offsets pass 2^32, the
+    caches of ordinary size.  Every cache row that no valid slot names keeps its sentinel; the first and the last
+    tokens' rows equal what the oracle writes for them into a pool just large enough."""
+    T, L, H, D, bs = 70_000, 32, 8, 128, 16
+    n, NB = H * D, (70_000 + 15) // 16 + 7
+    keys, values = randn_bf16(T, L * n, 23), randn_bf16(T, L * n, 24)
+    assert keys.numel() * 2 > 1 << 32
+    g = torch.Generator().manual_seed(25)
+    slots = torch.randperm(NB * bs, generator=g)[:T]
+    slots[3::53] = -1
+    bufs = [torch.full((2, NB, bs, H, D), 0xA5, dtype=torch.uint8, device=DEV) for _ in range(L)]
+    kc, vc = [b[0] for b in bufs], [b[1] for b in bufs]
+    ks = [torch.tensor(0.011 + 0.001 * l, device=DEV) for l in range(L)]
+    vs = [torch.tensor(0.013 + 0.001 * l, device=DEV) for l in range(L)]
+    ops.reshape_and_cache_flash_bulk(keys, values, kc, vc, slots.to(DEV), "fp8", ks, vs, H, D)
+    written = torch.zeros(NB * bs, dtype=torch.bool)
+    written[slots[slots >= 0]] = True
+    dwritten = written.to(DEV)
+    for c in kc + vc:
+        assert torch.equal((c.view(NB * bs, n) == 0xA5).all(dim=1), ~dwritten)
+    pick = torch.cat([torch.arange(1024), torch.arange(T - 1024, T)])
+    sub = slots[pick]
+    valid = sub >= 0
+    count = int(valid.sum())
+    remap = torch.full_like(sub, -1)
+    remap[valid] = torch.arange(count)
+    obufs = [torch.zeros(2, (count + bs - 1) // bs, bs, H, D, dtype=torch.uint8) for _ in range(L)]
+    oracle.reshape_and_cache_flash_bulk(keys[pick.to(DEV)].cpu(), values[pick.to(DEV)].cpu(), [b[0] for b in obufs],
+                                        [b[1] for b in obufs], remap, "fp8", [s.cpu() for s in ks], [s.cpu() for s in vs],
+                                        H, D)
+    at = sub[valid].to(DEV)
+    for l in range(L):
+        for which, c in enumerate((kc[l], vc[l])):
+            assert torch.equal(c.view(NB * bs, n)[at].cpu(), obufs[l][which].view(-1, n)[:count]), f"layer {l}"

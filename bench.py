@@ -1174,7 +1174,10 @@ def bench_bulk_variants(dev, steps, placement="compact"):
     stores and the next batch's loads, the workgroup shape, and the number of layer groups per token.  `placement`:
     "compact" = 40 caches of 8192 blocks and the source allocated first in this process (one HBM region on an idle
     GPU); "serving" = the headline's memory map (66 GiB of weights, an 80-layer pool of 65536 blocks, layers 40-79
-    written), where only the shapes and group counts that are candidates for the launch rule are timed."""
+    written), where only the shapes and group counts that are candidates for the launch rule are timed;
+    "serving-8b" = 8192 tokens x 16 layers on the 8B model's map (8 GiB of weights, a 32-layer pool of 229376 blocks,
+    layers 16-31 written) and "compact-8b" the same launch with 16 caches of 8192 blocks alone on the GPU: the launch
+    at the line between the two workgroup shapes, 256 lanes x 4 chunks against 1024 lanes x 1."""
     import ctypes
     tuning = load_tuning_library()
     if tuning is None:
@@ -1182,6 +1185,11 @@ def bench_bulk_variants(dev, steps, placement="compact"):
     if placement == "serving":
         mem = ServingMemoryMap(dev, 66, 80, 40, 65536, 16, 8, 128, torch.uint8)
         w = BulkWorkload("70B-SwiftKV", 16384, 40, 8, 128, 16, 65536, "fp8", 0.10, 2, 1.5, dev, bufs=mem.written_layers())
+    elif placement == "serving-8b":
+        mem = ServingMemoryMap(dev, 8, 32, 16, 229376, 16, 8, 128, torch.uint8)
+        w = BulkWorkload("8B-prefill-serving", 8192, 16, 8, 128, 16, 229376, "fp8", 0.0, 1, 1.5, dev, bufs=mem.written_layers())
+    elif placement == "compact-8b":
+        w = BulkWorkload("8B-prefill-compact", 8192, 16, 8, 128, 16, 8192, "fp8", 0.0, 1, 1.5, dev)
     else:
         w = BulkWorkload("70B-SwiftKV-compact", 16384, 40, 8, 128, 16, 8192, "fp8", 0.10, 2, 1.5, dev)
     tab = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
@@ -1214,6 +1222,11 @@ def bench_bulk_variants(dev, steps, placement="compact"):
              ("512 lanes x 2 chunks, 768 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "768"}),
              ("512 lanes x 2 chunks, 1024 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "1024"}),
              ("512 lanes x 2 chunks, 2048 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "2048"})]
+    if placement.endswith("-8b"):
+        cases = [("as shipped (256 lanes x 4 chunks, 2 groups of 8 layers)", {}),
+                 ("the same groups as batches of 1024 lanes x 1 chunk", {"ARCTIC_BULK_WIDE": "1"}),
+                 ("1024 lanes x 1 chunk, one group of 16 layers", {"ARCTIC_BULK_WIDE": "1", "ARCTIC_BULK_GROUPS": "1"}),
+                 ("256 lanes x 4 chunks, one group of 16 layers", {"ARCTIC_BULK_GROUPS": "1"})]
     if placement == "serving":
         cases = [c for c in cases if "loop over" not in c[0] and "resident" not in c[0] and "8 groups" not in c[0]]
         cases += [("512 lanes x 2 chunks, 4 groups of 10 layers", {"ARCTIC_BULK_SHAPE": "5", "ARCTIC_BULK_GROUPS": "4"}),
@@ -1533,7 +1546,8 @@ def main():
                          "kernel (time stamps written by the tuning build), with requests at once and in stages")
     ap.add_argument("--argmax-variants", action="store_true",
                     help="instead of the benchmark, time loop shapes of the row-argmax kernel through the tuning build")
-    ap.add_argument("--bulk-variants", nargs="?", const="compact", default=None, choices=["compact", "serving"],
+    ap.add_argument("--bulk-variants", nargs="?", const="compact", default=None,
+                    choices=["compact", "serving", "compact-8b", "serving-8b"],
                     help="instead of the benchmark, time launch variants of the bulk write through the tuning build, "
                          "in the compact placement (default) or on the headline's serving memory map; prints one "
                          "JSON object")
@@ -1567,7 +1581,9 @@ def main():
         print(json.dumps({"row_argmax_variants": bench_argmax_variants(dev, args.steps)}), flush=True)
         return
     if args.bulk_variants:
-        name = "bulk_write_variants_compact_pool" if args.bulk_variants == "compact" else "bulk_write_variants_serving_map"
+        name = {"compact": "bulk_write_variants_compact_pool", "serving": "bulk_write_variants_serving_map",
+                "compact-8b": "bulk_write_variants_8b_compact_pool",
+                "serving-8b": "bulk_write_variants_8b_serving_map"}[args.bulk_variants]
         print(json.dumps({name: bench_bulk_variants(dev, args.steps, args.bulk_variants)}), flush=True)
         return
     if args.only:

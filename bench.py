@@ -1255,6 +1255,116 @@ def bench_bulk_variants(dev, steps, placement="compact"):
                    "writes_the_same_bytes": same[name]} for name, v in out.items()}
 
 
+def bench_launch_shapes(dev, steps):
+    """A/B of launch shapes of three smaller kernels through the tuning build, each variant captured in a HIP graph
+    over rotating buffer sets and replayed in turn, three rounds: (a) the fp4 cache write (lanes per workgroup, groups
+    per lane; 2048, 8192 and 32768 tokens, 16 layers of 8 x 128); (b) the row gather of swiftkv_select's five tensors
+    (lanes per workgroup; 512 and 2048 rows of the 70B shape); (c) the bulk fp8 write at a decode size (512 tokens x
+    16 layers into 32768-block caches; workgroups of 64 to 1024 lanes, chunks per lane, layer groups per token)."""
+    import ctypes
+    tuning = load_tuning_library()
+    if tuning is None:
+        return "libarctic_tuning_mi355x.so is not built"
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    tuning.arctic_reshape_and_cache_flash_fp4.argtypes = [vp, vp, i64, i64, vp, vp, vp, vp, vp, i64, i32, i32, i32, i64, i64,
+                                                          i64, i64, i32, vp]
+    tuning.arctic_reshape_and_cache_flash_fp4.restype = i32
+    tuning.arctic_gather_rows.argtypes = [i32, vp, vp, vp, vp, vp, vp, i32, i64, i64, i32, vp]
+    tuning.arctic_gather_rows.restype = i32
+    knobs = ("ARCTIC_FP4_LANES", "ARCTIC_FP4_GROUPS", "ARCTIC_GATHER_LANES", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_GROUPS")
+
+    def rounds(cases, call, per_graph):
+        """us per call of every case: one graph per case (the environment is read when a launch is captured)."""
+        graphs = []
+        for name, env in cases:
+            for k in knobs:
+                os.environ.pop(k, None)
+            os.environ.update(env)
+            call()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                call()
+            graphs.append((name, graph))
+        for k in knobs:
+            os.environ.pop(k, None)
+        times = {name: [] for name, _ in cases}
+        for _ in range(3):
+            for name, graph in graphs:
+                warm_replays(graph.replay, min_ms=5.0)
+                times[name].append(round(statistics.median(event_times_us(graph.replay, max(10, steps // 4))) / per_graph, 2))
+        return times
+
+    out = {}
+    stream = lambda: torch.cuda.current_stream().cuda_stream
+    # (a) fp4 write
+    H, D, bs, L = 8, 128, 16, 16
+    g = torch.Generator(device=dev).manual_seed(5)
+    for T in (2048, 8192, 32768):
+        NB = 2 * T // bs
+        keys = [(torch.randn(T, H, D, generator=g, device=dev) * 0.5).to(torch.bfloat16) for _ in range(L)]
+        values = [(torch.randn(T, H, D, generator=g, device=dev) * 0.5).to(torch.bfloat16) for _ in range(L)]
+        kc, vc = ([torch.zeros(NB, bs, H, D // 2, dtype=torch.uint8, device=dev) for _ in range(L)] for _ in range(2))
+        ks, vs = ([torch.zeros(NB, bs, H, D // 16, dtype=torch.uint8, device=dev) for _ in range(L)] for _ in range(2))
+        slots = torch.randperm(NB * bs, generator=torch.Generator().manual_seed(5))[:T].to(dev)
+
+        def fp4():
+            for l in range(L):
+                rc = tuning.arctic_reshape_and_cache_flash_fp4(
+                    keys[l].data_ptr(), values[l].data_ptr(), H * D, H * D, kc[l].data_ptr(), vc[l].data_ptr(),
+                    ks[l].data_ptr(), vs[l].data_ptr(), slots.data_ptr(), T, H, D, bs, kc[l].stride(0), kc[l].stride(1),
+                    kc[l].stride(2), NB, 2, stream())
+                assert rc == 0, rc
+        cases = [("64 lanes, one group per lane (shipped)", {})] + \
+                [(f"{n} lanes, one group per lane", {"ARCTIC_FP4_LANES": str(n)}) for n in (128, 256, 512, 1024)] + \
+                [(f"256 lanes, {n} groups per lane", {"ARCTIC_FP4_GROUPS": str(n)}) for n in (2, 4)]
+        out[f"fp4_write_{T}_tokens_us_per_layer"] = rounds(cases, fp4, L)
+        del keys, values, kc, vc, ks, vs
+    # (b) row gather
+    hidden, kvw, sets = 8192, 40 * 1024, 4
+    for T in (512, 2048):
+        rn = lambda *s: torch.randn(*s, generator=g, device=dev).to(torch.bfloat16)
+        src = [[rn(T, hidden), rn(T, hidden), torch.arange(T, device=dev), rn(T, kvw), rn(T, kvw)] for _ in range(sets)]
+        dst = [[torch.empty_like(t) for t in s_] for s_ in src]
+        idx = torch.randperm(T, device=dev)
+
+        def gather():
+            for s_, d_ in zip(src, dst):
+                n = len(s_)
+                rc = tuning.arctic_gather_rows(
+                    n, (vp * n)(*[t.data_ptr() for t in s_]), (vp * n)(*[t.data_ptr() for t in d_]),
+                    (i64 * n)(*[t[0].numel() * t.element_size() for t in s_]),
+                    (i64 * n)(*[t.stride(0) * t.element_size() for t in s_]),
+                    (i64 * n)(*[t.stride(0) * t.element_size() for t in d_]), idx.data_ptr(), 8, T, T, 0, stream())
+                assert rc == 0, rc
+        cases = [("256 lanes (shipped)", {})] + [(f"{n} lanes", {"ARCTIC_GATHER_LANES": str(n)}) for n in (64, 128, 512, 1024)]
+        out[f"gather_rows_{T}_rows_us_per_call"] = rounds(cases, gather, sets)
+        del src, dst
+    # (c) bulk write at a decode size
+    sets = 8
+    ws = [BulkWorkload("decode", 512, 16, 8, 128, 16, 32768, "fp8", 0.0, 4, 1.5, dev)]
+    for i in range(1, sets):
+        ws.append(BulkWorkload("decode", 512, 16, 8, 128, 16, 32768, "fp8", 0.0, 4 + i, 1.5, dev, bufs=ws[0].bufs))
+    tab = lambda ts: (vp * len(ts))(*[t.data_ptr() for t in ts])
+
+    def bulk():
+        for w in ws:
+            rc = tuning.arctic_reshape_and_cache_flash_bulk(
+                w.keys.data_ptr(), w.values.data_ptr(), w.keys.stride(0), w.values.stride(0), tab(w.key_caches),
+                tab(w.value_caches), tab(w.k_scales), tab(w.v_scales), w.slots.data_ptr(), w.T, w.L, w.H, w.D, w.bs,
+                w.key_caches[0].stride(0), w.NB, 2, 1, stream())
+            assert rc == 0, rc
+    shapes = {4: "1024 x 1", 5: "512 x 2", 6: "256 x 2", 7: "256 x 1", 8: "512 x 1", 9: "64 x 4", 10: "64 x 8", 11: "128 x 4",
+              12: "128 x 8"}
+    cases = [("256 lanes x 4 chunks, 4 groups of 4 layers (shipped)", {})]
+    for shape, groups in ((4, 1), (4, 2), (5, 2), (8, 2), (6, 4), (7, 8), (9, 16), (9, 8), (10, 8), (10, 4), (11, 8), (11, 4),
+                          (12, 4), (12, 2)):
+        cases.append((f"{shapes[shape]} (lanes x chunks), {groups} groups of {16 // groups} layers",
+                      {"ARCTIC_BULK_SHAPE": str(shape), "ARCTIC_BULK_GROUPS": str(groups)}))
+    out["bulk_write_512_tokens_16_layers_us_per_call"] = rounds(cases, bulk, sets)
+    return out
+
+
 def bench_argmax_variants(dev, steps):
     """A/B of the row-argmax kernel's loop shapes through the tuning build: 512 rows x 128256 bf16 logits (131 MB),
     three rotating sets in one graph per variant, three rounds over all variants; results compared with torch's."""
@@ -1546,6 +1656,9 @@ def main():
                          "kernel (time stamps written by the tuning build), with requests at once and in stages")
     ap.add_argument("--argmax-variants", action="store_true",
                     help="instead of the benchmark, time loop shapes of the row-argmax kernel through the tuning build")
+    ap.add_argument("--launch-shapes", action="store_true",
+                    help="instead of the benchmark, time launch shapes of the fp4 write, the row gather and the bulk "
+                         "write at a decode size through the tuning build")
     ap.add_argument("--bulk-variants", nargs="?", const="compact", default=None,
                     choices=["compact", "serving", "compact-8b", "serving-8b"],
                     help="instead of the benchmark, time launch variants of the bulk write through the tuning build, "
@@ -1579,6 +1692,9 @@ def main():
         return
     if args.argmax_variants:
         print(json.dumps({"row_argmax_variants": bench_argmax_variants(dev, args.steps)}), flush=True)
+        return
+    if args.launch_shapes:
+        print(json.dumps({"launch_shapes": bench_launch_shapes(dev, args.steps)}), flush=True)
         return
     if args.bulk_variants:
         name = {"compact": "bulk_write_variants_compact_pool", "serving": "bulk_write_variants_serving_map",

@@ -55,8 +55,7 @@ def build(force: bool = True, verbose: bool = False) -> str:
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
         raise RuntimeError("arcticinference_amd: hipcc not found; cannot build " + LIB_BASENAME)
-    # "tuning": the measurement build of the same sources that the benchmark's variant sweeps load
-    cmd = ["make", "-C", _CSRC_DIR, "-j8", f"HIPCC={hipcc}", "all", "tuning"]
+    cmd = ["make", "-C", _CSRC_DIR, "-j8", f"HIPCC={hipcc}", "all"]
     if force:
         cmd.append("-B")
     proc = subprocess.run(cmd, capture_output=True, text=True)

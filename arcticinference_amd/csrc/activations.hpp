@@ -15,29 +15,11 @@ __device__ __forceinline__ float fast_exp(float x) {            // e^x
 __device__ __forceinline__ float sigmoid_f(float x) {
   return __builtin_amdgcn_rcpf(1.0f + fast_exp(-x));
 }
-// 1 + e^-x, kept finite (x >= -40) so that it can be multiplied into a shared denominator
-__device__ __forceinline__ float sigmoid_den(float x) {
-  return 1.0f + fast_exp(-fmaxf(x, -40.0f));
-}
 // gelu(x) = x * Phi(x) with Phi from Abramowitz & Stegun 7.1.26
 //   erfc(z) = (a1 t + ... + a5 t^5) exp(-z^2),  t = 1 / (1 + 0.3275911 z),  z >= 0
 // (|error| <= 1.5e-7, the level of fp32 rounding).  With z = |x| / sqrt(2) and
 // q = erfc(z) / 2:   gelu(x) = x - x q  for x >= 0  and  x q  for x < 0,
 // i.e. max(x, 0) - |x| q.  One reciprocal and one exp2 per value.
-// gelu_erf with t = 1 / gelu_erf_den(x) supplied by the caller
-__device__ __forceinline__ float gelu_erf_den(float x) {
-  return fmaf(0.3275911f * 0.70710678118654752440f, fabsf(x), 1.0f);
-}
-__device__ __forceinline__ float gelu_erf_given_t(float x, float t) {
-  const float ax = fabsf(x);
-  float poly = fmaf(0.5f * 1.061405429f, t, 0.5f * -1.453152027f);
-  poly = fmaf(poly, t, 0.5f * 1.421413741f);
-  poly = fmaf(poly, t, 0.5f * -0.284496736f);
-  poly = fmaf(poly, t, 0.5f * 0.254829592f);
-  poly *= t;
-  const float q = poly * __builtin_amdgcn_exp2f((x * (-0.5f * 1.4426950408889634f)) * x);
-  return fmaf(-ax, q, fmaxf(x, 0.0f));
-}
 __device__ __forceinline__ float gelu_erf(float x) {
   const float ax = fabsf(x);
   const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f * 0.70710678118654752440f, ax, 1.0f));

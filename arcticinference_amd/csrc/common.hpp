@@ -103,28 +103,14 @@ __device__ __forceinline__ uint4 load16(const void *p) {
   const u32x4 v = *(const ARCTIC_GLOBAL u32x4 *)p;
   return make_uint4(v.x, v.y, v.z, v.w);
 }
-// streaming variants: every byte on these paths is touched exactly once
-#ifndef ARCTIC_NT_LOAD
-#define ARCTIC_NT_LOAD 1
-#endif
-#ifndef ARCTIC_NT_STORE
-#define ARCTIC_NT_STORE 1
-#endif
+// streaming (non-temporal) variants: every byte on these paths is touched exactly once
 __device__ __forceinline__ uint4 load16_stream(const void *p) {
-#if ARCTIC_NT_LOAD
   const u32x4 v = __builtin_nontemporal_load((const ARCTIC_GLOBAL u32x4 *)p);
-#else
-  const u32x4 v = *(const ARCTIC_GLOBAL u32x4 *)p;
-#endif
   return make_uint4(v.x, v.y, v.z, v.w);
 }
 __device__ __forceinline__ void store16_stream(void *p, const uint4 &v) {
   const u32x4 t = {v.x, v.y, v.z, v.w};
-#if ARCTIC_NT_STORE
   __builtin_nontemporal_store(t, (ARCTIC_GLOBAL u32x4 *)p);
-#else
-  *(ARCTIC_GLOBAL u32x4 *)p = t;
-#endif
 }
 __device__ __forceinline__ void store16(void *p, const uint4 &v) {  // stays in the caches: read again soon
   const u32x4 t = {v.x, v.y, v.z, v.w};
@@ -132,27 +118,16 @@ __device__ __forceinline__ void store16(void *p, const uint4 &v) {  // stays in 
 }
 __device__ __forceinline__ void store8_stream(void *p, const uint2 &v) {
   const u32x2 t = {v.x, v.y};
-#if ARCTIC_NT_STORE
   __builtin_nontemporal_store(t, (ARCTIC_GLOBAL u32x2 *)p);
-#else
-  *(ARCTIC_GLOBAL u32x2 *)p = t;
-#endif
 }
 __device__ __forceinline__ void store4_stream(void *p, uint32_t v) {
-#if ARCTIC_NT_STORE
   __builtin_nontemporal_store(v, (ARCTIC_GLOBAL uint32_t *)p);
-#else
-  *(ARCTIC_GLOBAL uint32_t *)p = v;
-#endif
 }
 
-// A lane's unit of work on the speculator paths: E consecutive 16-bit elements
-// moved with one access (E = 8: 16 bytes; narrower units measured slower).
-template <int E>
-struct Chunk;
-
-template <>
-struct Chunk<8> {
+// A lane's unit of work on the speculator paths: eight consecutive 16-bit elements
+// moved with one 16-byte access (narrower units measured slower).
+struct Chunk {
+  static constexpr int kElems = 8;
   static constexpr int kBytes = 16;
   uint4 v;
   __device__ static __forceinline__ Chunk zero() { return Chunk{make_uint4(0, 0, 0, 0)}; }
@@ -165,42 +140,6 @@ struct Chunk<8> {
   template <typename T>
   __device__ static __forceinline__ Chunk pack(const float (&f)[8]) { return Chunk{pack8<T>(f)}; }
 };
-
-#ifdef ARCTIC_TUNING
-// measurement build only: 8-byte units (4 elements per lane), to time them against the 16-byte ones
-__device__ __forceinline__ uint2 load8(const void *p) {
-  const u32x2 v = *(const ARCTIC_GLOBAL u32x2 *)p;
-  return make_uint2(v.x, v.y);
-}
-__device__ __forceinline__ uint2 load8_stream(const void *p) {
-  const u32x2 v = __builtin_nontemporal_load((const ARCTIC_GLOBAL u32x2 *)p);
-  return make_uint2(v.x, v.y);
-}
-template <>
-struct Chunk<4> {
-  static constexpr int kBytes = 8;
-  uint2 v;
-  __device__ static __forceinline__ Chunk zero() { return Chunk{make_uint2(0, 0)}; }
-  __device__ static __forceinline__ Chunk load(const void *p) { return Chunk{load8(p)}; }
-  __device__ static __forceinline__ Chunk load_stream(const void *p) { return Chunk{load8_stream(p)}; }
-  __device__ __forceinline__ void store_stream(void *p) const { store8_stream(p, v); }
-  __device__ __forceinline__ void store(void *p) const {
-    const u32x2 t = {v.x, v.y};
-    *(ARCTIC_GLOBAL u32x2 *)p = t;
-  }
-  template <typename T>
-  __device__ __forceinline__ void unpack(float (&f)[4]) const {
-    f[0] = T::lo(v.x);
-    f[1] = T::hi(v.x);
-    f[2] = T::lo(v.y);
-    f[3] = T::hi(v.y);
-  }
-  template <typename T>
-  __device__ static __forceinline__ Chunk pack(const float (&f)[4]) {
-    return Chunk{make_uint2(T::pack(f[0], f[1]), T::pack(f[2], f[3]))};
-  }
-};
-#endif
 
 // ---- wave64 / workgroup reductions ------------------------------------------
 // DPP butterfly inside each row of 16 lanes, then the four row totals are read

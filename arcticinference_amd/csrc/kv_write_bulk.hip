@@ -24,7 +24,6 @@
 
 #include <algorithm>
 #include <cstdint>
-#include <cstdlib>
 #include <mutex>
 #include <type_traits>
 
@@ -78,11 +77,6 @@ struct BulkParams {
   unsigned index_blocks;
   int index_is_64;
   int select_mode;   // kSelectNone / kSelectByRowMap / kSelectByScan (the vector kernels take it as a template argument)
-#ifdef ARCTIC_TUNING
-  int loads_before_stores;  // measurement build: the next batch is requested before this one is converted and stored
-  unsigned items;           // measurement build: not 0 = workgroups loop over this many items (ARCTIC_BULK_PERSISTENT)
-  int lockstep;             // measurement build: a barrier behind every batch's requests (ARCTIC_BULK_LOCKSTEP)
-#endif
 };
 
 // How a launch finds the output rows of a token: not at all, through the inverse of the index list that the caller
@@ -202,7 +196,7 @@ __device__ __forceinline__ void select_leftover_rows(const BulkParams &p, unsign
 // kBulkThreads x kUnroll 16-byte chunks form one batch of a workgroup.  Three shapes are built, all with batches
 // of 1024 chunks: 1024 x 1 (launches of more than 8192 tokens: a workgroup moves up to five batches), 512 x 2 (the
 // same launches when rows are selected as well) and 256 x 4 (everything smaller: one or two batches per workgroup).
-template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll, int kSelect, bool kLoadsFirst = false>
+template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll, int kSelect>
 __device__ __forceinline__ void bulk_item(const BulkParams &p, const LayerTables &tab, unsigned block) {
   constexpr bool kCopy = std::is_same<Dst, Copy>::value;
   constexpr int kDstElemBytes = kCopy ? Src::kBytes : 1;
@@ -336,7 +330,6 @@ __device__ __forceinline__ void bulk_item(const BulkParams &p, const LayerTables
   while (c < total) {
     const int cn = c + kUnroll * kBulkThreads;
     uint4 nxt[kUnroll];
-    if constexpr (kLoadsFirst) load_batch(cn, nxt);   // (an instantiation of the measurement build only)
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int cu = c + u * kBulkThreads;
@@ -357,164 +350,20 @@ __device__ __forceinline__ void bulk_item(const BulkParams &p, const LayerTables
         }
       }
     }
-    if constexpr (!kLoadsFirst) load_batch(cn, nxt);
-#ifdef ARCTIC_TUNING
-    // measurement build (ARCTIC_BULK_LOCKSTEP, whole batches only): the waves of a workgroup request batch k + 1
-    // together, behind a barrier that waits for no memory
-    if (p.lockstep) {
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
-    }
-#endif
+    load_batch(cn, nxt);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) cur[u] = nxt[u];
     c = cn;
   }
 }
 
-template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll, int kSelect, bool kLoadsFirst = false>
+template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll, int kSelect>
 __global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_kernel(
     const BulkParams p, const LayerTables tab) {
-  bulk_item<Src, Dst, kPow2, kBulkThreads, kUnroll, kSelect, kLoadsFirst>(p, tab, blockIdx.x);
+  bulk_item<Src, Dst, kPow2, kBulkThreads, kUnroll, kSelect>(p, tab, blockIdx.x);
 }
 
-#ifdef ARCTIC_TUNING
-// Measurement build only (ARCTIC_BULK_PERSISTENT): a grid of fewer workgroups, each taking every gridDim.x-th item
-// in turn.  A kernel of its own, so that the kernel above is compiled exactly as in the library.
-template <typename Src, typename Dst, bool kPow2, int kBulkThreads, int kUnroll>
-__global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_looping_kernel(const BulkParams p, const LayerTables tab) {
-  for (unsigned item = blockIdx.x; item < p.items; item += gridDim.x) {
-    bulk_item<Src, Dst, kPow2, kBulkThreads, kUnroll, kSelectNone>(p, tab, item);
-    __syncthreads();   // the next item rewrites the row descriptors
-  }
-}
-#endif
 
-#ifdef ARCTIC_TUNING
-// Measurement build only (ARCTIC_BULK_RESIDENT): measured slower than one workgroup per token and layer group.
-// The same write by resident workgroups, for launches of thousands of tokens whose per-workgroup share is a
-// whole number of batches.  The grid is a few workgroups per CU (a multiple of groups_per_token, so that a
-// workgroup keeps its layer group); each walks over every (gridDim.x / groups_per_token)-th token.  What depends
-// on the layers alone - cache pointer and reciprocal scale of each row - is put into LDS once, and so are the slots
-// of the workgroup's tokens; what depends on the token is then one number, the byte offset of its slot's row inside
-// a cache, which is uniform and lives in scalar registers.  So there is nothing to rebuild and no barrier between
-// tokens, and the stream of batches runs across token boundaries.  Every batch is straight-line code - kUnroll
-// loads of the next batch, kUnroll conversions and stores of the current one, no lane left out - so that the compiler
-// knows exactly how many requests are outstanding and waits for the oldest only: loads and stores of a workgroup
-// overlap.  Tokens without a slot are skipped while walking the slot list and cost no source traffic.
-constexpr int kResidentMaxTokens = 1024;   // tokens per workgroup whose slots fit the LDS list
-
-__device__ __forceinline__ int64_t uniform64(int64_t v) {
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
-  return (int64_t)(((uint64_t)hi << 32) | lo);
-}
-
-template <typename Src, typename Dst, int kBulkThreads, int kUnroll>
-__global__ __launch_bounds__(kBulkThreads) void kv_write_bulk_resident_kernel(const BulkParams p, const LayerTables tab) {
-  constexpr bool kCopy = std::is_same<Dst, Copy>::value;
-  constexpr int kDstElemBytes = kCopy ? Src::kBytes : 1;
-  constexpr int kBatch = kBulkThreads * kUnroll;
-  __shared__ RowDesc rows[2 * kLayersPerLaunch];
-  __shared__ int64_t slots[kResidentMaxTokens];   // of this workgroup's tokens; -1: no row to write
-
-  const int group = blockIdx.x % (unsigned)p.groups_per_token;
-  const int step = gridDim.x / (unsigned)p.groups_per_token;
-  const int layer0 = group * p.layers_per_group;
-  const int nlayers = min(p.layers_per_group, p.num_layers - layer0);
-  const int cpr = p.chunks_per_row;
-  const int total = 2 * nlayers * cpr;   // chunks of one token that this workgroup moves: a multiple of kBatch
-  const int64_t column0 = (int64_t)layer0 * p.n * Src::kBytes;
-  const int64_t token0 = blockIdx.x / (unsigned)p.groups_per_token;
-  const int ntok = (int)((p.num_tokens - token0 + step - 1) / step);   // <= kResidentMaxTokens (the host sees to it)
-
-  for (int r = threadIdx.x; r < 2 * nlayers; r += kBulkThreads) {
-    const int layer = layer0 + (r >> 1);
-    const bool is_v = r & 1;
-    RowDesc d;
-    d.dst = (char *)(is_v ? tab.value_cache[layer] : tab.key_cache[layer]);
-    d.inv = 0.0;
-    if constexpr (!kCopy) d.inv = 1.0 / (double)(*(is_v ? tab.v_scale[layer] : tab.k_scale[layer]));
-    rows[r] = d;
-  }
-  for (int k = threadIdx.x; k < ntok; k += kBulkThreads) {
-    const int64_t slot = p.slot_mapping[token0 + (int64_t)k * step];
-    slots[k] = (slot >= 0 && slot < p.num_slots) ? slot : -1;
-  }
-  __syncthreads();
-
-  auto next_with_row = [&](int k, int64_t &slot) {   // uniform: every lane reads the same LDS words
-    slot = -1;
-    while (k < ntok && (slot = uniform64(slots[k])) < 0) ++k;
-    return k;
-  };
-  auto row_offset = [&](int64_t slot) -> int64_t {   // bytes from a cache's base to the slot's row
-    int64_t blk, off;
-    if (slot < 0x7fffffffLL) {
-      const uint32_t s32 = (uint32_t)slot, bs = (uint32_t)p.block_size;
-      blk = s32 / bs;
-      off = s32 - (uint32_t)blk * bs;
-    } else {
-      blk = slot / p.block_size;
-      off = slot - blk * p.block_size;
-    }
-    return (blk * p.block_stride + off * (int64_t)p.n) * kDstElemBytes;
-  };
-  auto load_batch = [&](int64_t token, int first, uint4 (&v)[kUnroll]) {
-    const char *ksrc = p.keys + token * p.key_stride_bytes + column0;
-    const char *vsrc = p.values + token * p.value_stride_bytes + column0;
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const int c = first + (int)threadIdx.x + u * kBulkThreads;
-      const int r = c >> p.chunk_shift, col = c & (cpr - 1);
-      v[u] = load16_stream(((r & 1) ? vsrc : ksrc) + ((int64_t)(r >> 1) * cpr + col) * 16);
-    }
-  };
-
-  int64_t slot;
-  int k = next_with_row(0, slot);
-  if (k >= ntok) return;
-  int64_t token = token0 + (int64_t)k * step;
-  int64_t offset = row_offset(slot);
-  int first = 0;
-  // One batch: request the batch behind it into `nxt`, convert and store `cur`.  Called with the two register sets
-  // in turn, so that no batch is ever copied from one set to the other (a copy would wait for its loads).
-  auto batch = [&](uint4 (&cur)[kUnroll], uint4 (&nxt)[kUnroll]) -> bool {
-    // where the batch behind this one lies: further on in the token, or at the start of the next token with a row
-    int nfirst = first + kBatch;
-    int64_t ntoken = token, noffset = offset;
-    bool last = false;
-    if (nfirst >= total) {
-      nfirst = 0;
-      k = next_with_row(k + 1, slot);
-      if (k < ntok) {
-        ntoken = token0 + (int64_t)k * step;
-        noffset = row_offset(slot);
-      } else {
-        last = true;   // nothing behind it: the loads below fetch this token's first batch again and are dropped
-      }
-    }
-    load_batch(ntoken, nfirst, nxt);
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const int c = first + (int)threadIdx.x + u * kBulkThreads;
-      const int r = c >> p.chunk_shift, col = c & (cpr - 1);
-      RowDesc d = rows[r];
-      d.dst += offset;
-      emit_chunk<Src, Dst>(cur[u], d, col);
-    }
-    token = ntoken;
-    offset = noffset;
-    first = nfirst;
-    return !last;
-  };
-  uint4 even[kUnroll], odd[kUnroll];
-  load_batch(token, first, even);
-  while (batch(even, odd) && batch(odd, even)) {
-  }
-}
-#endif  // ARCTIC_TUNING
 
 // Fallback for shapes or addresses that do not allow 16-byte accesses: one
 // element per lane per step, any alignment.  Same arithmetic, no vector access.
@@ -622,67 +471,6 @@ __global__ __launch_bounds__(kScalarThreads) void kv_write_bulk_scalar_kernel(
 template <typename Src, typename Dst, int kSelect>
 static void launch_vec_shape(const BulkParams &p, const LayerTables &tab, int64_t grid, bool wide, hipStream_t s) {
   const dim3 g((unsigned)grid);
-#ifdef ARCTIC_TUNING
-  // measurement build: ARCTIC_BULK_RESIDENT = workgroups per CU of the resident kernel (x 10 + 1: four chunks per lane)
-  if constexpr (kSelect == kSelectNone) {
-    const char *e = getenv("ARCTIC_BULK_RESIDENT");
-    const int v = e ? atoi(e) : 0;
-    if (v && p.chunk_shift >= 0) {
-      const int per_cu = v >= 10 ? v / 10 : v;
-      unsigned wg = (unsigned)std::min<int64_t>(grid, 256LL * per_cu);
-      wg -= wg % (unsigned)p.groups_per_token;
-      const bool four = v >= 10 && v % 10 == 1;
-      const int64_t per_wg = 2LL * p.layers_per_group * p.chunks_per_row;   // chunks of a token per workgroup
-      const bool fits = wg >= (unsigned)p.groups_per_token && p.num_layers % p.layers_per_group == 0 &&
-                        per_wg % (512 * (four ? 4 : 2)) == 0 &&
-                        (p.num_tokens + wg / p.groups_per_token - 1) / (wg / p.groups_per_token) <= kResidentMaxTokens;
-      if (fits) {
-        if (four)
-          hipLaunchKernelGGL((kv_write_bulk_resident_kernel<Src, Dst, 512, 4>), dim3(wg), dim3(512), 0, s, p, tab);
-        else
-          hipLaunchKernelGGL((kv_write_bulk_resident_kernel<Src, Dst, 512, 2>), dim3(wg), dim3(512), 0, s, p, tab);
-        return;
-      }
-    }
-  }
-  // ARCTIC_BULK_PERSISTENT: p.items is set and the grid cut down; ARCTIC_BULK_LOADS_FIRST: the other order in the loop
-  if constexpr (kSelect == kSelectNone) {
-    if (p.chunk_shift >= 0 && (p.items || p.loads_before_stores)) {
-      if (p.items && wide)
-        hipLaunchKernelGGL((kv_write_bulk_looping_kernel<Src, Dst, true, 512, 2>), g, dim3(512), 0, s, p, tab);
-      else if (p.items)
-        hipLaunchKernelGGL((kv_write_bulk_looping_kernel<Src, Dst, true, 256, 4>), g, dim3(256), 0, s, p, tab);
-      else if (wide)
-        hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 512, 2, kSelectNone, true>), g, dim3(512), 0, s, p, tab);
-      else
-        hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 256, 4, kSelectNone, true>), g, dim3(256), 0, s, p, tab);
-      return;
-    }
-  }
-  // ARCTIC_BULK_SHAPE = 1: 512 lanes x 4 chunks, 2: 1024 x 2, 3: 1024 x 4, 4: 1024 x 1, 5: 512 x 2, 6: 256 x 2, 7: 256 x 1, 8: 512 x 1,
-  // 9: 64 x 4, 10: 64 x 8, 11: 128 x 4, 12: 128 x 8 (one- and two-wave workgroups: 2 to 25 % slower at 512 tokens)
-  if constexpr (kSelect == kSelectNone) {
-    const char *e = getenv("ARCTIC_BULK_SHAPE");
-    const int shape = e ? atoi(e) : 0;
-    if (shape && p.chunk_shift >= 0) {
-      switch (shape) {
-        case 1: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 512, 4, kSelectNone>), g, dim3(512), 0, s, p, tab); break;
-        case 2: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 1024, 2, kSelectNone>), g, dim3(1024), 0, s, p, tab); break;
-        case 3: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 1024, 4, kSelectNone>), g, dim3(1024), 0, s, p, tab); break;
-        case 5: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 512, 2, kSelectNone>), g, dim3(512), 0, s, p, tab); break;
-        case 6: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 256, 2, kSelectNone>), g, dim3(256), 0, s, p, tab); break;
-        case 7: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 256, 1, kSelectNone>), g, dim3(256), 0, s, p, tab); break;
-        case 8: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 512, 1, kSelectNone>), g, dim3(512), 0, s, p, tab); break;
-        case 9: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 64, 4, kSelectNone>), g, dim3(64), 0, s, p, tab); break;
-        case 10: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 64, 8, kSelectNone>), g, dim3(64), 0, s, p, tab); break;
-        case 11: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 128, 4, kSelectNone>), g, dim3(128), 0, s, p, tab); break;
-        case 12: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 128, 8, kSelectNone>), g, dim3(128), 0, s, p, tab); break;
-        default: hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 1024, 1, kSelectNone>), g, dim3(1024), 0, s, p, tab); break;
-      }
-      return;
-    }
-  }
-#endif
   if (p.chunk_shift >= 0) {
     if (wide && kSelect == kSelectNone)   // the same batch of 1024 chunks by 1024 lanes: 0.5-2 % faster than 512 x 2
       hipLaunchKernelGGL((kv_write_bulk_kernel<Src, Dst, true, 1024, 1, kSelectNone>), g, dim3(1024), 0, s, p, tab);
@@ -910,21 +698,8 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
     } else {
       groups = (int)std::max<int64_t>(1, std::min<int64_t>(count, (2048 + num_tokens - 1) / num_tokens));
     }
-#ifdef ARCTIC_TUNING
-    if (const char *e = getenv("ARCTIC_BULK_GROUPS")) groups = std::max(1, std::min(count, atoi(e)));
-    if (const char *e = getenv("ARCTIC_BULK_WIDE")) wide = atoi(e) != 0;
-    p.loads_before_stores = 0;
-    if (const char *e = getenv("ARCTIC_BULK_LOADS_FIRST")) p.loads_before_stores = atoi(e) != 0;
-    p.items = 0;
-    p.lockstep = 0;
-#endif
     p.layers_per_group = (count + groups - 1) / groups;
     p.groups_per_token = (count + p.layers_per_group - 1) / p.layers_per_group;
-#ifdef ARCTIC_TUNING
-    if (const char *e = getenv("ARCTIC_BULK_LOCKSTEP"))   // only where every lane of a workgroup runs the same number of batches
-      p.lockstep = atoi(e) != 0 && vec && count % p.layers_per_group == 0 &&
-                   (2LL * p.layers_per_group * p.chunks_per_row) % 1024 == 0 && !p.indices;
-#endif
     const int lanes = !vec ? kScalarThreads : (wide && p.chunk_shift >= 0) ? 512 : 256;   // of the shape launched below
     const int64_t index_blocks = p.indices ? (p.num_out_rows + lanes - 1) / lanes : 0;
     const int64_t grid = num_tokens * p.groups_per_token + index_blocks;
@@ -932,19 +707,10 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
     if (grid > 0x7fffffffLL)
       return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: too many tokens (%lld)", fn, (long long)num_tokens);
 
-    int64_t workgroups = grid;
-#ifdef ARCTIC_TUNING
-    if (const char *e = getenv("ARCTIC_BULK_PERSISTENT")) {
-      if (atoi(e) > 0 && vec && !p.indices) {   // that many workgroups, each looping over the grid's items
-        p.items = (unsigned)grid;
-        workgroups = std::min<int64_t>(grid, atoi(e));
-      }
-    }
-#endif
     switch (kv_cache_dtype) {
-      case ARCTIC_KV_AUTO: dispatch_src<Copy>(vec, wide, src_dtype, p, tab, workgroups, s); break;
-      case ARCTIC_KV_FP8_E4M3: dispatch_src<E4M3>(vec, wide, src_dtype, p, tab, workgroups, s); break;
-      default: dispatch_src<E5M2>(vec, wide, src_dtype, p, tab, workgroups, s); break;
+      case ARCTIC_KV_AUTO: dispatch_src<Copy>(vec, wide, src_dtype, p, tab, grid, s); break;
+      case ARCTIC_KV_FP8_E4M3: dispatch_src<E4M3>(vec, wide, src_dtype, p, tab, grid, s); break;
+      default: dispatch_src<E5M2>(vec, wide, src_dtype, p, tab, grid, s); break;
     }
     const int rc = check_launch(fn);
     if (rc) return rc;

@@ -11,7 +11,6 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
-#include <cstdlib>
 
 #include <cstdint>
 
@@ -39,81 +38,71 @@ struct Fp4Params {
   int block_size;
 };
 
-// kGroups groups of 16 elements per lane, kThreads groups apart, so that a wave's 64 lanes stay on 64 consecutive groups
-// (2 KiB of source, 512 bytes of packed cache) in each of them.  All of a lane's requests go out before the first
-// group is looked at.
-template <typename T, int kGroups, int kThreads>
-__global__ __launch_bounds__(kThreads) void kv_write_fp4_kernel(const Fp4Params p) {
+// One group of 16 elements per lane, single-wave workgroups: a wave's 64 lanes stay on 64 consecutive groups (2 KiB
+// of source, 512 bytes of packed cache).
+constexpr int kFp4Lanes = 64;
+
+template <typename T>
+__global__ __launch_bounds__(kFp4Lanes) void kv_write_fp4_kernel(const Fp4Params p) {
   const int groups_per_row = p.num_heads * p.groups_per_head;
-  int64_t slot[kGroups];
-  uint4 lo[kGroups], hi[kGroups];
-  int64_t idx[kGroups];
   // the slot is requested first and the group's 32 bytes right behind it: their address does not depend on the slot,
   // so one round trip to memory serves both (a padding token throws its group away)
-#pragma unroll
-  for (int u = 0; u < kGroups; ++u) {
-    idx[u] = ((int64_t)blockIdx.x * kGroups + u) * kThreads + threadIdx.x;
-    const int64_t at = min(idx[u], p.total_groups - 1);   // lanes past the end read the last group and drop it
-    const int64_t row = at / groups_per_row;              // token * 2 + (0 = K, 1 = V)
-    const int in_row = (int)(at - row * groups_per_row);
-    const int64_t token = row >> 1;
-    slot[u] = p.slot_mapping[token];
-    const char *src = ((row & 1) ? p.value + token * p.value_stride_bytes : p.key + token * p.key_stride_bytes) +
-                      (int64_t)in_row * 32;
-    lo[u] = load16_stream(src);
-    hi[u] = load16_stream(src + 16);
-  }
-  __builtin_amdgcn_sched_barrier(0);   // keeps the loads above the tests of the slots
-#pragma unroll
-  for (int u = 0; u < kGroups; ++u) {
-    if (idx[u] >= p.total_groups) continue;
-    if (slot[u] < 0 || slot[u] >= p.num_slots) continue;  // padding token, or a slot outside the cache
-    const int64_t row = idx[u] / groups_per_row;
-    const int in_row = (int)(idx[u] - row * groups_per_row);
-    const int head = in_row / p.groups_per_head;
-    const int group = in_row - head * p.groups_per_head;
-    const bool is_v = row & 1;
-    const int64_t blk = slot[u] / p.block_size;
-    const int64_t off = slot[u] - blk * p.block_size;
+  const int64_t idx = (int64_t)blockIdx.x * kFp4Lanes + threadIdx.x;
+  const int64_t at_group = min(idx, p.total_groups - 1);   // lanes past the end read the last group and drop it
+  const int64_t row = at_group / groups_per_row;           // token * 2 + (0 = K, 1 = V)
+  const int in_row = (int)(at_group - row * groups_per_row);
+  const int64_t token = row >> 1;
+  const int64_t slot = p.slot_mapping[token];
+  const char *src = ((row & 1) ? p.value + token * p.value_stride_bytes : p.key + token * p.key_stride_bytes) +
+                    (int64_t)in_row * 32;
+  const uint4 lo = load16_stream(src);
+  const uint4 hi = load16_stream(src + 16);
+  __builtin_amdgcn_sched_barrier(0);   // keeps the loads above the tests of the slot
+  if (idx >= p.total_groups) return;
+  if (slot < 0 || slot >= p.num_slots) return;  // padding token, or a slot outside the cache
+  const int head = in_row / p.groups_per_head;
+  const int group = in_row - head * p.groups_per_head;
+  const bool is_v = row & 1;
+  const int64_t blk = slot / p.block_size;
+  const int64_t off = slot - blk * p.block_size;
 
-    float x[16];
-    {
-      float a[8], b[8];
-      unpack8<T>(lo[u], a);
-      unpack8<T>(hi[u], b);
+  float x[16];
+  {
+    float a[8], b[8];
+    unpack8<T>(lo, a);
+    unpack8<T>(hi, b);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        x[j] = a[j];
-        x[8 + j] = b[j];
-      }
+    for (int j = 0; j < 8; ++j) {
+      x[j] = a[j];
+      x[8 + j] = b[j];
     }
-    float amax = 0.f;
-#pragma unroll
-    for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(x[j]));  // a NaN never becomes the maximum
-
-    // scale = e4m3(amax / 6), saturating; SF = the value that byte decodes to
-    const float sf = __builtin_amdgcn_fmed3f(amax * 0.16666667163372039794921875f, 0.0f, 448.0f);
-    const uint32_t code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(sf, 0.0f, 0, false) & 0xffu;
-    const float SF = __builtin_amdgcn_cvt_f32_fp8((int)code, 0);
-    const float inv = (SF != 0.0f) ? 1.0f / SF : 0.0f;
-
-    uint32_t w0 = 0, w1 = 0;
-    w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[0] * inv, x[1] * inv, 1.0f, 0);
-    w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[2] * inv, x[3] * inv, 1.0f, 1);
-    w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[4] * inv, x[5] * inv, 1.0f, 2);
-    w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[6] * inv, x[7] * inv, 1.0f, 3);
-    w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[8] * inv, x[9] * inv, 1.0f, 0);
-    w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[10] * inv, x[11] * inv, 1.0f, 1);
-    w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[12] * inv, x[13] * inv, 1.0f, 2);
-    w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[14] * inv, x[15] * inv, 1.0f, 3);
-
-    uint8_t *cache = is_v ? p.value_cache : p.key_cache;
-    uint8_t *scales = is_v ? p.value_scale_cache : p.key_scale_cache;
-    const int64_t at = blk * p.block_stride + off * p.page_stride + (int64_t)head * p.head_stride;
-    const int64_t sat = blk * (p.block_stride / 8) + off * (p.page_stride / 8) + (int64_t)head * (p.head_stride / 8);
-    store8_stream(cache + at + (int64_t)group * 8, make_uint2(w0, w1));
-    ((ARCTIC_GLOBAL uint8_t *)scales)[sat + group] = (uint8_t)code;
   }
+  float amax = 0.f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(x[j]));  // a NaN never becomes the maximum
+
+  // scale = e4m3(amax / 6), saturating; SF = the value that byte decodes to
+  const float sf = __builtin_amdgcn_fmed3f(amax * 0.16666667163372039794921875f, 0.0f, 448.0f);
+  const uint32_t code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(sf, 0.0f, 0, false) & 0xffu;
+  const float SF = __builtin_amdgcn_cvt_f32_fp8((int)code, 0);
+  const float inv = (SF != 0.0f) ? 1.0f / SF : 0.0f;
+
+  uint32_t w0 = 0, w1 = 0;
+  w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[0] * inv, x[1] * inv, 1.0f, 0);
+  w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[2] * inv, x[3] * inv, 1.0f, 1);
+  w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[4] * inv, x[5] * inv, 1.0f, 2);
+  w0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w0, x[6] * inv, x[7] * inv, 1.0f, 3);
+  w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[8] * inv, x[9] * inv, 1.0f, 0);
+  w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[10] * inv, x[11] * inv, 1.0f, 1);
+  w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[12] * inv, x[13] * inv, 1.0f, 2);
+  w1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w1, x[14] * inv, x[15] * inv, 1.0f, 3);
+
+  uint8_t *cache = is_v ? p.value_cache : p.key_cache;
+  uint8_t *scales = is_v ? p.value_scale_cache : p.key_scale_cache;
+  const int64_t at = blk * p.block_stride + off * p.page_stride + (int64_t)head * p.head_stride;
+  const int64_t sat = blk * (p.block_stride / 8) + off * (p.page_stride / 8) + (int64_t)head * (p.head_stride / 8);
+  store8_stream(cache + at + (int64_t)group * 8, make_uint2(w0, w1));
+  ((ARCTIC_GLOBAL uint8_t *)scales)[sat + group] = (uint8_t)code;
 }
 
 }  // namespace arctic
@@ -169,40 +158,13 @@ extern "C" int arctic_reshape_and_cache_flash_fp4(
   p.num_slots = num_blocks > 0 ? num_blocks * (int64_t)block_size : INT64_MAX;
   hipStream_t s = (hipStream_t)stream;
   // One group per lane in workgroups of one wave: nothing is shared between lanes, and at 8192 tokens and beyond
-  // single-wave workgroups ran 1 to 1.5 % faster than 256-lane ones (equal below).  The measurement build also has
-  // other workgroup sizes (ARCTIC_FP4_LANES) and 2 or 4 groups per lane (ARCTIC_FP4_GROUPS); all measured slower.
-  int per_lane = 1, lanes = 64;
-#ifdef ARCTIC_TUNING
-  if (const char *e = getenv("ARCTIC_FP4_GROUPS")) per_lane = atoi(e);
-  if (const char *e = getenv("ARCTIC_FP4_LANES")) lanes = atoi(e);
-  if (per_lane != 1) lanes = 256;
-#endif
-  const int64_t per_workgroup = (int64_t)lanes * per_lane;
-  const int64_t grid = (p.total_groups + per_workgroup - 1) / per_workgroup;
+  // single-wave workgroups ran 1 to 1.5 % faster than 256-lane ones (equal below); 512 and 1024 lanes and two or
+  // four groups per lane all measured slower.
+  const int64_t grid = (p.total_groups + kFp4Lanes - 1) / kFp4Lanes;
   if (grid > 0x7fffffffLL) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: too many tokens", fn);
-#define ARCTIC_FP4_LAUNCH(G, LANES)                                                                          \
-  do {                                                                                                       \
-    if (dtype == ARCTIC_DTYPE_BF16)                                                                          \
-      hipLaunchKernelGGL((kv_write_fp4_kernel<BF16, G, LANES>), dim3((unsigned)grid), dim3(LANES), 0, s, p); \
-    else                                                                                                     \
-      hipLaunchKernelGGL((kv_write_fp4_kernel<F16, G, LANES>), dim3((unsigned)grid), dim3(LANES), 0, s, p);  \
-  } while (0)
-  switch (per_workgroup) {
-#ifdef ARCTIC_TUNING
-    case 128: ARCTIC_FP4_LAUNCH(1, 128); break;
-    case 256: ARCTIC_FP4_LAUNCH(1, 256); break;
-    case 512:
-      if (per_lane == 2) ARCTIC_FP4_LAUNCH(2, 256);
-      else ARCTIC_FP4_LAUNCH(1, 512);
-      break;
-    case 1024:
-      if (per_lane == 4) ARCTIC_FP4_LAUNCH(4, 256);
-      else ARCTIC_FP4_LAUNCH(1, 1024);
-      break;
-#endif
-    case 64: ARCTIC_FP4_LAUNCH(1, 64); break;
-    default: return fail(ARCTIC_ERR_UNSUPPORTED, "%s: no kernel built for %d lanes x %d groups", fn, lanes, per_lane);
-  }
-#undef ARCTIC_FP4_LAUNCH
+  if (dtype == ARCTIC_DTYPE_BF16)
+    hipLaunchKernelGGL((kv_write_fp4_kernel<BF16>), dim3((unsigned)grid), dim3(kFp4Lanes), 0, s, p);
+  else
+    hipLaunchKernelGGL((kv_write_fp4_kernel<F16>), dim3((unsigned)grid), dim3(kFp4Lanes), 0, s, p);
   return check_launch(fn);
 }

@@ -13,7 +13,6 @@
 
 #include <algorithm>
 #include <cstdint>
-#include <cstdlib>
 
 #include "common.hpp"
 
@@ -106,14 +105,12 @@ struct HalfElem {
 // kVec: the body of a row, from its first 16-byte boundary on, is read in 16-byte chunks; the elements in front of
 // that boundary (a row pitch that is no multiple of 16 bytes puts every row somewhere else), those behind the last
 // whole chunk, and everything when !kVec (a pointer that is not even element-aligned) are read one by one.
-// kUnroll chunks per lane form a batch; kPipelined: the next batch is requested before the current one is looked at;
-// kStaggered: the odd waves take half a batch on its own first, so that neighbouring waves are half a batch apart;
+// kUnroll chunks per lane form a batch;
 // kLockstep: a workgroup barrier (no memory wait) behind every batch's requests, so that every wave of the row has
 // asked for batch k before any wave asks for batch k + 1 (a CU serves its oldest wave first: without the barrier the
 // oldest wave runs through all its batches before the youngest gets its first one in).
 // kHead: rows may start between two 16-byte boundaries (without it the host has checked that none does).
-template <typename Elem, bool kVec, int kUnroll = 4, bool kPipelined = false, bool kStaggered = false,
-          bool kLockstep = false, bool kHead = false>
+template <typename Elem, bool kVec, int kUnroll = 4, bool kLockstep = false, bool kHead = false>
 __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ out, const char *__restrict__ in,
                                                           int64_t row_stride_bytes, int cols, int64_t max_index) {
   __shared__ uint64_t wave_key[16];
@@ -179,18 +176,7 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
         if (c < chunks) look_at_chunk(c, raw[u]);
       }
     };
-    if constexpr (kPipelined) {
-      uint4 cur[kUnroll], nxt[kUnroll];
-      int c0 = threadIdx.x;
-      request(c0, cur);
-      while (c0 < chunks) {
-        request(c0 + stride, nxt);
-        look_at(c0, cur);
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) cur[u] = nxt[u];
-        c0 += stride;
-      }
-    } else if constexpr (kLockstep) {
+    if constexpr (kLockstep) {
       const int batches = (chunks + stride - 1) / stride;   // the same for every wave, as the barrier needs it
       int c0 = threadIdx.x;
       for (int b = 0; b < batches; ++b, c0 += stride) {
@@ -203,23 +189,6 @@ __global__ __launch_bounds__(1024) void row_argmax_kernel(int64_t *__restrict__ 
       }
     } else {
       int c0 = threadIdx.x;
-      if constexpr (kStaggered) {
-        if ((threadIdx.x >> 6) & 1) {
-          constexpr int kLead = kUnroll / 2;
-          uint4 lead[kLead];
-#pragma unroll
-          for (int u = 0; u < kLead; ++u) {
-            const int c = c0 + u * (int)blockDim.x;
-            if (c < chunks) lead[u] = load16_stream(body + (int64_t)c * 16);
-          }
-#pragma unroll
-          for (int u = 0; u < kLead; ++u) {
-            const int c = c0 + u * (int)blockDim.x;
-            if (c < chunks) look_at_chunk(c, lead[u]);
-          }
-          c0 += kLead * (int)blockDim.x;
-        }
-      }
       for (; c0 < chunks; c0 += stride) {
         uint4 raw[kUnroll];
         request(c0, raw);
@@ -289,35 +258,6 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
   int threads = (int)std::min<int64_t>(1024, std::max<int64_t>(64, ((cols / per_chunk / 4 + 63) / 64) * 64));
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)rows), block((unsigned)threads);
-#ifdef ARCTIC_TUNING
-  // measurement build: ARCTIC_ARGMAX_VARIANT = 1 pipelined batches of 4, 2 batches of 8, 3 pipelined batches of 8,
-  // 4 pipelined batches of 2, 5 batches of 2, 6 batches of 4 with the odd waves half a batch ahead, 7 batches of 1; + 8: half the lanes
-  int variant = 0;
-  if (const char *e = getenv("ARCTIC_ARGMAX_VARIANT")) variant = atoi(e);
-  if (variant & 8) threads = std::max(64, threads / 2);
-  variant &= ~8;   // + 16: a barrier behind every batch's requests (batches of 4, 2 or 1: 16, 17, 18)
-#define ARCTIC_ARGMAX_VEC(ELEM)                                                                                          \
-  do {                                                                                                                   \
-    const dim3 b((unsigned)threads);                                                                                     \
-    if (!aligned_rows) { /* the variants are built for aligned rows */                                                   \
-      hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false, false, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); \
-      break;                                                                                                             \
-    }                                                                                                                    \
-    switch (variant) {                                                                                                   \
-      case 1: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
-      case 2: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 8, false>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
-      case 3: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 8, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
-      case 4: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 2, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
-      case 5: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 2, false>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
-      case 6: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
-      case 7: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 1, false>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
-      case 16: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
-      case 17: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 2, false, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
-      case 18: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 1, false, false, true>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
-      default: hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false>), grid, b, 0, s, out, (const char *)logits, stride_bytes, cols, max_index); break; \
-    }                                                                                                                    \
-  } while (0)
-#else
   // Launches of about one and a half to three workgroups per CU (the 256 CUs of this GPU; a decode batch of a few
   // hundred rows) keep their waves in step, a chunk at a time: the two workgroups of a CU then finish together with
   // little left to do, 5 % faster at 384 and 512 rows.  With fewer rows a wave needs four chunks in flight to cover
@@ -326,19 +266,18 @@ extern "C" int arctic_argmax_clamp(int64_t *out, const void *logits, int64_t row
 #define ARCTIC_ARGMAX_VEC(ELEM)                                                                                   \
   do {                                                                                                            \
     if (!aligned_rows && lockstep)                                                                                \
-      hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 1, false, false, true, true>), grid, block, 0, s, out,    \
+      hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 1, true, true>), grid, block, 0, s, out,    \
                          (const char *)logits, stride_bytes, cols, max_index);                                    \
     else if (!aligned_rows)                                                                                       \
-      hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false, false, false, true>), grid, block, 0, s, out,   \
+      hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 4, false, true>), grid, block, 0, s, out,   \
                          (const char *)logits, stride_bytes, cols, max_index);                                    \
     else if (lockstep)                                                                                            \
-      hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 1, false, false, true>), grid, block, 0, s, out,          \
+      hipLaunchKernelGGL((row_argmax_kernel<ELEM, true, 1, true>), grid, block, 0, s, out,          \
                          (const char *)logits, stride_bytes, cols, max_index);                                    \
     else                                                                                                          \
       hipLaunchKernelGGL((row_argmax_kernel<ELEM, true>), grid, block, 0, s, out, (const char *)logits,           \
                          stride_bytes, cols, max_index);                                                          \
   } while (0)
-#endif
 #define ARCTIC_ARGMAX_LAUNCH(ELEM)                                                                          \
   do {                                                                                                      \
     if (vec)                                                                                                \

@@ -16,7 +16,6 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
-#include <cstdlib>
 
 #include "common.hpp"
 
@@ -55,7 +54,7 @@ struct Unit<2> { typedef unsigned short type; };
 template <>
 struct Unit<1> { typedef unsigned char type; };
 
-template <int kBytes, int kGatherThreads>
+template <int kBytes>
 __device__ __forceinline__ void move_units(const char *src, char *dst, int64_t first, int64_t end) {
   typedef typename Unit<kBytes>::type U;
   typedef const U ARCTIC_GLOBAL *SrcPtr;
@@ -63,23 +62,23 @@ __device__ __forceinline__ void move_units(const char *src, char *dst, int64_t f
   U v[kGatherUnroll];
 #pragma unroll
   for (int k = 0; k < kGatherUnroll; ++k) {
-    const int64_t u = first + (int64_t)k * kGatherThreads;
+    const int64_t u = first + (int64_t)k * kGatherLanes;
     if (u < end) v[k] = __builtin_nontemporal_load((SrcPtr)(src + u * kBytes));
   }
 #pragma unroll
   for (int k = 0; k < kGatherUnroll; ++k) {
-    const int64_t u = first + (int64_t)k * kGatherThreads;
+    const int64_t u = first + (int64_t)k * kGatherLanes;
     if (u < end) __builtin_nontemporal_store(v[k], (DstPtr)(dst + u * kBytes));
   }
 }
 
-template <typename Index, int kGatherThreads>
-__global__ __launch_bounds__(kGatherThreads) void row_gather_kernel(GatherTable tab, const Index *__restrict__ indices,
+template <typename Index>
+__global__ __launch_bounds__(kGatherLanes) void row_gather_kernel(GatherTable tab, const Index *__restrict__ indices,
                                                                     int64_t num_indices, int64_t num_indexed_rows,
                                                                     int scatter) {
   // the 1024 units of this workgroup may straddle tensors; each tensor's share is moved in turn
-  const int64_t begin = (int64_t)blockIdx.x * (kGatherThreads * kGatherUnroll);
-  const int64_t end = begin + kGatherThreads * kGatherUnroll;
+  const int64_t begin = (int64_t)blockIdx.x * (kGatherLanes * kGatherUnroll);
+  const int64_t end = begin + kGatherLanes * kGatherUnroll;
   // the grid's second dimension holds at most 65535 rows; beyond that a workgroup takes several
   for (int64_t row = blockIdx.y; row < num_indices; row += gridDim.y) {
     const int64_t idx = (int64_t)indices[row];
@@ -95,11 +94,11 @@ __global__ __launch_bounds__(kGatherThreads) void row_gather_kernel(GatherTable 
       const int64_t first = lo - tab.first_unit[t] + threadIdx.x;
       const int64_t last = hi - tab.first_unit[t];
       switch (tab.unit_shift[t]) {
-        case 4: move_units<16, kGatherThreads>(src, dst, first, last); break;
-        case 3: move_units<8, kGatherThreads>(src, dst, first, last); break;
-        case 2: move_units<4, kGatherThreads>(src, dst, first, last); break;
-        case 1: move_units<2, kGatherThreads>(src, dst, first, last); break;
-        default: move_units<1, kGatherThreads>(src, dst, first, last); break;
+        case 4: move_units<16>(src, dst, first, last); break;
+        case 3: move_units<8>(src, dst, first, last); break;
+        case 2: move_units<4>(src, dst, first, last); break;
+        case 1: move_units<2>(src, dst, first, last); break;
+        default: move_units<1>(src, dst, first, last); break;
       }
     }
   }
@@ -158,35 +157,17 @@ extern "C" int arctic_gather_rows(int num_tensors, const void *const *src, void 
     tab.end_unit[c] = units;
   }
   if (units == 0) return ARCTIC_OK;
-  int lanes = kGatherLanes;
-#ifdef ARCTIC_TUNING
-  if (const char *e = getenv("ARCTIC_GATHER_LANES")) lanes = atoi(e);   // measurement build: 64, 128, 512 or 1024
-#endif
-  const int64_t per_group = (int64_t)lanes * kGatherUnroll;
+  const int64_t per_group = (int64_t)kGatherLanes * kGatherUnroll;
   const int64_t groups = (units + per_group - 1) / per_group;
   if (groups > 0x7fffffffLL) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: rows too long", fn);
 
   const dim3 grid((unsigned)groups, (unsigned)std::min<int64_t>(num_indices, 65535));
   hipStream_t s = (hipStream_t)stream;
-#define ARCTIC_GATHER_LAUNCH(LANES)                                                                                \
-  do {                                                                                                             \
-    if (index_bytes == 8)                                                                                          \
-      hipLaunchKernelGGL((row_gather_kernel<int64_t, LANES>), grid, dim3(LANES), 0, s, tab,                        \
-                         (const int64_t *)indices, num_indices, num_indexed_rows, scatter);                        \
-    else                                                                                                           \
-      hipLaunchKernelGGL((row_gather_kernel<int32_t, LANES>), grid, dim3(LANES), 0, s, tab,                        \
-                         (const int32_t *)indices, num_indices, num_indexed_rows, scatter);                        \
-  } while (0)
-  switch (lanes) {
-#ifdef ARCTIC_TUNING
-    case 64: ARCTIC_GATHER_LAUNCH(64); break;
-    case 128: ARCTIC_GATHER_LAUNCH(128); break;
-    case 512: ARCTIC_GATHER_LAUNCH(512); break;
-    case 1024: ARCTIC_GATHER_LAUNCH(1024); break;
-#endif
-    case kGatherLanes: ARCTIC_GATHER_LAUNCH(kGatherLanes); break;
-    default: return fail(ARCTIC_ERR_UNSUPPORTED, "%s: no kernel built for %d lanes", fn, lanes);
-  }
-#undef ARCTIC_GATHER_LAUNCH
+  if (index_bytes == 8)
+    hipLaunchKernelGGL((row_gather_kernel<int64_t>), grid, dim3(kGatherLanes), 0, s, tab,
+                       (const int64_t *)indices, num_indices, num_indexed_rows, scatter);
+  else
+    hipLaunchKernelGGL((row_gather_kernel<int32_t>), grid, dim3(kGatherLanes), 0, s, tab,
+                       (const int32_t *)indices, num_indices, num_indexed_rows, scatter);
   return check_launch(fn);
 }

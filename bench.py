@@ -1149,462 +1149,6 @@ def bench_valu_rates(dev, steps):
     return out
 
 
-def load_tuning_library():
-    """libarctic_tuning_mi355x.so: the library's sources compiled with -DARCTIC_TUNING (`make -C
-    arcticinference_amd/csrc tuning`, also done by __graft_entry__.build()), in which environment variables select
-    kernel variants and launch shapes.  Only the sweeps below use it."""
-    import ctypes
-    path = os.path.join(ROOT, "arcticinference_amd", "libarctic_tuning_mi355x.so")
-    if not os.path.exists(path):
-        return None
-    lib = ctypes.CDLL(path)
-    vp, i64, i32, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
-    lib.arctic_sum_lstm.argtypes = [vp] * 9 + [i64, i32, i64, i64, i64, i64, f32, f32, f32, i32, i32, vp]
-    lib.arctic_sum_lstm.restype = i32
-    lib.arctic_reshape_and_cache_flash_bulk.argtypes = [vp, vp, i64, i64, vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i64,
-                                                        i64, i32, i32, vp]
-    lib.arctic_reshape_and_cache_flash_bulk.restype = i32
-    lib.arctic_argmax_clamp.argtypes = [vp, vp, i64, i32, i64, i64, i32, vp]
-    lib.arctic_argmax_clamp.restype = i32
-    return lib
-
-
-def bench_bulk_variants(dev, steps, placement="compact"):
-    """A/B of launch variants of the bulk write (70B shape, fp8) through the tuning build: the order of a batch's
-    stores and the next batch's loads, the workgroup shape, and the number of layer groups per token.  `placement`:
-    "compact" = 40 caches of 8192 blocks and the source allocated first in this process (one HBM region on an idle
-    GPU); "serving" = the headline's memory map (66 GiB of weights, an 80-layer pool of 65536 blocks, layers 40-79
-    written), where only the shapes and group counts that are candidates for the launch rule are timed;
-    "serving-8b" = 8192 tokens x 16 layers on the 8B model's map (8 GiB of weights, a 32-layer pool of 229376 blocks,
-    layers 16-31 written) and "compact-8b" the same launch with 16 caches of 8192 blocks alone on the GPU: the launch
-    at the line between the two workgroup shapes, 256 lanes x 4 chunks against 1024 lanes x 1."""
-    import ctypes
-    tuning = load_tuning_library()
-    if tuning is None:
-        return "libarctic_tuning_mi355x.so is not built"
-    if placement == "serving":
-        mem = ServingMemoryMap(dev, 66, 80, 40, 65536, 16, 8, 128, torch.uint8)
-        w = BulkWorkload("70B-SwiftKV", 16384, 40, 8, 128, 16, 65536, "fp8", 0.10, 2, 1.5, dev, bufs=mem.written_layers())
-    elif placement == "serving-8b":
-        mem = ServingMemoryMap(dev, 8, 32, 16, 229376, 16, 8, 128, torch.uint8)
-        w = BulkWorkload("8B-prefill-serving", 8192, 16, 8, 128, 16, 229376, "fp8", 0.0, 1, 1.5, dev, bufs=mem.written_layers())
-    elif placement == "compact-8b":
-        w = BulkWorkload("8B-prefill-compact", 8192, 16, 8, 128, 16, 8192, "fp8", 0.0, 1, 1.5, dev)
-    else:
-        w = BulkWorkload("70B-SwiftKV-compact", 16384, 40, 8, 128, 16, 8192, "fp8", 0.10, 2, 1.5, dev)
-    tab = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
-    kc, vc, ks, vs = tab(w.key_caches), tab(w.value_caches), tab(w.k_scales), tab(w.v_scales)
-    stream = torch.cuda.current_stream().cuda_stream
-
-    def launch():
-        rc = tuning.arctic_reshape_and_cache_flash_bulk(
-            w.keys.data_ptr(), w.values.data_ptr(), w.keys.stride(0), w.values.stride(0), kc, vc, ks, vs,
-            w.slots.data_ptr(), w.T, w.L, w.H, w.D, w.bs, w.key_caches[0].stride(0), w.NB, 2, 1, stream)
-        assert rc == 0
-
-    cases = [("as shipped (1024 lanes x 1 chunk, 2 groups of 20 layers, a batch's stores before the next batch's loads)", {}),
-             ("as shipped + a workgroup barrier (no memory wait) behind every batch's requests", {"ARCTIC_BULK_LOCKSTEP": "1"}),
-             ("512 lanes x 2 chunks", {"ARCTIC_BULK_SHAPE": "5"}),
-             ("512 lanes x 2 chunks, the next batch's loads before this batch's stores", {"ARCTIC_BULK_LOADS_FIRST": "1"}),
-             ("256 lanes x 4 chunks", {"ARCTIC_BULK_WIDE": "0"}),
-             ("one group of 40 layers per token", {"ARCTIC_BULK_GROUPS": "1"}),
-             ("4 groups of 10 layers per token", {"ARCTIC_BULK_GROUPS": "4"}),
-             ("8 groups of 5 layers per token", {"ARCTIC_BULK_GROUPS": "8"}),
-             ("512 lanes x 4 chunks", {"ARCTIC_BULK_SHAPE": "1"}),
-             ("512 lanes x 4 chunks, one group of 40 layers", {"ARCTIC_BULK_SHAPE": "1", "ARCTIC_BULK_GROUPS": "1"}),
-             ("1024 lanes x 2 chunks", {"ARCTIC_BULK_SHAPE": "2"}),
-             ("1024 lanes x 2 chunks, one group of 40 layers", {"ARCTIC_BULK_SHAPE": "2", "ARCTIC_BULK_GROUPS": "1"}),
-             ("1024 lanes x 4 chunks, one group of 40 layers", {"ARCTIC_BULK_SHAPE": "3", "ARCTIC_BULK_GROUPS": "1"}),
-             ("resident workgroups that stream across tokens (slots and row descriptors in LDS, straight-line batches), 2 per CU",
-              {"ARCTIC_BULK_RESIDENT": "2"}),
-             ("resident workgroups that stream across tokens, 3 per CU", {"ARCTIC_BULK_RESIDENT": "3"}),
-             ("resident workgroups that stream across tokens, 4 per CU", {"ARCTIC_BULK_RESIDENT": "4"}),
-             ("512 lanes x 2 chunks, 768 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "768"}),
-             ("512 lanes x 2 chunks, 1024 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "1024"}),
-             ("512 lanes x 2 chunks, 2048 workgroups that loop over the items", {"ARCTIC_BULK_PERSISTENT": "2048"})]
-    if placement.endswith("-8b"):
-        cases = [("as shipped (256 lanes x 4 chunks, 2 groups of 8 layers)", {}),
-                 ("the same groups as batches of 1024 lanes x 1 chunk", {"ARCTIC_BULK_WIDE": "1"}),
-                 ("1024 lanes x 1 chunk, one group of 16 layers", {"ARCTIC_BULK_WIDE": "1", "ARCTIC_BULK_GROUPS": "1"}),
-                 ("256 lanes x 4 chunks, one group of 16 layers", {"ARCTIC_BULK_GROUPS": "1"})]
-    if placement == "serving":
-        cases = [c for c in cases if "loop over" not in c[0] and "resident" not in c[0] and "8 groups" not in c[0]]
-        cases += [("512 lanes x 2 chunks, 4 groups of 10 layers", {"ARCTIC_BULK_SHAPE": "5", "ARCTIC_BULK_GROUPS": "4"}),
-                  ("256 lanes x 4 chunks, 5 groups of 8 layers", {"ARCTIC_BULK_WIDE": "0", "ARCTIC_BULK_GROUPS": "5"})]
-    out = {name: [] for name, _ in cases}
-    written, same = {}, {}
-    for _ in range(3):
-        for name, env in cases:
-            for k in ("ARCTIC_BULK_LOADS_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT", "ARCTIC_BULK_RESIDENT", "ARCTIC_BULK_LOCKSTEP"):
-                os.environ.pop(k, None)
-            os.environ.update(env)
-            # what the variant writes into the first and the last layer's caches, against the first variant's
-            probed = [w.key_caches[0], w.value_caches[0], w.key_caches[-1], w.value_caches[-1]]
-            for t in probed:
-                t.view(torch.int32).zero_()
-            for _ in range(3):
-                launch()
-            sums = [int(t.view(torch.int32).sum(dtype=torch.int64)) for t in probed]
-            written.setdefault("first", sums)
-            same[name] = same.get(name, True) and sums == written["first"]
-            out[name].append(round(statistics.mean(event_times_us(launch, max(10, steps // 4))), 1))
-    for k in ("ARCTIC_BULK_LOADS_FIRST", "ARCTIC_BULK_WIDE", "ARCTIC_BULK_GROUPS", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_PERSISTENT", "ARCTIC_BULK_RESIDENT", "ARCTIC_BULK_LOCKSTEP"):
-        os.environ.pop(k, None)
-    return {name: {"kernel_us_rounds": v, "GBps": round(w.bytes / statistics.mean(v) / 1e3),
-                   "hbm_frac": round(w.bytes / statistics.mean(v) / 1e3 / HBM_PEAK_GBS, 4),
-                   "writes_the_same_bytes": same[name]} for name, v in out.items()}
-
-
-def bench_launch_shapes(dev, steps):
-    """A/B of launch shapes of three smaller kernels through the tuning build, each variant captured in a HIP graph
-    over rotating buffer sets and replayed in turn, three rounds: (a) the fp4 cache write (lanes per workgroup, groups
-    per lane; 2048, 8192 and 32768 tokens, 16 layers of 8 x 128); (b) the row gather of swiftkv_select's five tensors
-    (lanes per workgroup; 512 and 2048 rows of the 70B shape); (c) the bulk fp8 write at a decode size (512 tokens x
-    16 layers into 32768-block caches; workgroups of 64 to 1024 lanes, chunks per lane, layer groups per token)."""
-    import ctypes
-    tuning = load_tuning_library()
-    if tuning is None:
-        return "libarctic_tuning_mi355x.so is not built"
-    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
-    tuning.arctic_reshape_and_cache_flash_fp4.argtypes = [vp, vp, i64, i64, vp, vp, vp, vp, vp, i64, i32, i32, i32, i64, i64,
-                                                          i64, i64, i32, vp]
-    tuning.arctic_reshape_and_cache_flash_fp4.restype = i32
-    tuning.arctic_gather_rows.argtypes = [i32, vp, vp, vp, vp, vp, vp, i32, i64, i64, i32, vp]
-    tuning.arctic_gather_rows.restype = i32
-    knobs = ("ARCTIC_FP4_LANES", "ARCTIC_FP4_GROUPS", "ARCTIC_GATHER_LANES", "ARCTIC_BULK_SHAPE", "ARCTIC_BULK_GROUPS")
-
-    def rounds(cases, call, per_graph):
-        """us per call of every case: one graph per case (the environment is read when a launch is captured)."""
-        graphs = []
-        for name, env in cases:
-            for k in knobs:
-                os.environ.pop(k, None)
-            os.environ.update(env)
-            call()
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                call()
-            graphs.append((name, graph))
-        for k in knobs:
-            os.environ.pop(k, None)
-        times = {name: [] for name, _ in cases}
-        for _ in range(3):
-            for name, graph in graphs:
-                warm_replays(graph.replay, min_ms=5.0)
-                times[name].append(round(statistics.median(event_times_us(graph.replay, max(10, steps // 4))) / per_graph, 2))
-        return times
-
-    out = {}
-    stream = lambda: torch.cuda.current_stream().cuda_stream
-    # (a) fp4 write
-    H, D, bs, L = 8, 128, 16, 16
-    g = torch.Generator(device=dev).manual_seed(5)
-    for T in (2048, 8192, 32768):
-        NB = 2 * T // bs
-        keys = [(torch.randn(T, H, D, generator=g, device=dev) * 0.5).to(torch.bfloat16) for _ in range(L)]
-        values = [(torch.randn(T, H, D, generator=g, device=dev) * 0.5).to(torch.bfloat16) for _ in range(L)]
-        kc, vc = ([torch.zeros(NB, bs, H, D // 2, dtype=torch.uint8, device=dev) for _ in range(L)] for _ in range(2))
-        ks, vs = ([torch.zeros(NB, bs, H, D // 16, dtype=torch.uint8, device=dev) for _ in range(L)] for _ in range(2))
-        slots = torch.randperm(NB * bs, generator=torch.Generator().manual_seed(5))[:T].to(dev)
-
-        def fp4():
-            for l in range(L):
-                rc = tuning.arctic_reshape_and_cache_flash_fp4(
-                    keys[l].data_ptr(), values[l].data_ptr(), H * D, H * D, kc[l].data_ptr(), vc[l].data_ptr(),
-                    ks[l].data_ptr(), vs[l].data_ptr(), slots.data_ptr(), T, H, D, bs, kc[l].stride(0), kc[l].stride(1),
-                    kc[l].stride(2), NB, 2, stream())
-                assert rc == 0, rc
-        cases = [("64 lanes, one group per lane (shipped)", {})] + \
-                [(f"{n} lanes, one group per lane", {"ARCTIC_FP4_LANES": str(n)}) for n in (128, 256, 512, 1024)] + \
-                [(f"256 lanes, {n} groups per lane", {"ARCTIC_FP4_GROUPS": str(n)}) for n in (2, 4)]
-        out[f"fp4_write_{T}_tokens_us_per_layer"] = rounds(cases, fp4, L)
-        del keys, values, kc, vc, ks, vs
-    # (b) row gather
-    hidden, kvw, sets = 8192, 40 * 1024, 4
-    for T in (512, 2048):
-        rn = lambda *s: torch.randn(*s, generator=g, device=dev).to(torch.bfloat16)
-        src = [[rn(T, hidden), rn(T, hidden), torch.arange(T, device=dev), rn(T, kvw), rn(T, kvw)] for _ in range(sets)]
-        dst = [[torch.empty_like(t) for t in s_] for s_ in src]
-        idx = torch.randperm(T, device=dev)
-
-        def gather():
-            for s_, d_ in zip(src, dst):
-                n = len(s_)
-                rc = tuning.arctic_gather_rows(
-                    n, (vp * n)(*[t.data_ptr() for t in s_]), (vp * n)(*[t.data_ptr() for t in d_]),
-                    (i64 * n)(*[t[0].numel() * t.element_size() for t in s_]),
-                    (i64 * n)(*[t.stride(0) * t.element_size() for t in s_]),
-                    (i64 * n)(*[t.stride(0) * t.element_size() for t in d_]), idx.data_ptr(), 8, T, T, 0, stream())
-                assert rc == 0, rc
-        cases = [("256 lanes (shipped)", {})] + [(f"{n} lanes", {"ARCTIC_GATHER_LANES": str(n)}) for n in (64, 128, 512, 1024)]
-        out[f"gather_rows_{T}_rows_us_per_call"] = rounds(cases, gather, sets)
-        del src, dst
-    # (c) bulk write at a decode size
-    sets = 8
-    ws = [BulkWorkload("decode", 512, 16, 8, 128, 16, 32768, "fp8", 0.0, 4, 1.5, dev)]
-    for i in range(1, sets):
-        ws.append(BulkWorkload("decode", 512, 16, 8, 128, 16, 32768, "fp8", 0.0, 4 + i, 1.5, dev, bufs=ws[0].bufs))
-    tab = lambda ts: (vp * len(ts))(*[t.data_ptr() for t in ts])
-
-    def bulk():
-        for w in ws:
-            rc = tuning.arctic_reshape_and_cache_flash_bulk(
-                w.keys.data_ptr(), w.values.data_ptr(), w.keys.stride(0), w.values.stride(0), tab(w.key_caches),
-                tab(w.value_caches), tab(w.k_scales), tab(w.v_scales), w.slots.data_ptr(), w.T, w.L, w.H, w.D, w.bs,
-                w.key_caches[0].stride(0), w.NB, 2, 1, stream())
-            assert rc == 0, rc
-    shapes = {4: "1024 x 1", 5: "512 x 2", 6: "256 x 2", 7: "256 x 1", 8: "512 x 1", 9: "64 x 4", 10: "64 x 8", 11: "128 x 4",
-              12: "128 x 8"}
-    cases = [("256 lanes x 4 chunks, 4 groups of 4 layers (shipped)", {})]
-    for shape, groups in ((4, 1), (4, 2), (5, 2), (8, 2), (6, 4), (7, 8), (9, 16), (9, 8), (10, 8), (10, 4), (11, 8), (11, 4),
-                          (12, 4), (12, 2)):
-        cases.append((f"{shapes[shape]} (lanes x chunks), {groups} groups of {16 // groups} layers",
-                      {"ARCTIC_BULK_SHAPE": str(shape), "ARCTIC_BULK_GROUPS": str(groups)}))
-    out["bulk_write_512_tokens_16_layers_us_per_call"] = rounds(cases, bulk, sets)
-    return out
-
-
-def bench_argmax_variants(dev, steps):
-    """A/B of the row-argmax kernel's loop shapes through the tuning build: 512 rows x 128256 bf16 logits (131 MB),
-    three rotating sets in one graph per variant, three rounds over all variants; results compared with torch's."""
-    tuning = load_tuning_library()
-    if tuning is None:
-        return "libarctic_tuning_mi355x.so is not built"
-    T, V, sets = 512, 128256, 3
-    g = torch.Generator(device=dev).manual_seed(8)
-    logits = [torch.randn(T, V, generator=g, device=dev).to(torch.bfloat16) for _ in range(sets)]
-    outs = [torch.empty(T, dtype=torch.int64, device=dev) for _ in range(sets)]
-    want = [torch.argmax(x, dim=-1).clamp_(0, V - 1) for x in logits]
-    nbytes = T * V * 2 + T * 8
-    cases = [(0, "batches of 4 chunks per lane, 1024 lanes (shipped for fewer than 257 and more than 768 rows)"), (1, "the same, next batch requested first"),
-             (2, "batches of 8"), (3, "batches of 8, next batch requested first"),
-             (4, "batches of 2, next batch requested first"), (5, "batches of 2"),
-             (6, "batches of 4, odd waves half a batch ahead of the even ones"),
-             (7, "batches of 1"),
-             (16, "batches of 4 with a workgroup barrier behind every batch's requests"),
-             (17, "batches of 2 with a workgroup barrier behind every batch's requests"),
-             (18, "batches of 1 with a workgroup barrier behind every batch's requests (shipped for 257 to 768 rows)"),
-             (24, "512 lanes, batches of 4 with a workgroup barrier behind every batch's requests"),
-             (9, "512 lanes, batches of 4, next batch first"),
-             (11, "512 lanes, batches of 8, next batch first")]
-
-    def run():
-        stream = torch.cuda.current_stream().cuda_stream
-        for i in range(sets):
-            assert tuning.arctic_argmax_clamp(outs[i].data_ptr(), logits[i].data_ptr(), T, V, V, V - 1, 2, stream) == 0
-
-    graphs, out = {}, {}
-    for code, what in cases:
-        os.environ["ARCTIC_ARGMAX_VARIANT"] = str(code)
-        run()
-        torch.cuda.synchronize()
-        ok = all(torch.equal(a, b) for a, b in zip(outs, want))
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            run()
-        graphs[code] = graph
-        out[str(code)] = {"variant": what, "equals_torch": ok, "us": []}
-    os.environ.pop("ARCTIC_ARGMAX_VARIANT", None)
-    for _ in range(3):
-        for code, graph in graphs.items():
-            warm_replays(graph.replay)
-            out[str(code)]["us"].append(round(statistics.mean(event_times_us(graph.replay, max(10, steps // 2))) / sets, 2))
-    for v in out.values():
-        m = statistics.mean(v["us"])
-        v.update({"us_per_call_graph_rounds": v.pop("us"), "GBps": round(nbytes / m / 1e3), "hbm_frac": round(nbytes / m / 1e3 / HBM_PEAK_GBS, 4)})
-    return out
-
-
-# ARCTIC_LSTM_VARIANT values of the tuning build (sum_lstm.hip): bits 0-2 = arithmetic / ordering variants,
-# bits 3-5 = launch shape, 66 = variant 2 with barriers between the request groups; "S<n>" = schedule n of the
-# staged kernel (ARCTIC_LSTM_STAGED)
-LSTM_VARIANTS = [
-    (0, "loads c f pc i o, one row per 512-lane workgroup, output gate after the second row sum"),
-    (1, "input gate loaded and consumed before forget gate and previous cell (c i f pc o)"),
-    (2, "output gate's sigmoid ahead of the second row sum (what the shapes outside the staged kernel take)"),
-    (3, "input gate first + output gate's sigmoid ahead of the second row sum"),
-    (4, "shared reciprocals: one for the forget and input gates, one for the state GELU and the output gate"),
-    (8, "two rows per workgroup, second row's loads issued behind the first row's"),
-    (11, "two rows per workgroup + input gate first + early output gate"),
-    (16, "two 16-byte chunks per lane (256 lanes per row)"),
-    (24, "two chunks per lane and two rows per workgroup"),
-    (34, "8-byte chunks, 1024 lanes per row (twice the waves, half the work each), early output gate"),
-    (66, "the row's gates requested gate by gate: a workgroup barrier between the groups of requests"),
-    ("S0", "staged kernel, every chunk requested at once, outputs and previous cell through the caches"),
-    ("S1", "staged kernel: cell gate first; forget gate's s behind the first sum of squares; rest of the forget gate, "
-           "previous cell and input gate behind the candidate's GELU; output gate behind the forget gate's part and "
-           "consumed last"),
-    ("S2", "the same + scale / shift vectors requested where they are needed, not ahead of the row"),
-    ("S3", "the same + streaming stores of both outputs"),
-    ("S4", "the same + streaming load of the previous cell"),
-    ("S12", "the same + a workgroup barrier (no memory wait) behind the requests that follow the candidate's GELU "
-            "(shipped)"),
-    ("S11", "S4 + that barrier behind the first requests instead"),
-    ("S13", "S4 + that barrier behind the output gate's requests instead"),
-    ("S14", "S4 + all three barriers"),
-    ("S15", "S4 + the barriers behind the last two groups of requests"),
-    ("S5", "S4 with the output gate's sigmoid ahead of the second row sum"),
-    ("S6", "S4 with other request points: 2 | 4 | 7 | 9 chunks out"),
-    ("S7", "S4 with other request points: 3 | 4 | 7 | 7"),
-    ("S8", "S4 with other request points: 2 | 3 | 5 | 7"),
-    ("S9", "S4 with other request points: 5 | 7 | 9 | 9"),
-    ("S10", "every chunk requested at once, with the streaming stores and the streaming load of the previous cell"),
-]
-
-
-def bench_lstm_timeline(dev, steps):
-    """When the waves of one sum_lstm launch reach eight points of their life, from time stamps (the GPU's constant
-    100 MHz clock) that the measurement build's staged kernel writes: the shipped schedule next to the same kernel
-    with every chunk requested at once.  512 x 4096 bf16, eight rotating sets x three chained steps in one HIP graph;
-    the stamps of the graph's last launch are read, in microseconds after its first wave's start.  The stamps slow
-    a launch down by about a microsecond, so they show the order of events, not the operator's speed."""
-    import numpy as np
-    tuning = load_tuning_library()
-    if tuning is None:
-        return "libarctic_tuning_mi355x.so is not built"
-    T, Hd, sets = 512, 4096, 8
-    g = torch.Generator(device=dev).manual_seed(3)
-    rn = lambda *s: torch.randn(*s, generator=g, device=dev).to(torch.bfloat16)
-    S = [[rn(T, 4 * Hd) for _ in range(3)] for _ in range(sets)]
-    Z = [[rn(T, 4 * Hd) for _ in range(3)] for _ in range(sets)]
-    C0 = [rn(T, Hd) for _ in range(sets)]
-    vec = lambda m: (m + 0.02 * torch.randn(Hd, generator=g, device=dev)).to(torch.bfloat16)
-    w_cell, b_cell, w_state, b_state = vec(1.0), vec(0.0), vec(1.0), vec(0.0)
-    ST = [[torch.empty(T, Hd, dtype=torch.bfloat16, device=dev) for _ in range(3)] for _ in range(sets)]
-    CE = [[torch.empty(T, Hd, dtype=torch.bfloat16, device=dev) for _ in range(3)] for _ in range(sets)]
-    trace = torch.zeros(T * 8 * 8, dtype=torch.int64, device=dev)
-    os.environ["ARCTIC_LSTM_TRACE"] = hex(trace.data_ptr())
-
-    def run_all():
-        stream = torch.cuda.current_stream().cuda_stream
-        for i in range(sets):
-            cell = C0[i]
-            for k in range(3):
-                rc = tuning.arctic_sum_lstm(ST[i][k].data_ptr(), CE[i][k].data_ptr(), S[i][k].data_ptr(), Z[i][k].data_ptr(),
-                                            cell.data_ptr(), w_cell.data_ptr(), b_cell.data_ptr(), w_state.data_ptr(),
-                                            b_state.data_ptr(), T, Hd, 4 * Hd, 4 * Hd, Hd, Hd, 1.0, 1e-6, 1e-6, 0, 2, stream)
-                assert rc == 0
-                cell = CE[i][k]
-
-    points = ["wave started", "first requests out", "cell gate in, squares summed", "first row sum known",
-              "forget gate, previous cell, input gate in; new cell stored", "second row sum known", "state GELU done",
-              "output gate in; state stored"]
-    out = {}
-    for code, what in ((100, "every chunk requested at once"), (112, "requests in stages (shipped schedule)")):
-        os.environ["ARCTIC_LSTM_STAGED"] = str(code)
-        run_all()
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            run_all()
-        warm_replays(graph.replay)
-        us = statistics.mean(event_times_us(graph.replay, max(10, steps // 4))) / (sets * 3)
-        t = trace.cpu().numpy().reshape(T, 8, 8).astype(np.float64)
-        t = (t - t[:, :, 0].min()) * 0.01   # ticks of 10 ns -> us after the first wave's start
-        rows = {}
-        for k, name in enumerate(points):
-            lower, upper = t[:T // 2, :, k].ravel(), t[T // 2:, :, k].ravel()
-            rows[name] = {"older_workgroup_of_a_cu_median_p90": [round(float(np.median(lower)), 2), round(float(np.percentile(lower, 90)), 2)],
-                          "younger_workgroup_of_a_cu_median_p90": [round(float(np.median(upper)), 2), round(float(np.percentile(upper, 90)), 2)],
-                          "all_waves_max": round(float(t[:, :, k].max()), 2)}
-        out[what] = {"us_per_call_graph_with_stamps": round(us, 2), "us_after_first_wave_start": rows}
-        del graph
-    os.environ.pop("ARCTIC_LSTM_STAGED", None)
-    os.environ.pop("ARCTIC_LSTM_TRACE", None)
-    return out
-
-
-def bench_lstm_variants(dev, steps):
-    """A/B of sum_lstm kernel variants on the speculator workload (512 x 4096 bf16, eight rotating buffer sets, three
-    chained steps per set inside one HIP graph), all in this process.  Each variant is also compared with the
-    first variant's outputs: share of bit-identical elements and largest difference."""
-    tuning = load_tuning_library()
-    if tuning is None:
-        return "libarctic_tuning_mi355x.so is not built"
-    T, Hd, sets = 512, 4096, 8
-    g = torch.Generator(device=dev).manual_seed(3)
-    rn = lambda *s: torch.randn(*s, generator=g, device=dev).to(torch.bfloat16)
-    S = [[rn(T, 4 * Hd) for _ in range(3)] for _ in range(sets)]
-    Z = [[rn(T, 4 * Hd) for _ in range(3)] for _ in range(sets)]
-    C0 = [rn(T, Hd) for _ in range(sets)]
-    vec = lambda m: (m + 0.02 * torch.randn(Hd, generator=g, device=dev)).to(torch.bfloat16)
-    w_cell, b_cell, w_state, b_state = vec(1.0), vec(0.0), vec(1.0), vec(0.0)
-    sw = 0.5 ** (0.5 / 3)
-    alpha = ((1 - sw * sw) * (Hd / 2)) ** 0.5 / sw
-    ST = [[torch.empty(T, Hd, dtype=torch.bfloat16, device=dev) for _ in range(3)] for _ in range(sets)]
-    CE = [[torch.empty(T, Hd, dtype=torch.bfloat16, device=dev) for _ in range(3)] for _ in range(sets)]
-    per_call = 22 * Hd * T
-
-    def run_all():
-        stream = torch.cuda.current_stream().cuda_stream
-        for i in range(sets):
-            cell = C0[i]
-            for k in range(3):
-                rc = tuning.arctic_sum_lstm(ST[i][k].data_ptr(), CE[i][k].data_ptr(), S[i][k].data_ptr(), Z[i][k].data_ptr(),
-                                            cell.data_ptr(), w_cell.data_ptr(), b_cell.data_ptr(), w_state.data_ptr(),
-                                            b_state.data_ptr(), T, Hd, 4 * Hd, 4 * Hd, Hd, Hd, alpha, 1e-6, 1e-6, 0, 2, stream)
-                assert rc == 0
-                cell = CE[i][k]
-
-    floor = load_floor_kernels()
-    out, base = {}, None
-    rounds = 3   # every variant is timed in each round, so drift over the run shows up as spread, not as a ranking
-    graphs = {}
-    for code, what in LSTM_VARIANTS:
-        os.environ.pop("ARCTIC_LSTM_STAGED", None)
-        if str(code).startswith("S"):
-            os.environ["ARCTIC_LSTM_STAGED"] = str(code)[1:]
-        else:
-            os.environ["ARCTIC_LSTM_VARIANT"] = str(code)
-        run_all()
-        torch.cuda.synchronize()
-        got = [t.clone() for i in range(sets) for t in (ST[i][2], CE[i][2])]
-        if base is None:
-            base = got
-        same = sum(int((a == b).sum()) for a, b in zip(got, base)) / sum(a.numel() for a in got)
-        worst = max(float((a.float() - b.float()).abs().max()) for a, b in zip(got, base))
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            run_all()
-        graphs[code] = graph
-        out[str(code)] = {"variant": what, "bit_identical_to_variant_0": round(same, 5), "max_abs_diff": worst, "us": []}
-    os.environ.pop("ARCTIC_LSTM_VARIANT", None)
-    os.environ.pop("ARCTIC_LSTM_STAGED", None)
-    if floor is not None:
-        OS = [torch.empty(T, Hd, dtype=torch.bfloat16, device=dev) for _ in range(2)]
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            stream = torch.cuda.current_stream().cuda_stream
-            for i in range(sets):
-                for k in range(3):
-                    floor.floor_lstm_traffic(S[i][k].data_ptr(), Z[i][k].data_ptr(), C0[i].data_ptr(), OS[0].data_ptr(),
-                                             OS[1].data_ptr(), T, Hd, stream)
-        graphs["floor"] = graph
-        out["floor"] = {"variant": "lstm_traffic_kernel: the same loads and stores requested at once, no arithmetic", "us": []}
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            stream = torch.cuda.current_stream().cuda_stream
-            for i in range(sets):
-                for k in range(3):
-                    floor.floor_lstm_traffic_staged(S[i][k].data_ptr(), Z[i][k].data_ptr(), C0[i].data_ptr(),
-                                                    OS[0].data_ptr(), OS[1].data_ptr(), T, Hd, stream)
-        graphs["floor_staged"] = graph
-        out["floor_staged"] = {"variant": "lstm_traffic_staged_kernel: the same loads and stores requested in the shipped "
-                                          "kernel's stages, no arithmetic", "us": []}
-    for _ in range(rounds):
-        for key, graph in graphs.items():
-            warm_replays(graph.replay)
-            us = event_times_us(graph.replay, max(10, steps // 2))
-            out[str(key)]["us"].append(round(statistics.mean(us) / (sets * 3), 3))
-    for v in out.values():
-        v["us_per_call_graph_rounds"] = v.pop("us")
-        m = statistics.mean(v["us_per_call_graph_rounds"])
-        v["us_per_call_graph"] = round(m, 2)
-        v["hbm_frac_graph"] = round(per_call / m / 1e3 / HBM_PEAK_GBS, 4)
-    return out
-
-
 def calibration_copy(dev):
     """A plain 1 GiB device copy: known bytes that a counter run of the same command scales FETCH_SIZE / WRITE_SIZE by."""
     src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
@@ -1648,22 +1192,6 @@ def main():
     ap.add_argument("--only", choices=sorted(ONLY), default=None,
                     help="instead of the benchmark, run one of the extra measurements alone (for profiling it); "
                          "prints one JSON object")
-    ap.add_argument("--lstm-variants", action="store_true",
-                    help="instead of the benchmark, time the sum_lstm kernel variants of the tuning build against "
-                         "each other and against the traffic-only kernel; prints one JSON object")
-    ap.add_argument("--lstm-timeline", action="store_true",
-                    help="instead of the benchmark, print when the waves of a sum_lstm launch reach the stages of the "
-                         "kernel (time stamps written by the tuning build), with requests at once and in stages")
-    ap.add_argument("--argmax-variants", action="store_true",
-                    help="instead of the benchmark, time loop shapes of the row-argmax kernel through the tuning build")
-    ap.add_argument("--launch-shapes", action="store_true",
-                    help="instead of the benchmark, time launch shapes of the fp4 write, the row gather and the bulk "
-                         "write at a decode size through the tuning build")
-    ap.add_argument("--bulk-variants", nargs="?", const="compact", default=None,
-                    choices=["compact", "serving", "compact-8b", "serving-8b"],
-                    help="instead of the benchmark, time launch variants of the bulk write through the tuning build, "
-                         "in the compact placement (default) or on the headline's serving memory map; prints one "
-                         "JSON object")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) so that a counter run of this "
                          "command can scale FETCH_SIZE / WRITE_SIZE")
@@ -1683,24 +1211,6 @@ def main():
 
     if args.placement_sweep:
         print(json.dumps({"placement_sweep": placement_sweep(ops, dev, max(5, args.steps // 5))}), flush=True)
-        return
-    if args.lstm_variants:
-        print(json.dumps({"sum_lstm_variants": bench_lstm_variants(dev, args.steps)}), flush=True)
-        return
-    if args.lstm_timeline:
-        print(json.dumps({"sum_lstm_wave_timeline": bench_lstm_timeline(dev, args.steps)}), flush=True)
-        return
-    if args.argmax_variants:
-        print(json.dumps({"row_argmax_variants": bench_argmax_variants(dev, args.steps)}), flush=True)
-        return
-    if args.launch_shapes:
-        print(json.dumps({"launch_shapes": bench_launch_shapes(dev, args.steps)}), flush=True)
-        return
-    if args.bulk_variants:
-        name = {"compact": "bulk_write_variants_compact_pool", "serving": "bulk_write_variants_serving_map",
-                "compact-8b": "bulk_write_variants_8b_compact_pool",
-                "serving-8b": "bulk_write_variants_8b_serving_map"}[args.bulk_variants]
-        print(json.dumps({name: bench_bulk_variants(dev, args.steps, args.bulk_variants)}), flush=True)
         return
     if args.only:
         if args.calibrate_copy:

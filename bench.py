@@ -36,6 +36,7 @@ import argparse
 import json
 import os
 import statistics
+import subprocess
 import sys
 import time
 
@@ -560,6 +561,94 @@ def bench_bulk_select(ops, dev, steps):
                 fn(i)
         warm_replays(graph.replay)
         out[name] = {"us_per_step_graph": round(statistics.median(event_times_us(graph.replay, max(10, steps // 2))) / sets, 2)}
+    return out
+
+
+def host_overhead_route(route, calls=3000):
+    """Host wall time per eager call with the GPU out of the picture: tiny inputs (4 tokens, 8 rows), so that a
+    kernel is over long before the host has issued the next one; `calls` calls are issued back to back and the
+    wall clock is divided by their number (one synchronisation in front, one behind, outside the clock).
+    route "ctypes": this package's py_custom_ops (Python shims over the C ABI).  route "torch_ext": the same
+    library behind a compiled torch extension, C++ from the dispatcher down (the file named by
+    ARCTIC_TORCH_EXT).  Runs in a process of its own: both routes define the arctic_inference namespace."""
+    dev = torch.device("cuda:0")
+    if route == "ctypes":
+        from arcticinference_amd import py_custom_ops as ops
+        assert ops.try_load_torch_library()
+        bulk, lstm, ln = ops.reshape_and_cache_flash_bulk, ops.sum_lstm, ops.speculator_ln
+    else:
+        torch.ops.load_library(os.environ["ARCTIC_TORCH_EXT"])
+        ns = torch.ops.arctic_inference
+        bulk, lstm, ln = ns.reshape_and_cache_flash_bulk, ns.sum_lstm_cuda, ns.speculator_ln_cuda
+
+    def per_call_us(f):
+        for _ in range(200):
+            f()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            t0 = time.perf_counter()
+            for _ in range(calls):
+                f()
+            t1 = time.perf_counter()
+            torch.cuda.synchronize()
+            us = (t1 - t0) * 1e6 / calls
+            best = us if best is None else min(best, us)
+        return round(best, 2)
+
+    out = {}
+    x = torch.randn(8, 4096, device=dev).to(torch.bfloat16)
+    s4 = torch.randn(8, 16384, device=dev).to(torch.bfloat16)
+    w = torch.ones(4096, device=dev, dtype=torch.bfloat16)
+    out["speculator_ln"] = per_call_us(lambda: ln(x, w, w, 1e-6))
+    out["sum_lstm"] = per_call_us(lambda: lstm(s4, s4, x, w, w, w, w, 1.0, 1e-6, 1e-6, False))
+    T, H, D, NB, bs = 4, 8, 128, 64, 16
+    for L in (16, 40):
+        keys = torch.randn(T, L * H * D, device=dev).to(torch.bfloat16)
+        values = torch.randn(T, L * H * D, device=dev).to(torch.bfloat16)
+        pool = [torch.zeros(2, NB, bs, H, D, dtype=torch.uint8, device=dev) for _ in range(L)]
+        kc, vc = [b[0] for b in pool], [b[1] for b in pool]
+        ks = [torch.ones((), device=dev) for _ in range(L)]
+        vs = [torch.ones((), device=dev) for _ in range(L)]
+        slots = torch.arange(T, device=dev)
+        out[f"reshape_and_cache_flash_bulk_{L}_layers"] = per_call_us(
+            lambda: bulk(keys, values, kc, vc, slots, "fp8", ks, vs, H, D))
+
+        # what the caller itself spends per step on the four lists it passes (llama_swiftkv.py:594-615: two views of
+        # every layer's cache tensor and two attribute reads), for scale
+        def caller_lists():
+            a, b, c, d = [], [], [], []
+            for l in range(L):
+                kv = pool[l]
+                a.append(kv[0])
+                b.append(kv[1])
+                c.append(ks[l])
+                d.append(vs[l])
+            return a, b, c, d
+        t0 = time.perf_counter()
+        for _ in range(300):
+            caller_lists()
+        out[f"caller_builds_its_four_lists_{L}_layers"] = round((time.perf_counter() - t0) * 1e6 / 300, 2)
+    return out
+
+
+def bench_host_overhead():
+    """Host microseconds per eager call through both integration routes, each measured in a child process."""
+    ext = os.path.join(ROOT, "oracle", "_ref", "arctic_torch_ext.so")
+    routes = {"route_1_py_custom_ops_ctypes": ("ctypes", {})}
+    if os.path.exists(ext):
+        routes["route_2_torch_extension_cpp"] = ("torch_ext", {"ARCTIC_TORCH_EXT": ext})
+    out = {"what": "host wall time per eager call in microseconds, tiny inputs (4 tokens / 8 rows), 3000 calls issued "
+                   "back to back, best of 3 rounds; the GPU work of a call is shorter than the host's"}
+    for name, (route, env) in routes.items():
+        proc = subprocess.run([sys.executable, os.path.abspath(__file__), "--host-overhead-route", route],
+                              capture_output=True, text=True, env=dict(os.environ, **env), timeout=300)
+        if proc.returncode != 0:
+            out[name] = "failed: " + (proc.stderr.strip().splitlines() or ["no output"])[-1]
+            continue
+        out[name] = json.loads(proc.stdout.strip().splitlines()[-1])
+    if "route_2_torch_extension_cpp" not in routes:
+        out["route_2_torch_extension_cpp"] = "oracle/_ref/arctic_torch_ext.so is not built (make -C oracle torch_ext)"
     return out
 
 
@@ -1174,6 +1263,7 @@ ONLY = {
     "bulk_write_and_select_decode_70b": lambda ops, dev, a: bench_bulk_select(ops, dev, a.steps),
     "swiftkv_select_decode_70b": lambda ops, dev, a: bench_row_gather(ops, dev, a.steps),
     "bulk_fp8_70b_tp_sharded_heads_compact_pool": lambda ops, dev, a: bench_bulk_tp_heads(ops, dev, a.steps),
+    "host_us_per_call": lambda ops, dev, a: bench_host_overhead(),
 }
 
 
@@ -1192,6 +1282,7 @@ def main():
     ap.add_argument("--only", choices=sorted(ONLY), default=None,
                     help="instead of the benchmark, run one of the extra measurements alone (for profiling it); "
                          "prints one JSON object")
+    ap.add_argument("--host-overhead-route", choices=["ctypes", "torch_ext"], default=None, help=argparse.SUPPRESS)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) so that a counter run of this "
                          "command can scale FETCH_SIZE / WRITE_SIZE")
@@ -1201,6 +1292,9 @@ def main():
                  "independent, so more GPUs only run the same kernel on their own share); use --gpus 1")
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+    if args.host_overhead_route:   # the child process of bench_host_overhead()
+        print(json.dumps(host_overhead_route(args.host_overhead_route)), flush=True)
+        return
 
     from arcticinference_amd import py_custom_ops as ops
     if not ops.try_load_torch_library():
@@ -1371,6 +1465,7 @@ def main():
         extras["bulk_write_and_select_decode_70b"] = bench_bulk_select(ops, dev, args.steps)
         torch.cuda.empty_cache()
         extras["suffix_decoding_cpu"] = bench_suffix_decoding()
+        extras["host_us_per_call"] = bench_host_overhead()
         log(f"extras: {extras}")
 
     result = {

@@ -294,9 +294,8 @@ def test_errors(ops):
 
 def test_layers_that_do_not_look_like_layer_0_are_turned_away(ops):
     """The kernel takes one block stride, block count and block size for all layers; a layer that differs, or a scale
-    that is not an fp32 device tensor, is an error here (the reference would write out of bounds).  A set of layers
-    that passed is remembered by its addresses, so the same wrong set must fail on every call, and a good set must
-    still work after a bad one."""
+    that is not an fp32 device tensor, is an error here (the reference would write out of bounds).  Every layer is
+    looked at on every call: the same wrong set must fail each time, and a good set must still work after a bad one."""
     case = make_bulk_case(T=6, L=3, H=2, D=64, bs=16, NB=4, kv_cache_dtype="fp8", seed=21)
     d = bulk_case_to(case, DEV)
     a = list(bulk_args(d))
@@ -311,5 +310,66 @@ def test_layers_that_do_not_look_like_layer_0_are_turned_away(ops):
         with pytest.raises(RuntimeError, match="at least 6 rows"):
             ops.reshape_and_cache_flash_bulk(a[0][:4], *a[1:])
         with pytest.raises(RuntimeError, match="384 columns"):
-            ops.reshape_and_cache_flash_bulk(a[0][:, :256], *a[1:])
+            ops.reshape_and_cache_flash_bulk(a[0][:, :256].contiguous(), *a[1:])
     run_both(ops, case)
+
+
+def test_same_addresses_under_another_geometry_are_turned_away(ops):
+    """A set of per-layer tensors that was accepted once says nothing about the next call: the same addresses can come
+    back under another shape (a pool rebuilt after sleep / wake lands where the old one lay).  Layer 1 is a view of
+    a LARGER allocation with twice the blocks at half the block stride, at the address a valid call has just used, so
+    every write would stay inside its allocation whatever the check did; the call must be refused on the host."""
+    L, H, D, bs, NB = 3, 2, 64, 16, 4
+    case = make_bulk_case(T=6, L=L, H=H, D=D, bs=bs, NB=NB, kv_cache_dtype="fp8", seed=22)
+    d = bulk_case_to(case, DEV)
+    big = torch.zeros(4 * 2 * NB * bs * H * D, dtype=torch.uint8, device=DEV)       # twice what a layer needs
+    as_layer = big[: 2 * NB * bs * H * D].view(2, NB, bs, H, D)
+    as_layer.copy_(d["bufs"][1])
+    d["bufs"][1], d["key_caches"][1], d["value_caches"][1] = as_layer, as_layer[0], as_layer[1]
+    case_args = list(bulk_args(d))
+    ops.reshape_and_cache_flash_bulk(*case_args)                                       # the valid call
+    oracle.reshape_and_cache_flash_bulk(*bulk_args(case))
+    torch.cuda.synchronize()
+    assert_bulk_equal(d["bufs"], case["bufs"])
+    before = big.clone()
+    other = big[: 2 * 2 * NB * (bs // 2) * H * D].view(2, 2 * NB, bs // 2, H, D)      # same data_ptr, other geometry
+    assert other[0].data_ptr() == as_layer[0].data_ptr()
+    kc, vc = list(case_args[2]), list(case_args[3])
+    kc[1], vc[1] = other[0], other[1]
+    for _ in range(2):
+        with pytest.raises(RuntimeError, match="must share dtype, block stride, number of blocks"):
+            ops.reshape_and_cache_flash_bulk(case_args[0], case_args[1], kc, vc, *case_args[4:])
+    # a scale of another type at the address of an accepted one
+    ks = list(case_args[6])
+    ks[1] = ks[1].view(torch.int32)
+    with pytest.raises(RuntimeError, match="must be float32"):
+        ops.reshape_and_cache_flash_bulk(*case_args[:6], ks, *case_args[7:])
+    torch.cuda.synchronize()
+    assert torch.equal(big, before)                                                     # nothing was launched
+    ops.reshape_and_cache_flash_bulk(*case_args)                                       # and the valid set still works
+    torch.cuda.synchronize()
+    assert_bulk_equal(d["bufs"], case["bufs"])
+
+
+def test_rows_narrower_than_the_layers_as_in_the_reference_unit_test(ops):
+    """The reference reads row t at t * keys.stride(0) whatever keys.size(1) says, and its own unit test
+    (tests/unit_tests/test_custom_ops.py:63-104) passes keys of shape [L * T, H * D] with 2-D caches [T, H * D]: 4 layers,
+    2 tokens, 2 heads of 16, fp32, "auto".  Accepted here too (the last row read ends inside the tensor's storage)
+    and equal to the oracle's flat formula; a tensor whose storage ends earlier is refused."""
+    L, T, H, D = 4, 2, 2, 16
+    g = torch.Generator().manual_seed(5)
+    keys, values = torch.randn(L * T, H * D, generator=g), torch.randn(L * T, H * D, generator=g)
+    kc = [torch.randn(T, H * D, generator=g) for _ in range(L)]
+    vc = [torch.randn(T, H * D, generator=g) for _ in range(L)]
+    slots = torch.randint(0, T, (T,), generator=g)
+    scales = [torch.tensor(0.1) for _ in range(L)]
+    dkc, dvc = [t.to(DEV) for t in kc], [t.to(DEV) for t in vc]
+    dscales = [t.to(DEV) for t in scales]
+    ops.reshape_and_cache_flash_bulk(keys.to(DEV), values.to(DEV), dkc, dvc, slots.to(DEV), "auto", dscales, dscales, H, D)
+    oracle.reshape_and_cache_flash_bulk(keys, values, kc, vc, slots, "auto", scales, scales, H, D)
+    torch.cuda.synchronize()
+    for got, want in zip(dkc + dvc, kc + vc):
+        assert torch.equal(got.cpu(), want)
+    with pytest.raises(RuntimeError, match="128 columns"):
+        ops.reshape_and_cache_flash_bulk(keys[:4].to(DEV), values.to(DEV), dkc, dvc, slots.to(DEV), "auto", dscales, dscales,
+                                         H, D)

@@ -74,30 +74,36 @@ def test_meta_tensors_trace_shapes_without_data(loaded):
 
 
 def test_argument_checks_mirror_the_reference(loaded):
-    # the shims run the reference's TORCH_CHECKs before touching the device, so the
+    # the host layer runs the reference's TORCH_CHECKs before touching the device, so the
     # ones that precede the device check can be exercised with CPU tensors
+    ln, lstm, bulk = ops._IMPLS["speculator_ln_cuda"], ops._IMPLS["sum_lstm_cuda"], ops._IMPLS["reshape_and_cache_flash_bulk"]
     x32 = torch.randn(4, 64)
+    slots = torch.zeros(4, dtype=torch.int64)
     with pytest.raises(RuntimeError, match="speculator_ln: only fp16 and bf16 are supported."):
-        ops._speculator_ln_impl(x32, None, None, 1e-6)
+        ln(x32, None, None, 1e-6)
     with pytest.raises(RuntimeError, match="speculator_ln: input must be CUDA"):
-        ops._speculator_ln_impl(x32.bfloat16(), None, None, 1e-6)
+        ln(x32.bfloat16(), None, None, 1e-6)
     with pytest.raises(RuntimeError, match="sum_lstm: only fp16 and bf16 are supported."):
-        ops._sum_lstm_impl(x32, x32, x32, None, None, None, None, 1.0, 1e-6, 1e-6, False)
+        lstm(x32, x32, x32, None, None, None, None, 1.0, 1e-6, 1e-6, False)
     with pytest.raises(RuntimeError, match="sum_lstm: inputs must be CUDA tensors"):
-        ops._sum_lstm_impl(x32.half(), x32.half(), x32.half(), None, None, None, None, 1.0, 1e-6, 1e-6, False)
+        lstm(x32.half(), x32.half(), x32.half(), None, None, None, None, 1.0, 1e-6, 1e-6, False)
+    cache = torch.zeros(2, 4, 1, 64)
     with pytest.raises(RuntimeError, match="Unsupported data type of kv cache: nvfp4"):
-        ops._kv_dtype_code(torch.bfloat16, "nvfp4")
+        bulk(x32, x32, [cache], [cache], slots, "nvfp4", [x32], [x32], 1, 64)
     with pytest.raises(RuntimeError, match="Unsupported input type of kv cache"):
-        ops._kv_dtype_code(torch.int8, "auto")
-    assert ops._kv_dtype_code(torch.float16, "fp8") == (_native.DTYPE_F16, _native.KV_FP8_E4M3)
-    assert ops._kv_dtype_code(torch.float32, "fp8_e4m3") == (_native.DTYPE_F32, _native.KV_FP8_E4M3)
-    assert ops._kv_dtype_code(torch.bfloat16, "fp8_e5m2") == (_native.DTYPE_BF16, _native.KV_FP8_E5M2)
-    assert ops._kv_dtype_code(torch.bfloat16, "auto") == (_native.DTYPE_BF16, _native.KV_AUTO)
+        bulk(x32.to(torch.int8), x32.to(torch.int8), [cache], [cache], slots, "auto", [x32], [x32], 1, 64)
+    for accepted in ("auto", "fp8", "fp8_e4m3", "fp8_e5m2"):   # the strings of quant_utils.cuh:532-567 get past the dispatch
+        with pytest.raises(RuntimeError, match="element size|same device"):
+            bulk(x32, x32, [cache.double()], [cache.double()], slots, accepted, [x32], [x32], 1, 64)
     # empty layer list is a no-op (reference :87-89), mismatched list lengths are an error (:91-94)
-    ops._reshape_and_cache_flash_bulk_impl(x32, x32, [], [], torch.zeros(4, dtype=torch.int64), "auto", [], [], 1, 64)
+    bulk(x32, x32, [], [], slots, "auto", [], [], 1, 64)
     with pytest.raises(RuntimeError, match="value_caches"):
-        ops._reshape_and_cache_flash_bulk_impl(x32, x32, [x32], [], torch.zeros(4, dtype=torch.int64), "auto", [x32],
-                                               [x32], 1, 64)
+        bulk(x32, x32, [x32], [], slots, "auto", [x32], [x32], 1, 64)
+    with pytest.raises(RuntimeError, match="not a Tensor"):
+        bulk(x32, x32, [cache], [None], slots, "auto", [x32], [x32], 1, 64)
+    # per-layer geometry is compared with layer 0's on every call, whatever was accepted before
+    with pytest.raises(RuntimeError, match="must share dtype, block stride, number of blocks"):
+        bulk(x32, x32, [cache, cache.view(4, 2, 1, 64)], [cache, cache], slots, "auto", [x32] * 2, [x32] * 2, 1, 32)
 
 
 def test_missing_library_fails_loudly(monkeypatch):
@@ -106,6 +112,7 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_native, "library_path", lambda: None)
     monkeypatch.setattr(_native, "_lib", None)
     monkeypatch.setattr(ops, "_registered", False)
+    monkeypatch.setattr(ops, "_IMPLS", {})
     assert ops.try_load_torch_library() is False
     x = torch.randn(4, 64, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match="not loaded"):

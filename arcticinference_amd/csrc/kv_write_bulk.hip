@@ -552,7 +552,7 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
                       const float *const *k_scale_ptrs, const float *const *v_scale_ptrs,
                       const int64_t *slot_mapping, int64_t num_tokens, int num_layers, int num_heads, int head_size,
                       int block_size, int64_t block_stride, int64_t num_blocks, int src_dtype, int kv_cache_dtype,
-                      const SelectArgs &sel_in, void *stream) {
+                      const SelectArgs &sel_in, void *stream, bool check_only = false) {
   if (num_layers == 0 || num_tokens == 0) return ARCTIC_OK;  // reference :87-89
   if (num_layers < 0 || num_layers > ARCTIC_MAX_LAYERS)
     return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: num_layers=%d outside [0, %d]", fn, num_layers,
@@ -619,9 +619,12 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
   const int epc = 16 / es;  // elements per 16-byte chunk
   // 16-byte loads need aligned rows; stores are 16 B (copy), 8 B (fp8 from 16-bit) or 4 B (fp8 from fp32)
   const int store_bytes = quant ? epc : 16;
+  // (a single source row needs no pitch; with an index list the index workgroups read rows up to num_src_rows)
+  const bool one_source_row =
+      (sel.mode != kSelectNone && sel.indices ? std::max(num_tokens, sel.num_src_rows) : num_tokens) == 1;
   bool vec = (n % epc == 0) && aligned(keys, 16) && aligned(values, 16) &&
-             ((key_stride * es) % 16 == 0 || num_tokens == 1) &&
-             ((value_stride * es) % 16 == 0 || num_tokens == 1) && ((block_stride * des) % store_bytes == 0);
+             ((key_stride * es) % 16 == 0 || one_source_row) &&
+             ((value_stride * es) % 16 == 0 || one_source_row) && ((block_stride * des) % store_bytes == 0);
   for (int l = 0; vec && l < num_layers; ++l)
     vec = aligned(key_cache_ptrs[l], store_bytes) && aligned(value_cache_ptrs[l], store_bytes);
   if (vec && sel.mode != kSelectNone)
@@ -630,90 +633,97 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
           ((sel.out_value_stride * es) % 16 == 0 || sel.num_out_rows <= 1);
 
   hipStream_t s = (hipStream_t)stream;
-  for (int first = 0; first < num_layers; first += kLayersPerLaunch) {
-    const int count = std::min(kLayersPerLaunch, num_layers - first);
-    LayerTables tab;
-    for (int l = 0; l < kLayersPerLaunch; ++l) {
-      const bool in = l < count;
-      tab.key_cache[l] = in ? key_cache_ptrs[first + l] : nullptr;
-      tab.value_cache[l] = in ? value_cache_ptrs[first + l] : nullptr;
-      tab.k_scale[l] = (in && quant) ? k_scale_ptrs[first + l] : nullptr;
-      tab.v_scale[l] = (in && quant) ? v_scale_ptrs[first + l] : nullptr;
-    }
-    BulkParams p;
-    p.keys = (const char *)keys + (int64_t)first * n * es;
-    p.values = (const char *)values + (int64_t)first * n * es;
-    p.slot_mapping = slot_mapping;
-    const bool select = sel.mode != kSelectNone;
-    p.select_mode = sel.mode;
-    p.row_map = sel.mode == kSelectByRowMap ? sel.row_map : nullptr;
-    p.keys_out = select ? (char *)sel.keys_out + (int64_t)first * n * es : nullptr;
-    p.values_out = select ? (char *)sel.values_out + (int64_t)first * n * es : nullptr;
-    p.out_key_stride_bytes = sel.out_key_stride * es;
-    p.out_value_stride_bytes = sel.out_value_stride * es;
-    p.num_out_rows = select ? sel.num_out_rows : 0;
-    p.indices = select ? sel.indices : nullptr;
-    p.index_is_64 = sel.index_bytes == 8;
-    p.num_tokens = num_tokens;
-    p.num_src_rows = sel.num_src_rows;
-    p.key_stride_bytes = key_stride * es;
-    p.value_stride_bytes = value_stride * es;
-    p.block_stride = block_stride;
-    p.num_slots = num_blocks > 0 ? num_blocks * (int64_t)block_size : INT64_MAX;
-    p.num_layers = count;
-    p.n = n;
-    p.block_size = block_size;
-    p.chunks_per_row = vec ? n / epc : 0;
-    p.chunk_shift = -1;
-    if (vec && (p.chunks_per_row & (p.chunks_per_row - 1)) == 0) p.chunk_shift = __builtin_ctz(p.chunks_per_row);
+  // More than kLayersPerLaunch layers take several launches.  Pass 0 plans every launch and checks its grid, so that
+  // a call that is refused has launched nothing; pass 1 launches (a single launch is checked just before it is made).
+  for (int pass = (check_only || num_layers > kLayersPerLaunch) ? 0 : 1; pass < (check_only ? 1 : 2); ++pass) {
+    for (int first = 0; first < num_layers; first += kLayersPerLaunch) {
+      const int count = std::min(kLayersPerLaunch, num_layers - first);
+      LayerTables tab;
+      for (int l = 0; l < kLayersPerLaunch; ++l) {
+        const bool in = l < count;
+        tab.key_cache[l] = in ? key_cache_ptrs[first + l] : nullptr;
+        tab.value_cache[l] = in ? value_cache_ptrs[first + l] : nullptr;
+        tab.k_scale[l] = (in && quant) ? k_scale_ptrs[first + l] : nullptr;
+        tab.v_scale[l] = (in && quant) ? v_scale_ptrs[first + l] : nullptr;
+      }
+      BulkParams p;
+      p.keys = (const char *)keys + (int64_t)first * n * es;
+      p.values = (const char *)values + (int64_t)first * n * es;
+      p.slot_mapping = slot_mapping;
+      const bool select = sel.mode != kSelectNone;
+      p.select_mode = sel.mode;
+      p.row_map = sel.mode == kSelectByRowMap ? sel.row_map : nullptr;
+      p.keys_out = select ? (char *)sel.keys_out + (int64_t)first * n * es : nullptr;
+      p.values_out = select ? (char *)sel.values_out + (int64_t)first * n * es : nullptr;
+      p.out_key_stride_bytes = sel.out_key_stride * es;
+      p.out_value_stride_bytes = sel.out_value_stride * es;
+      p.num_out_rows = select ? sel.num_out_rows : 0;
+      p.indices = select ? sel.indices : nullptr;
+      p.index_is_64 = sel.index_bytes == 8;
+      p.num_tokens = num_tokens;
+      p.num_src_rows = sel.num_src_rows;
+      p.key_stride_bytes = key_stride * es;
+      p.value_stride_bytes = value_stride * es;
+      p.block_stride = block_stride;
+      p.num_slots = num_blocks > 0 ? num_blocks * (int64_t)block_size : INT64_MAX;
+      p.num_layers = count;
+      p.n = n;
+      p.block_size = block_size;
+      p.chunks_per_row = vec ? n / epc : 0;
+      p.chunk_shift = -1;
+      if (vec && (p.chunks_per_row & (p.chunks_per_row - 1)) == 0) p.chunk_shift = __builtin_ctz(p.chunks_per_row);
 
-    // A token's layers are split over `groups` workgroups.  Measured best on gfx950 (sweeps over the group count and
-    // both shapes at 64 to 16384 tokens, 16 and 40 layers):
-    //  - above 8192 tokens, the 512-lane shape with up to five batches of 1024 chunks per workgroup (20 layers of
-    //    8 x 128 bf16) and at least about 1024 workgroups; a workgroup that would get less than two batches takes
-    //    the 256-lane shape instead;
-    //  - below that, the 256-lane shape with about two batches of 1024 chunks per workgroup (8 such layers), more
-    //    and smaller workgroups when fewer than about 2048 would exist otherwise, but never less than one batch each.
-    int groups = 1;
-    bool wide = false;
-    if (vec) {
-      const int64_t chunks_per_layer = 2LL * p.chunks_per_row;
-      const int min_layers = (int)std::max<int64_t>(1, (1024 + chunks_per_layer - 1) / chunks_per_layer);
-      if (num_tokens > 8192) {
-        int64_t g = std::max<int64_t>((1024 + num_tokens - 1) / num_tokens, (chunks_per_layer * count + 5119) / 5120);
-        g = std::max<int64_t>(1, std::min<int64_t>(g, count));
-        const int64_t layers_per_group = (count + g - 1) / g;
-        if (layers_per_group * chunks_per_layer >= 2048) {
-          wide = true;
-          groups = (int)g;
+      // A token's layers are split over `groups` workgroups.  Measured best on gfx950 (sweeps over the group count and
+      // both shapes at 64 to 16384 tokens, 16 and 40 layers):
+      //  - above 8192 tokens, the 512-lane shape with up to five batches of 1024 chunks per workgroup (20 layers of
+      //    8 x 128 bf16) and at least about 1024 workgroups; a workgroup that would get less than two batches takes
+      //    the 256-lane shape instead;
+      //  - below that, the 256-lane shape with about two batches of 1024 chunks per workgroup (8 such layers), more
+      //    and smaller workgroups when fewer than about 2048 would exist otherwise, but never less than one batch each.
+      int groups = 1;
+      bool wide = false;
+      if (vec) {
+        const int64_t chunks_per_layer = 2LL * p.chunks_per_row;
+        const int min_layers = (int)std::max<int64_t>(1, (1024 + chunks_per_layer - 1) / chunks_per_layer);
+        if (num_tokens > 8192) {
+          int64_t g = std::max<int64_t>((1024 + num_tokens - 1) / num_tokens, (chunks_per_layer * count + 5119) / 5120);
+          g = std::max<int64_t>(1, std::min<int64_t>(g, count));
+          const int64_t layers_per_group = (count + g - 1) / g;
+          if (layers_per_group * chunks_per_layer >= 2048) {
+            wide = true;
+            groups = (int)g;
+          } else {
+            const int64_t want = (2048 + num_tokens - 1) / num_tokens;
+            groups = (int)std::max<int64_t>(1, std::min<int64_t>(want, count / min_layers));
+          }
         } else {
-          const int64_t want = (2048 + num_tokens - 1) / num_tokens;
+          const int64_t two_batches = std::max<int64_t>(1, (2048 + chunks_per_layer - 1) / chunks_per_layer);   // layers
+          const int64_t want =
+              std::max<int64_t>((count + two_batches - 1) / two_batches, (2048 + num_tokens - 1) / num_tokens);
           groups = (int)std::max<int64_t>(1, std::min<int64_t>(want, count / min_layers));
         }
       } else {
-        const int64_t two_batches = std::max<int64_t>(1, (2048 + chunks_per_layer - 1) / chunks_per_layer);   // layers
-        const int64_t want = std::max<int64_t>((count + two_batches - 1) / two_batches, (2048 + num_tokens - 1) / num_tokens);
-        groups = (int)std::max<int64_t>(1, std::min<int64_t>(want, count / min_layers));
+        groups = (int)std::max<int64_t>(1, std::min<int64_t>(count, (2048 + num_tokens - 1) / num_tokens));
       }
-    } else {
-      groups = (int)std::max<int64_t>(1, std::min<int64_t>(count, (2048 + num_tokens - 1) / num_tokens));
-    }
-    p.layers_per_group = (count + groups - 1) / groups;
-    p.groups_per_token = (count + p.layers_per_group - 1) / p.layers_per_group;
-    const int lanes = !vec ? kScalarThreads : (wide && p.chunk_shift >= 0) ? 512 : 256;   // of the shape launched below
-    const int64_t index_blocks = p.indices ? (p.num_out_rows + lanes - 1) / lanes : 0;
-    const int64_t grid = num_tokens * p.groups_per_token + index_blocks;
-    p.index_blocks = (unsigned)index_blocks;
-    if (grid > 0x7fffffffLL)
-      return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: too many tokens (%lld)", fn, (long long)num_tokens);
+      p.layers_per_group = (count + groups - 1) / groups;
+      p.groups_per_token = (count + p.layers_per_group - 1) / p.layers_per_group;
+      // lanes of the shape launched below
+      const int lanes = !vec ? kScalarThreads : (wide && p.chunk_shift >= 0) ? 512 : 256;
+      const int64_t index_blocks = p.indices ? (p.num_out_rows + lanes - 1) / lanes : 0;
+      const int64_t grid = num_tokens * p.groups_per_token + index_blocks;
+      p.index_blocks = (unsigned)index_blocks;
+      if (grid > 0x7fffffffLL)
+        return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: too many tokens (%lld)", fn, (long long)num_tokens);
+      if (pass == 0) continue;
 
-    switch (kv_cache_dtype) {
-      case ARCTIC_KV_AUTO: dispatch_src<Copy>(vec, wide, src_dtype, p, tab, grid, s); break;
-      case ARCTIC_KV_FP8_E4M3: dispatch_src<E4M3>(vec, wide, src_dtype, p, tab, grid, s); break;
-      default: dispatch_src<E5M2>(vec, wide, src_dtype, p, tab, grid, s); break;
+      switch (kv_cache_dtype) {
+        case ARCTIC_KV_AUTO: dispatch_src<Copy>(vec, wide, src_dtype, p, tab, grid, s); break;
+        case ARCTIC_KV_FP8_E4M3: dispatch_src<E4M3>(vec, wide, src_dtype, p, tab, grid, s); break;
+        default: dispatch_src<E5M2>(vec, wide, src_dtype, p, tab, grid, s); break;
+      }
+      const int rc = check_launch(fn);
+      if (rc) return rc;
     }
-    const int rc = check_launch(fn);
-    if (rc) return rc;
   }
   return ARCTIC_OK;
 }
@@ -779,24 +789,37 @@ static __device__ __align__(256) int64_t scratch[ARCTIC_SELECT_STATIC_MAX_TOKENS
 
 namespace {
 constexpr int kMaxDevices = 64;
+// Per device: its copy of `scratch` (nullptr until first asked for), and what orders the calls that use it.  The
+// array is shared by every call on the GPU, so a call on another stream than the last one first makes its stream
+// wait for `last_use`, an event recorded behind the last call's kernels: calls on different streams then use the
+// array one after the other instead of racing on it.  Under stream capture nothing of this is recorded.
+struct DeviceScratch {
+  int64_t *ptr = nullptr;
+  hipEvent_t last_use = nullptr;
+  hipStream_t last_stream = nullptr;
+  bool used = false;
+};
 std::mutex g_scratch_mutex;
-int64_t *g_scratch_ptr[kMaxDevices];  // this device's copy of `scratch`, nullptr until first asked for
+DeviceScratch g_scratch[kMaxDevices];
 }  // namespace
 
-static int scratch_on_current_device(const char *fn, int64_t **out) {
+static int scratch_on_current_device(const char *fn, DeviceScratch **out) {
   int dev = -1;
   hipError_t err = hipGetDevice(&dev);
   if (err != hipSuccess) return fail(ARCTIC_ERR_LAUNCH, "%s: hipGetDevice failed: %s", fn, hipGetErrorString(err));
   if (dev < 0 || dev >= kMaxDevices) return fail(ARCTIC_ERR_UNSUPPORTED, "%s: device index %d not supported", fn, dev);
-  std::lock_guard<std::mutex> lock(g_scratch_mutex);
-  if (!g_scratch_ptr[dev]) {
+  DeviceScratch &d = g_scratch[dev];
+  if (!d.ptr) {
     void *ptr = nullptr;
     err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (err != hipSuccess || !ptr)
       return fail(ARCTIC_ERR_LAUNCH, "%s: hipGetSymbolAddress failed on device %d: %s", fn, dev, hipGetErrorString(err));
-    g_scratch_ptr[dev] = (int64_t *)ptr;
+    err = hipEventCreateWithFlags(&d.last_use, hipEventDisableTiming);
+    if (err != hipSuccess)
+      return fail(ARCTIC_ERR_LAUNCH, "%s: hipEventCreateWithFlags failed on device %d: %s", fn, dev, hipGetErrorString(err));
+    d.ptr = (int64_t *)ptr;
   }
-  *out = g_scratch_ptr[dev];
+  *out = &d;
   return ARCTIC_OK;
 }
 
@@ -817,17 +840,44 @@ extern "C" int arctic_reshape_and_cache_flash_bulk_select_static(
   if (num_indices < 0) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: negative number of indices", fn);
   if (num_indices > 0 && !indices) return fail(ARCTIC_ERR_INVALID_ARGUMENT, "%s: null indices", fn);
   // short index lists are scanned by the token workgroups and need no row map; longer ones get theirs in `scratch`
-  int64_t *row_map = nullptr;
-  if (num_layers != 0 && num_tokens > 0 && num_indices > ARCTIC_SELECT_SCAN_MAX_INDICES) {
-    int rc = scratch_on_current_device(fn, &row_map);
-    if (rc) return rc;
-    // every entry below num_tokens is rewritten, so nothing of an earlier call is seen
-    rc = build_row_map(fn, row_map, num_tokens, indices, index_bytes, num_indices, stream);
-    if (rc) return rc;
+  if (num_layers == 0 || num_tokens <= 0 || num_indices <= ARCTIC_SELECT_SCAN_MAX_INDICES) {
+    const SelectArgs sel = {kSelectByScan, nullptr, keys_out, values_out, out_key_stride, out_value_stride, num_indices,
+                            indices, index_bytes, num_src_rows};
+    return bulk_entry(fn, keys, values, key_stride, value_stride, key_cache_ptrs, value_cache_ptrs, k_scale_ptrs,
+                      v_scale_ptrs, slot_mapping, num_tokens, num_layers, num_heads, head_size, block_size,
+                      block_stride, num_blocks, src_dtype, kv_cache_dtype, sel, stream);
   }
-  const SelectArgs sel = {row_map ? kSelectByRowMap : kSelectByScan, row_map, keys_out, values_out, out_key_stride,
-                          out_value_stride, num_indices, indices, index_bytes, num_src_rows};
-  return bulk_entry(fn, keys, values, key_stride, value_stride, key_cache_ptrs, value_cache_ptrs, k_scale_ptrs,
-                    v_scale_ptrs, slot_mapping, num_tokens, num_layers, num_heads, head_size, block_size, block_stride,
-                    num_blocks, src_dtype, kv_cache_dtype, sel, stream);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);   // one call at a time plans its use of the array
+  DeviceScratch *d = nullptr;
+  int rc = scratch_on_current_device(fn, &d);
+  if (rc) return rc;
+  const SelectArgs sel = {kSelectByRowMap, d->ptr, keys_out, values_out, out_key_stride, out_value_stride, num_indices,
+                          indices, index_bytes, num_src_rows};
+  // every argument is checked before the first kernel is enqueued: a call that is refused has launched nothing
+  rc = bulk_entry(fn, keys, values, key_stride, value_stride, key_cache_ptrs, value_cache_ptrs, k_scale_ptrs,
+                  v_scale_ptrs, slot_mapping, num_tokens, num_layers, num_heads, head_size, block_size, block_stride,
+                  num_blocks, src_dtype, kv_cache_dtype, sel, stream, /*check_only=*/true);
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &capture) != hipSuccess) capture = hipStreamCaptureStatusNone;
+  const bool eager = capture == hipStreamCaptureStatusNone;
+  if (eager && d->used && d->last_stream != s) {
+    const hipError_t err = hipStreamWaitEvent(s, d->last_use, 0);
+    if (err != hipSuccess) return fail(ARCTIC_ERR_LAUNCH, "%s: hipStreamWaitEvent failed: %s", fn, hipGetErrorString(err));
+  }
+  // every entry below num_tokens is rewritten, so nothing of an earlier call is seen
+  rc = build_row_map(fn, d->ptr, num_tokens, indices, index_bytes, num_indices, stream);
+  if (rc) return rc;
+  rc = bulk_entry(fn, keys, values, key_stride, value_stride, key_cache_ptrs, value_cache_ptrs, k_scale_ptrs,
+                  v_scale_ptrs, slot_mapping, num_tokens, num_layers, num_heads, head_size, block_size, block_stride,
+                  num_blocks, src_dtype, kv_cache_dtype, sel, stream);
+  if (eager) {
+    const hipError_t err = hipEventRecord(d->last_use, s);
+    if (err != hipSuccess && rc == ARCTIC_OK)
+      rc = fail(ARCTIC_ERR_LAUNCH, "%s: hipEventRecord failed: %s", fn, hipGetErrorString(err));
+    d->last_stream = s;
+    d->used = true;
+  }
+  return rc;
 }

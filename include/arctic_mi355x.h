@@ -173,10 +173,16 @@ int arctic_reshape_and_cache_flash_bulk_select(
  *   indices      device, num_indices entries of index_bytes (4 or 8) each; required when num_indices > 0
  *   other arguments as arctic_reshape_and_cache_flash_bulk_select
  *
- * All calls on one GPU share that GPU's array: calls with long index lists that may run at the same time on one
- * GPU (different streams without an ordering between them) race on it and must use the workspace form instead.
- * The first such call on a device looks the array's address up (hipGetSymbolAddress); make that call outside graph
- * capture.
+ * Every argument is checked before the first kernel is enqueued; a call that is refused has launched nothing.
+ *
+ * All calls on one GPU share that GPU's array.  Calls on one stream use it one after the other.  A call on another
+ * stream than the previous one first makes its stream wait (hipStreamWaitEvent) for an event that the library
+ * recorded behind the previous call's kernels, so calls on streams that nothing else orders take turns at the
+ * array instead of racing on it.  Under stream capture neither the wait nor the event is recorded: replays of graphs
+ * that hold such a call must not overlap on one GPU, with each other or with an eager call; use the workspace form
+ * where they may.
+ * The first call with a long list on a device looks the array's address up (hipGetSymbolAddress) and creates that
+ * event; make that call outside graph capture.
  */
 int arctic_reshape_and_cache_flash_bulk_select_static(
     const void *keys, const void *values, int64_t key_stride, int64_t value_stride,

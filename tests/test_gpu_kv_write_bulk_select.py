@@ -81,6 +81,16 @@ def test_rows_that_force_the_element_wise_kernel(ops, kv):
     run_select(ops, case, idx, 9, out_pad=1)
 
 
+@pytest.mark.parametrize("kv", ["auto", "fp8"])
+def test_one_slot_but_more_source_rows_with_a_pitch_that_is_no_multiple_of_16_bytes(ops, kv):
+    """A single token needs no row pitch, so a lone slot used to qualify for 16-byte accesses whatever the pitch;
+    with an index list the launch also reads source rows beyond the slot mapping, at multiples of that pitch.  Rows
+    of 256 elements (16-byte chunks possible) 259 elements apart, one slot, three source rows, all three selected."""
+    case = make_bulk_case(T=3, L=2, H=2, D=64, bs=16, NB=2, kv_cache_dtype=kv, seed=46, key_pad=3)
+    case["slot_mapping"] = case["slot_mapping"][:1].contiguous()
+    run_select(ops, case, torch.tensor([2, 0, 1, 2]), 6)
+
+
 def test_random_configurations(ops):
     """Seeded sweep over shapes, dtypes, layouts, pitches, padding and selections (none, few, all, shuffled)."""
     import random

@@ -3,6 +3,7 @@ it stands in for (arctic_build_row_map + arctic_reshape_and_cache_flash_bulk_sel
 every cache byte and every selected row bit for bit, on two calls in a row, the second with a smaller input, so that
 whatever the first call left in the library's device array would show.  All calls go through the C ABI."""
 import ctypes
+import functools
 
 import pytest
 import torch
@@ -105,6 +106,119 @@ def test_two_calls_in_a_row_the_second_smaller(ops):
     check_pair(lib, tiny, torch.empty(0, dtype=torch.int64))
 
 
+def static_call(lib, d, idx, k_out, v_out, stream):
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select_static(
+        *common_args(d), idx.data_ptr(), idx.element_size(), idx.numel(), d["keys"].size(0), k_out.data_ptr(),
+        v_out.data_ptr(), k_out.stride(0), v_out.stride(0), stream)
+    assert rc == 0, lib.arctic_last_error()
+
+
+def workspace_result(lib, case, idx):
+    """(cache buffers, k_out, v_out) as the workspace form leaves them, on the host."""
+    d = bulk_case_to(case, DEV)
+    k_out, v_out = out_buffers(idx.numel() + 2, case["keys"].size(1), case["keys"].dtype)
+    stream = torch.cuda.current_stream().cuda_stream
+    row_map = torch.empty(d["slot_mapping"].numel(), dtype=torch.int64, device=DEV)
+    assert lib.arctic_build_row_map(row_map.data_ptr(), row_map.numel(), idx.data_ptr(), idx.element_size(), idx.numel(),
+                                    stream) == 0
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select(
+        *common_args(d), row_map.data_ptr(), idx.data_ptr(), idx.element_size(), idx.numel(), d["keys"].size(0),
+        k_out.data_ptr(), v_out.data_ptr(), k_out.stride(0), v_out.stride(0), stream)
+    assert rc == 0, lib.arctic_last_error()
+    torch.cuda.synchronize()
+    return [b.cpu() for b in d["bufs"]], k_out.cpu(), v_out.cpu()
+
+
+def assert_same(got, want, what):
+    bits = lambda t: t.cpu().contiguous().view(torch.uint8)
+    bufs, k_out, v_out = got
+    for a, b in zip(bufs, want[0]):
+        assert torch.equal(bits(a), bits(b)), f"{what}: cache bytes differ from the workspace form's"
+    assert torch.equal(bits(k_out), bits(want[1])) and torch.equal(bits(v_out), bits(want[2])), f"{what}: selected rows differ"
+
+
+@functools.lru_cache(maxsize=None)
+def two_long_list_cases():
+    """A large and a small case whose index lists need the row map; the host copies are read only."""
+    g = torch.Generator().manual_seed(9)
+    a = make_bulk_case(T=20000, L=8, H=8, D=128, bs=16, NB=1300, kv_cache_dtype="fp8", seed=65, std=1.5, pad_fraction=0.1)
+    idx_a = torch.randperm(20000, generator=g)[:9000].to(DEV)
+    b = make_bulk_case(T=2500, L=2, H=8, D=128, bs=16, NB=160, kv_cache_dtype="fp8", seed=66, std=1.5, pad_fraction=0.1)
+    idx_b = torch.cat([torch.randperm(2500, generator=g)[:2200], torch.tensor([5, 5, 2499])]).to(torch.int32).to(DEV)
+    return (a, idx_a), (b, idx_b)
+
+
+def test_nothing_is_allocated_and_calls_queue_up_without_a_wait_between_them(ops):
+    """What the entry point is for: after a first call on the device (which looks the array's address up), a call
+    leaves the free device memory as it found it (hipMemGetInfo), and two calls issued back to back on one stream,
+    the second smaller, with no synchronisation in between, both give the workspace form's result."""
+    lib = _native.load()
+    (a, idx_a), (b, idx_b) = two_long_list_cases()
+    want_a, want_b = workspace_result(lib, a, idx_a), workspace_result(lib, b, idx_b)
+    da, db = bulk_case_to(a, DEV), bulk_case_to(b, DEV)
+    ka, va = out_buffers(idx_a.numel() + 2, a["keys"].size(1), a["keys"].dtype)
+    kb, vb = out_buffers(idx_b.numel() + 2, b["keys"].size(1), b["keys"].dtype)
+    stream = torch.cuda.current_stream().cuda_stream
+    static_call(lib, da, idx_a, ka, va, stream)      # first calls: the array's address is looked up, both kernel
+    static_call(lib, db, idx_b, kb, vb, stream)      # shapes have run once
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    static_call(lib, da, idx_a, ka, va, stream)
+    static_call(lib, db, idx_b, kb, vb, stream)      # no wait in between: the stream orders the two uses of the array
+    free_after = torch.cuda.mem_get_info()[0]
+    torch.cuda.synchronize()
+    assert free_after == free_before, f"free device memory changed by {free_before - free_after} bytes across two calls"
+    assert_same((da["bufs"], ka, va), want_a, "first call")
+    assert_same((db["bufs"], kb, vb), want_b, "second call")
+
+
+def test_calls_on_two_streams_take_turns_at_the_array(ops):
+    """Two calls with long lists on two streams that nothing orders: the library makes the second stream wait for the
+    first call's use of the array (an event behind its kernels), so both give the workspace form's result.  The first
+    call is large (its kernel runs for tens of microseconds), the second small and issued right behind it."""
+    lib = _native.load()
+    (a, idx_a), (b, idx_b) = two_long_list_cases()
+    want_a, want_b = workspace_result(lib, a, idx_a), workspace_result(lib, b, idx_b)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    for round_ in range(3):
+        da, db = bulk_case_to(a, DEV), bulk_case_to(b, DEV)
+        ka, va = out_buffers(idx_a.numel() + 2, a["keys"].size(1), a["keys"].dtype)
+        kb, vb = out_buffers(idx_b.numel() + 2, b["keys"].size(1), b["keys"].dtype)
+        torch.cuda.synchronize()
+        static_call(lib, da, idx_a, ka, va, s1.cuda_stream)
+        static_call(lib, db, idx_b, kb, vb, s2.cuda_stream)
+        static_call(lib, da, idx_a, ka, va, s1.cuda_stream)     # back on the first stream: waits for the second's use
+        torch.cuda.synchronize()
+        assert_same((da["bufs"], ka, va), want_a, f"round {round_}, first stream")
+        assert_same((db["bufs"], kb, vb), want_b, f"round {round_}, second stream")
+
+
+def test_recorded_into_a_hip_graph(ops):
+    """A call with a long list recorded into a HIP graph (after a first call outside capture) and replayed three
+    times, with eager work and synchronisations between the replays; every replay gives the eager result."""
+    lib = _native.load()
+    (_, _), (b, idx_b) = two_long_list_cases()
+    want = workspace_result(lib, b, idx_b)
+    d = bulk_case_to(b, DEV)
+    fresh = [buf.clone() for buf in d["bufs"]]
+    k_out, v_out = out_buffers(idx_b.numel() + 2, b["keys"].size(1), b["keys"].dtype)
+    static_call(lib, d, idx_b, k_out, v_out, torch.cuda.current_stream().cuda_stream)   # outside capture
+    torch.cuda.synchronize()
+    assert_same((d["bufs"], k_out, v_out), want, "eager call")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_call(lib, d, idx_b, k_out, v_out, torch.cuda.current_stream().cuda_stream)
+    for replay in range(3):
+        for buf, init in zip(d["bufs"], fresh):
+            buf.copy_(init)
+        k_out.view(torch.uint8).fill_(0xA5)
+        v_out.view(torch.uint8).fill_(0xA5)
+        (torch.ones(1000, device=DEV) * 2).sum().item()      # the program's own eager work and a synchronisation
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_same((d["bufs"], k_out, v_out), want, f"replay {replay}")
+
+
 def test_size_limit_and_argument_errors(ops):
     lib = _native.load()
     case = make_bulk_case(T=8, L=2, H=2, D=64, bs=16, NB=2, kv_cache_dtype="fp8", seed=63)
@@ -121,5 +235,16 @@ def test_size_limit_and_argument_errors(ops):
     assert rc == 1 and b"null indices" in lib.arctic_last_error()
     rc = lib.arctic_reshape_and_cache_flash_bulk_select_static(*args, idx.data_ptr(), 2, 4, 8, *tail[4:])
     assert rc == 2 and b"int32 or int64" in lib.arctic_last_error()
+    # a list long enough to need the array, refused for its other arguments: nothing may have been enqueued by then
+    long_idx = torch.arange(3000, device=DEV) % 8
+    long_tail = (long_idx.data_ptr(), 8, 3000, 8, out.data_ptr(), out.data_ptr(), 256, 256, None)
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select_static(*args, *long_tail[:4], None, *long_tail[5:])
+    assert rc == 1 and b"null keys_out" in lib.arctic_last_error()
+    bad_type = list(args)
+    bad_type[16] = 7
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select_static(*bad_type, *long_tail)
+    assert rc == 2 and b"Unsupported input type" in lib.arctic_last_error()
+    rc = lib.arctic_reshape_and_cache_flash_bulk_select_static(*args, long_idx.data_ptr(), 8, 1 << 31, 8, *long_tail[4:])
+    assert rc == 1 and b"2^31 output rows" in lib.arctic_last_error()
     torch.cuda.synchronize()
     assert not out.any()

@@ -158,15 +158,21 @@ def event_times_us(fn, iters):
 
 def read_traffic(path):
     """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by
-    a copy kernel of known size); the figure is kept next to the profile it came from."""
+    a copy kernel of known size); the figure is kept next to the profile it came from, with the day it was
+    measured and the commit of the library it was measured on.  Returns (bytes or None, {key: text})."""
+    fields = {}
     try:
         with open(path) as f:
             for line in f:
-                if line.strip().startswith("hbm_bytes_per_launch"):
-                    return int(float(line.split("=")[1].split()[0]))
+                if "=" in line and not line.lstrip().startswith("#"):
+                    key, value = line.split("=", 1)
+                    fields[key.strip()] = value.strip()
     except OSError:
-        pass
-    return None
+        return None, fields
+    try:
+        return int(float(fields["hbm_bytes_per_launch"].split()[0])), fields
+    except (KeyError, ValueError):
+        return None, fields
 
 
 def cpu_baseline_bulk(w: BulkWorkload, target_seconds=10.0):
@@ -213,6 +219,57 @@ def cpu_baseline_bulk(w: BulkWorkload, target_seconds=10.0):
         "note": "the reference has no CPU implementation of the bulk write (its fallback, llama_swiftkv.py:623-650, is "
                 "vLLM's CUDA operator), so a port of its kernel is the only CPU form there is; the speculator operators, "
                 "which do have a PyTorch fallback in the reference, are timed both ways in extras.speculator.cpu_baseline",
+    }
+
+
+def cpu_baseline_bulk_pytorch(w: BulkWorkload, layers=4, target_seconds=3.0):
+    """The bulk write as PyTorch CPU operations on a sample: per layer
+    cache_l.view(-1, n).index_copy_(0, slots[valid], cvt(keys[valid, l*n:(l+1)*n])) and the same for the values,
+    cvt = (x.float() / scale).clamp(-448, 448).to(float8_e4m3fn).  The reference has no CPU form of this operator;
+    this is how one would write it with library routines (it is the closed form the oracle is pinned against)."""
+    n, L = w.n, min(layers, w.L)
+    threads = torch.get_num_threads()
+
+    def prepare(sample_tokens):
+        g = torch.Generator().manual_seed(98)
+        sample = torch.randperm(w.T, generator=g)[:sample_tokens]
+        sub = w.slots_cpu[sample]
+        valid = sub >= 0
+        nvalid = int(valid.sum())
+        dst = torch.randperm(nvalid, generator=g)
+        keys = w.keys[:, : L * n][sample.to(w.keys.device)].cpu().contiguous()
+        values = w.values[:, : L * n][sample.to(w.keys.device)].cpu().contiguous()
+        nb = (nvalid + w.bs - 1) // w.bs
+        caches = [torch.zeros(2, nb * w.bs, n, dtype=torch.uint8) for _ in range(L)]
+        ks = [float(s) for s in w.k_scales[:L]]
+        vs = [float(s) for s in w.v_scales[:L]]
+
+        def cvt(x, scale):
+            return (x.float() / scale).clamp_(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
+
+        def run():
+            t0 = time.perf_counter()
+            for l in range(L):
+                caches[l][0].index_copy_(0, dst, cvt(keys[valid, l * n:(l + 1) * n], ks[l]))
+                caches[l][1].index_copy_(0, dst, cvt(values[valid, l * n:(l + 1) * n], vs[l]))
+            return time.perf_counter() - t0
+
+        return run, nvalid * L * w.bytes_per_unit
+
+    run, nbytes = prepare(min(w.T, 256))
+    run()
+    rate = nbytes / run()
+    tokens = int(min(w.T, max(256, 0.5 * rate / (L * w.bytes_per_unit))))     # about half a second per pass
+    run, nbytes = prepare(tokens)
+    total_dt, passes = 0.0, 0
+    while total_dt < target_seconds and passes < 50:
+        total_dt, passes = total_dt + run(), passes + 1
+    return {
+        "value": round(passes * nbytes / total_dt / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "pytorch",
+        "sample": f"{passes} passes over {tokens} of {w.T} tokens x {L} of {w.L} layers of the same workload "
+                  f"({passes * nbytes / 1e6:.0f} MB algorithmic) in {total_dt:.2f} s; per-layer fancy-index read, "
+                  f"float division, clamp, float8_e4m3fn cast and index_copy_ with torch's intra-op threads",
+        "cpu_model": cpu_model(),
     }
 
 
@@ -568,14 +625,20 @@ def host_overhead_route(route, calls=3000):
     """Host wall time per eager call with the GPU out of the picture: tiny inputs (4 tokens, 8 rows), so that a
     kernel is over long before the host has issued the next one; `calls` calls are issued back to back and the
     wall clock is divided by their number (one synchronisation in front, one behind, outside the clock).
-    route "ctypes": this package's py_custom_ops (Python shims over the C ABI).  route "torch_ext": the same
-    library behind a compiled torch extension, C++ from the dispatcher down (the file named by
-    ARCTIC_TORCH_EXT).  Runs in a process of its own: both routes define the arctic_inference namespace."""
+    route "py_custom_ops": this package's module functions (the C++ host layer called directly).  route
+    "torch_ops": the same host layer through torch.ops.arctic_inference.* as this package registers it (what
+    torch.compile and callers of the registered operators take).  route "torch_ext": the same library behind the
+    reference's own torch_bindings.cpp compiled with this package's forwards (the file named by ARCTIC_TORCH_EXT).
+    Runs in a process of its own: the last route defines the arctic_inference namespace a second time."""
     dev = torch.device("cuda:0")
-    if route == "ctypes":
+    if route in ("py_custom_ops", "torch_ops"):
         from arcticinference_amd import py_custom_ops as ops
         assert ops.try_load_torch_library()
-        bulk, lstm, ln = ops.reshape_and_cache_flash_bulk, ops.sum_lstm, ops.speculator_ln
+        if route == "py_custom_ops":
+            bulk, lstm, ln = ops.reshape_and_cache_flash_bulk, ops.sum_lstm, ops.speculator_ln
+        else:
+            ns = torch.ops.arctic_inference
+            bulk, lstm, ln = ns.reshape_and_cache_flash_bulk, ns.sum_lstm_cuda, ns.speculator_ln_cuda
     else:
         torch.ops.load_library(os.environ["ARCTIC_TORCH_EXT"])
         ns = torch.ops.arctic_inference
@@ -635,9 +698,9 @@ def host_overhead_route(route, calls=3000):
 def bench_host_overhead():
     """Host microseconds per eager call through both integration routes, each measured in a child process."""
     ext = os.path.join(ROOT, "oracle", "_ref", "arctic_torch_ext.so")
-    routes = {"route_1_py_custom_ops_ctypes": ("ctypes", {})}
+    routes = {"route_1_py_custom_ops": ("py_custom_ops", {}), "route_1_through_torch_ops": ("torch_ops", {})}
     if os.path.exists(ext):
-        routes["route_2_torch_extension_cpp"] = ("torch_ext", {"ARCTIC_TORCH_EXT": ext})
+        routes["route_2_reference_torch_bindings"] = ("torch_ext", {"ARCTIC_TORCH_EXT": ext})
     out = {"what": "host wall time per eager call in microseconds, tiny inputs (4 tokens / 8 rows), 3000 calls issued "
                    "back to back, best of 3 rounds; the GPU work of a call is shorter than the host's"}
     for name, (route, env) in routes.items():
@@ -647,8 +710,8 @@ def bench_host_overhead():
             out[name] = "failed: " + (proc.stderr.strip().splitlines() or ["no output"])[-1]
             continue
         out[name] = json.loads(proc.stdout.strip().splitlines()[-1])
-    if "route_2_torch_extension_cpp" not in routes:
-        out["route_2_torch_extension_cpp"] = "oracle/_ref/arctic_torch_ext.so is not built (make -C oracle torch_ext)"
+    if "route_2_reference_torch_bindings" not in routes:
+        out["route_2_reference_torch_bindings"] = "oracle/_ref/arctic_torch_ext.so is not built (make -C oracle torch_ext)"
     return out
 
 
@@ -1275,14 +1338,15 @@ def main():
     ap.add_argument("--weight-gib", type=int, default=66, help="resident-weights placeholder allocated before the KV pool")
     ap.add_argument("--pool-blocks", type=int, default=65536, help="blocks per layer of the 80-layer KV pool")
     ap.add_argument("--no-extras", action="store_true", help="skip the speculator / decode-mix measurements")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-cpu", action="store_true",
+                    help="skip the CPU baselines and the host time per call (which runs child processes)")
     ap.add_argument("--placement-sweep", action="store_true",
                     help="instead of the benchmark, time the 70B-shape launch with the caches in each 8 GiB chunk "
                          "of the GPU's memory and spread over its regions; prints one JSON object")
     ap.add_argument("--only", choices=sorted(ONLY), default=None,
                     help="instead of the benchmark, run one of the extra measurements alone (for profiling it); "
                          "prints one JSON object")
-    ap.add_argument("--host-overhead-route", choices=["ctypes", "torch_ext"], default=None, help=argparse.SUPPRESS)
+    ap.add_argument("--host-overhead-route", choices=["py_custom_ops", "torch_ops", "torch_ext"], default=None, help=argparse.SUPPRESS)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) so that a counter run of this "
                          "command can scale FETCH_SIZE / WRITE_SIZE")
@@ -1393,11 +1457,14 @@ def main():
         torch.cuda.empty_cache()
     if args.calibrate_copy:
         calibration_copy(dev)
-    traffic = read_traffic(os.path.join(ROOT, "profiles", "kv_write_bulk_fp8_70b.traffic.txt"))
+    traffic, traffic_fields = read_traffic(os.path.join(ROOT, "profiles", "kv_write_bulk_fp8_70b.traffic.txt"))
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                "traffic_source": "not measured in this run: carried over from profiles/kv_write_bulk_fp8_70b.traffic.txt "
-                                  "(two rocprofv3 --pmc runs of this command, FETCH_SIZE and WRITE_SIZE scaled by a 1 GiB copy)",
+                "traffic_source": "not measured in this run (a process cannot read the HBM counters of its own kernels): "
+                                  "carried over from profiles/kv_write_bulk_fp8_70b.traffic.txt, two rocprofv3 --pmc runs "
+                                  "of this command, FETCH_SIZE and WRITE_SIZE scaled by a 1 GiB copy, measured on "
+                                  f"{traffic_fields.get('measured_on', 'an unrecorded day')} with the library at commit "
+                                  f"{traffic_fields.get('library_commit', 'unrecorded')}",
                 "placement": "serving memory map (config.memory_map): the written caches span two of the HBM's three "
                              "address regions",
                 "achieved_compact": compact["GBps"], "frac_compact": compact["hbm_frac"],
@@ -1413,10 +1480,12 @@ def main():
                 "algorithmic_bytes": w.bytes}
     log(f"bulk fp8 70B shape: {ms_per_step:.3f} ms/step wall, kernel {kernel_us:.1f} us, {achieved:.0f} GB/s")
 
-    cpu = None
+    cpu = cpu_pytorch = None
     if not args.no_cpu:
         cpu = cpu_baseline_bulk(w)
         log(f"cpu baseline: {cpu}")
+        cpu_pytorch = cpu_baseline_bulk_pytorch(w)
+        log(f"cpu baseline, PyTorch formulation: {cpu_pytorch}")
 
     workload_text = (f"bulk KV write at the 70B SwiftKV shape: {w.T} tokens x {w.L} layers x {w.H} KV heads x {w.D}, "
                      f"block {w.bs}, fp8-e4m3 cache, amax/448 scales, 10% slots = -1, the rest distinct random "
@@ -1465,7 +1534,8 @@ def main():
         extras["bulk_write_and_select_decode_70b"] = bench_bulk_select(ops, dev, args.steps)
         torch.cuda.empty_cache()
         extras["suffix_decoding_cpu"] = bench_suffix_decoding()
-        extras["host_us_per_call"] = bench_host_overhead()
+        if not args.no_cpu:   # child processes: left out with the other host-side measurements
+            extras["host_us_per_call"] = bench_host_overhead()
         log(f"extras: {extras}")
 
     result = {
@@ -1475,7 +1545,7 @@ def main():
         "vs_baseline": None, "dtype": "fp8_e4m3",
         "data": "synthetic",
         "config": cfg,
-        "roofline": roofline, "cpu_baseline": cpu, "extras": extras,
+        "roofline": roofline, "cpu_baseline": cpu, "cpu_baseline_pytorch": cpu_pytorch, "extras": extras,
     }
     print(json.dumps(result), flush=True)
 

@@ -8,6 +8,7 @@
 
 #include <string>
 #include <tuple>
+#include <vector>
 
 #include "torch_host.hpp"
 
@@ -71,6 +72,51 @@ void reshape_and_cache_flash_bulk_select(const at::Tensor &keys, const at::Tenso
   bulk(keys, values, key_caches, value_caches, slot_mapping, kv_cache_dtype, k_scales, v_scales, num_heads, head_size,
        &select);
 }
+
+// The per-layer tensors of a bulk write, checked once and held, for a caller that writes the same layers on every
+// step (SwiftKV's caller rebuilds its four lists of views on every engine step, llama_swiftkv.py:594-615, which costs
+// it more host time than the write).  The object keeps an alias of every tensor, so the addresses in its tables stay
+// allocated and the geometry it checked cannot change under it; it must be rebuilt when the pool is (the caller
+// knows: its kv_cache objects are new ones then).
+class PreparedLayers {
+ public:
+  PreparedLayers(const py::handle &key_caches, const py::handle &value_caches, const py::handle &k_scales,
+                 const py::handle &v_scales) {
+    const TensorSequence kc(key_caches, "key_caches must be a list of Tensors"),
+        vc(value_caches, "value_caches must be a list of Tensors"), ks(k_scales, "k_scales must be a list of Tensors"),
+        vs(v_scales, "v_scales must be a list of Tensors");
+    const TensorSequence *lists[4] = {&kc, &vc, &ks, &vs};
+    for (const TensorSequence *list : lists)
+      for (int64_t i = 0; i < list->size(); ++i) held_.push_back((*list)[i].alias());
+    // the tables are made from the held aliases, not from the caller's objects
+    offsets_[0] = 0;
+    for (int k = 0; k < 4; ++k) offsets_[k + 1] = offsets_[k] + lists[k]->size();
+    const arctic_host::LayerLists layers = {
+        {kc.size(), vc.size(), ks.size(), vs.size()},
+        [](const void *ctx, int list, int64_t l) -> const at::Tensor & {
+          const PreparedLayers *self = (const PreparedLayers *)ctx;
+          return self->held_[(size_t)(self->offsets_[list] + l)];
+        },
+        this};
+    checked_ = arctic_host::check_layers(layers);
+  }
+  int64_t num_layers() const { return checked_.num_layers; }
+  void write(const at::Tensor &keys, const at::Tensor &values, const at::Tensor &slot_mapping,
+             const std::string &kv_cache_dtype, int64_t num_heads, int64_t head_size) const {
+    arctic_host::bulk_write(keys, values, checked_, slot_mapping, kv_cache_dtype, num_heads, head_size, nullptr);
+  }
+  void write_select(const at::Tensor &keys, const at::Tensor &values, const at::Tensor &slot_mapping,
+                    const std::string &kv_cache_dtype, int64_t num_heads, int64_t head_size,
+                    const at::Tensor &logits_indices, const at::Tensor &k_out, const at::Tensor &v_out) const {
+    const arctic_host::SelectRows select = {logits_indices, k_out, v_out};
+    arctic_host::bulk_write(keys, values, checked_, slot_mapping, kv_cache_dtype, num_heads, head_size, &select);
+  }
+
+ private:
+  std::vector<at::Tensor> held_;
+  int64_t offsets_[5];
+  arctic_host::CheckedLayers checked_;
+};
 
 void reshape_and_cache_flash_fp4(const at::Tensor &key, const at::Tensor &value, const at::Tensor &key_cache,
                                  const at::Tensor &value_cache, const at::Tensor &slot_mapping,
@@ -163,4 +209,10 @@ PYBIND11_MODULE(_host_ext, m) {
   m.def("gather_rows", &gather_rows);
   m.def("scatter_rows", &scatter_rows);
   m.def("speculator_argmax_cuda", &speculator_argmax_cuda);
+  py::class_<PreparedLayers>(m, "BulkKVLayers")
+      .def(py::init<const py::handle &, const py::handle &, const py::handle &, const py::handle &>(),
+           py::arg("key_caches"), py::arg("value_caches"), py::arg("k_scales"), py::arg("v_scales"))
+      .def_property_readonly("num_layers", &PreparedLayers::num_layers)
+      .def("write", &PreparedLayers::write)
+      .def("write_select", &PreparedLayers::write_select);
 }

@@ -57,12 +57,65 @@ bool rows_dense(const at::Tensor &t) {
 
 void check_rc(int rc) { TORCH_CHECK(rc == 0, arctic_last_error()); }
 
+// A size on its way into an `int` parameter of the C ABI: out of range is an error here, not a wrapped value there.
+int to_int(int64_t v, const char *what) {
+  TORCH_CHECK(v >= 0 && v <= 0x7fffffffLL, what, " = ", v, " is outside [0, 2^31)");
+  return (int)v;
+}
+
 }  // namespace
 
-void bulk_write(const at::Tensor &keys, const at::Tensor &values, const LayerLists &layers,
+CheckedLayers check_layers(const LayerLists &layers) {
+  CheckedLayers c;
+  const int64_t num_layers = layers.count[0];
+  c.num_layers = num_layers;
+  if (num_layers == 0) return c;
+  TORCH_CHECK(num_layers == layers.count[1], "Expected num_layers == value_caches.size() to be true");
+  TORCH_CHECK(num_layers == layers.count[2], "Expected num_layers == k_scales.size() to be true");
+  TORCH_CHECK(num_layers == layers.count[3], "Expected num_layers == v_scales.size() to be true");
+  const at::Tensor &first = layers(0, 0), &first_v = layers(1, 0);
+  c.block_size = first.size(1);
+  c.block_stride = first.stride(0);
+  TORCH_CHECK(c.block_stride == first_v.stride(0), "Expected block_stride == value_caches[0].stride(0) to be true");
+  // From here on: not checked by the reference (it reinterprets the pointers); a mismatch there corrupts memory,
+  // here it is an error.  Every layer's K and V view must look like layer 0's: the kernel takes one block stride,
+  // block size and number of blocks for all of them.
+  c.num_blocks = first.size(0);
+  c.cache_element_size = first.element_size();
+  c.device = first.device();
+  const auto dtype0 = first.scalar_type();
+  c.key_caches.resize(num_layers);
+  c.value_caches.resize(num_layers);
+  c.k_scales.assign(num_layers, nullptr);
+  c.v_scales.assign(num_layers, nullptr);
+  for (int64_t l = 0; l < num_layers; ++l) {
+    const at::Tensor &k = layers(0, l), &v = layers(1, l);
+    TORCH_CHECK(k.scalar_type() == dtype0 && v.scalar_type() == dtype0 && k.stride(0) == c.block_stride &&
+                    v.stride(0) == c.block_stride && k.size(0) == c.num_blocks && v.size(0) == c.num_blocks &&
+                    k.size(1) == c.block_size && v.size(1) == c.block_size && k.device() == c.device &&
+                    v.device() == c.device,
+                "reshape_and_cache_flash_bulk: key and value caches of all layers must share dtype, block stride, "
+                "number of blocks, block size and device");
+    c.key_caches[l] = k.data_ptr();
+    c.value_caches[l] = v.data_ptr();
+  }
+  // the scales matter to an fp8 write only, so what is wrong with them is kept until one is asked for
+  for (int64_t l = 0; l < num_layers && !c.scales_problem; ++l) {
+    const at::Tensor &k = layers(2, l), &v = layers(3, l);
+    if (k.scalar_type() != at::kFloat || v.scalar_type() != at::kFloat)
+      c.scales_problem = "reshape_and_cache_flash_bulk: k_scales / v_scales must be float32";
+    else if (k.device() != c.device || v.device() != c.device)
+      c.scales_problem = "reshape_and_cache_flash_bulk: all tensors must be on the same device";
+    c.k_scales[l] = (const float *)k.data_ptr();
+    c.v_scales[l] = (const float *)v.data_ptr();
+  }
+  return c;
+}
+
+void bulk_write(const at::Tensor &keys, const at::Tensor &values, const CheckedLayers &layers,
                 const at::Tensor &slot_mapping, const std::string &kv_cache_dtype, int64_t num_heads,
                 int64_t head_size, const SelectRows *select) {
-  const int64_t num_layers = layers.count[0];
+  const int64_t num_layers = layers.num_layers;
   int64_t n_sel = 0;
   if (select) {
     const char *fn = "reshape_and_cache_flash_bulk_select";
@@ -97,17 +150,16 @@ void bulk_write(const at::Tensor &keys, const at::Tensor &values, const LayerLis
       if (n_sel) {
         const at::Tensor src[2] = {keys.narrow(1, 0, width), values.narrow(1, 0, width)};
         const at::Tensor *dst[2] = {&select->k_out, &select->v_out};
-        const TensorList sources = {2, [](const void *c, int64_t i) -> const at::Tensor & { return ((const at::Tensor *)c)[i]; }, src};
-        const TensorList outs = {2, [](const void *c, int64_t i) -> const at::Tensor & { return *((const at::Tensor *const *)c)[i]; }, dst};
+        const TensorList sources = {
+            2, [](const void *c, int64_t i) -> const at::Tensor & { return ((const at::Tensor *)c)[i]; }, src};
+        const TensorList outs = {
+            2, [](const void *c, int64_t i) -> const at::Tensor & { return *((const at::Tensor *const *)c)[i]; }, dst};
         move_rows("gather_rows", sources, idx, outs, false);
       }
       return;
     }
   }
 
-  TORCH_CHECK(num_layers == layers.count[1], "Expected num_layers == value_caches.size() to be true");
-  TORCH_CHECK(num_layers == layers.count[2], "Expected num_layers == k_scales.size() to be true");
-  TORCH_CHECK(num_layers == layers.count[3], "Expected num_layers == v_scales.size() to be true");
   // DISPATCH_BY_KV_CACHE_DTYPE, csrc/custom_ops/quant_utils.cuh:532-567
   int kv = -1;
   if (kv_cache_dtype == "auto") kv = ARCTIC_KV_AUTO;
@@ -122,24 +174,17 @@ void bulk_write(const at::Tensor &keys, const at::Tensor &values, const LayerLis
     default: break;
   }
   TORCH_CHECK(src >= 0, "Unsupported input type of kv cache: ", keys.scalar_type());
-  const at::Tensor &first = layers(0, 0), &first_v = layers(1, 0);
-  const int64_t block_size = first.size(1);
-  const int64_t block_stride = first.stride(0);
-  TORCH_CHECK(block_stride == first_v.stride(0), "Expected block_stride == value_caches[0].stride(0) to be true");
   TORCH_CHECK(slot_mapping.scalar_type() == at::kLong, "expected scalar type Long but found ", slot_mapping.scalar_type());
-  // From here on: not checked by the reference (it reinterprets the pointers); a mismatch there corrupts memory,
-  // here it is an error.
+  // not checked by the reference either
   TORCH_CHECK(values.scalar_type() == keys.scalar_type(), "reshape_and_cache_flash_bulk: keys and values dtype differ");
   TORCH_CHECK(keys.stride(-1) == 1 && values.stride(-1) == 1,
               "reshape_and_cache_flash_bulk: last dimension of keys/values must be contiguous");
   TORCH_CHECK(slot_mapping.dim() == 1 && (num_tokens <= 1 || slot_mapping.stride(0) == 1),
               "reshape_and_cache_flash_bulk: slot_mapping must be 1-D and contiguous");
   const int64_t want_elem = kv == ARCTIC_KV_AUTO ? keys.element_size() : 1;
-  TORCH_CHECK(first.element_size() == want_elem && first_v.element_size() == want_elem,
-              "reshape_and_cache_flash_bulk: cache element size ", first.element_size(), " does not match kv_cache_dtype '",
-              kv_cache_dtype, "' (expected ", want_elem, ")");
-  TORCH_CHECK(first.device() == keys.device() && values.device() == keys.device() &&
-                  slot_mapping.device() == keys.device(),
+  TORCH_CHECK(layers.cache_element_size == want_elem, "reshape_and_cache_flash_bulk: cache element size ",
+              layers.cache_element_size, " does not match kv_cache_dtype '", kv_cache_dtype, "' (expected ", want_elem, ")");
+  TORCH_CHECK(layers.device == keys.device() && values.device() == keys.device() && slot_mapping.device() == keys.device(),
               "reshape_and_cache_flash_bulk: all tensors must be on the same device");
   // Row t is read at t * stride(0), `width` elements long.  The reference looks at stride(0) only, and its own unit
   // test (tests/unit_tests/test_custom_ops.py:79-80) passes keys of shape [L * T, H * D]; rows narrower than `width`
@@ -152,43 +197,18 @@ void bulk_write(const at::Tensor &keys, const at::Tensor &values, const LayerLis
   };
   TORCH_CHECK(covers(keys) && covers(values), "reshape_and_cache_flash_bulk: keys and values must be 2-D with at least ",
               num_tokens, " rows (one per slot) and ", width, " columns (layers x heads x head_size)");
-  // Every layer's K and V view must look like layer 0's: the kernel takes one block stride, block size and number
-  // of blocks for all of them.  Looked at on every call: an address does not identify a tensor's shape.
-  const bool quant = kv != ARCTIC_KV_AUTO;
-  std::vector<const void *> kc(num_layers), vc(num_layers);
-  std::vector<const float *> ks(num_layers, nullptr), vs(num_layers, nullptr);
-  const auto dtype0 = first.scalar_type();
-  const int64_t num_blocks = first.size(0);
-  const auto device0 = first.device();
-  for (int64_t l = 0; l < num_layers; ++l) {
-    const at::Tensor &k = layers(0, l), &v = layers(1, l);
-    TORCH_CHECK(k.scalar_type() == dtype0 && v.scalar_type() == dtype0 && k.stride(0) == block_stride &&
-                    v.stride(0) == block_stride && k.size(0) == num_blocks && v.size(0) == num_blocks &&
-                    k.size(1) == block_size && v.size(1) == block_size && k.device() == device0 && v.device() == device0,
-                "reshape_and_cache_flash_bulk: key and value caches of all layers must share dtype, block stride, "
-                "number of blocks, block size and device");
-    kc[l] = k.data_ptr();
-    vc[l] = v.data_ptr();
-  }
-  if (quant) {
-    for (int64_t l = 0; l < num_layers; ++l) {
-      const at::Tensor &k = layers(2, l), &v = layers(3, l);
-      TORCH_CHECK(k.scalar_type() == at::kFloat && v.scalar_type() == at::kFloat,
-                  "reshape_and_cache_flash_bulk: k_scales / v_scales must be float32");
-      TORCH_CHECK(k.device() == device0 && v.device() == device0,
-                  "reshape_and_cache_flash_bulk: all tensors must be on the same device");
-      ks[l] = (const float *)k.data_ptr();
-      vs[l] = (const float *)v.data_ptr();
-    }
-  }
+  if (kv != ARCTIC_KV_AUTO) TORCH_CHECK(!layers.scales_problem, layers.scales_problem);
 
+  const int layer_count = to_int(num_layers, "num_layers"), heads = to_int(num_heads, "num_heads");
+  const int head = to_int(head_size, "head_size"), block = to_int(layers.block_size, "block_size");
   const DeviceGuard guard(keys.device());
   void *stream = current_stream();
   if (!select) {
     check_rc(arctic_reshape_and_cache_flash_bulk(
-        keys.data_ptr(), values.data_ptr(), keys.stride(0), values.stride(0), kc.data(), vc.data(), ks.data(), vs.data(),
-        (const int64_t *)slot_mapping.data_ptr(), num_tokens, (int)num_layers, (int)num_heads, (int)head_size,
-        (int)block_size, block_stride, num_blocks, src, kv, stream));
+        keys.data_ptr(), values.data_ptr(), keys.stride(0), values.stride(0), layers.key_caches.data(),
+        layers.value_caches.data(), layers.k_scales.data(), layers.v_scales.data(),
+        (const int64_t *)slot_mapping.data_ptr(), num_tokens, layer_count, heads, head, block, layers.block_stride,
+        layers.num_blocks, src, kv, stream));
     return;
   }
   // A long list: the inverse of logits_indices (which output row, if any, a token goes to) is built first; up to
@@ -200,11 +220,19 @@ void bulk_write(const at::Tensor &keys, const at::Tensor &values, const LayerLis
                                   stream));
   }
   check_rc(arctic_reshape_and_cache_flash_bulk_select(
-      keys.data_ptr(), values.data_ptr(), keys.stride(0), values.stride(0), kc.data(), vc.data(), ks.data(), vs.data(),
-      (const int64_t *)slot_mapping.data_ptr(), num_tokens, (int)num_layers, (int)num_heads, (int)head_size,
-      (int)block_size, block_stride, num_blocks, src, kv, row_map.defined() ? (const int64_t *)row_map.data_ptr() : nullptr,
-      idx.data_ptr(), (int)idx.element_size(), n_sel, keys.size(0), select->k_out.data_ptr(), select->v_out.data_ptr(),
+      keys.data_ptr(), values.data_ptr(), keys.stride(0), values.stride(0), layers.key_caches.data(),
+      layers.value_caches.data(), layers.k_scales.data(), layers.v_scales.data(),
+      (const int64_t *)slot_mapping.data_ptr(), num_tokens, layer_count, heads, head, block, layers.block_stride,
+      layers.num_blocks, src, kv, row_map.defined() ? (const int64_t *)row_map.data_ptr() : nullptr, idx.data_ptr(),
+      (int)idx.element_size(), n_sel, keys.size(0), select->k_out.data_ptr(), select->v_out.data_ptr(),
       select->k_out.stride(0), select->v_out.stride(0), stream));
+}
+
+void bulk_write(const at::Tensor &keys, const at::Tensor &values, const LayerLists &layers,
+                const at::Tensor &slot_mapping, const std::string &kv_cache_dtype, int64_t num_heads,
+                int64_t head_size, const SelectRows *select) {
+  // (looked at on every call: an address does not identify a tensor's shape)
+  bulk_write(keys, values, check_layers(layers), slot_mapping, kv_cache_dtype, num_heads, head_size, select);
 }
 
 void cache_write_fp4(const at::Tensor &key, const at::Tensor &value, const at::Tensor &key_cache,
@@ -241,7 +269,7 @@ void cache_write_fp4(const at::Tensor &key, const at::Tensor &value, const at::T
   check_rc(arctic_reshape_and_cache_flash_fp4(
       key.data_ptr(), value.data_ptr(), key.stride(0), value.stride(0), key_cache.data_ptr(), value_cache.data_ptr(),
       key_scale_cache.data_ptr(), value_scale_cache.data_ptr(), (const int64_t *)slot_mapping.data_ptr(),
-      slot_mapping.size(0), (int)num_heads, (int)head_size, (int)block_size, block_stride, page_stride, head_stride,
+      slot_mapping.size(0), to_int(num_heads, "num_heads"), to_int(head_size, "head_size"), to_int(block_size, "block_size"), block_stride, page_stride, head_stride,
       key_cache.size(0), half_code(key), current_stream()));
 }
 
@@ -314,14 +342,14 @@ at::Tensor add_ln_act(const char *fn, const at::Tensor &input, const OptTensor &
   if (given(token_ids)) {
     check_rc(arctic_speculator_embed_add_ln_act(
         out_2d.data_ptr(), in_2d.data_ptr(), z->data_ptr(), (const int64_t *)token_ids->data_ptr(), optional_ptr(weight),
-        optional_ptr(bias), rows, (int)hidden, in_2d.stride(0), z->stride(0), z->size(0), (float)alpha, (float)eps, act,
+        optional_ptr(bias), rows, to_int(hidden, "hidden"), in_2d.stride(0), z->stride(0), z->size(0), (float)alpha, (float)eps, act,
         (float)out_scale, code, current_stream()));
   } else if (!z_2d.defined() && act == ARCTIC_ACT_NONE && out_scale == 1.0) {
     check_rc(arctic_speculator_ln(out_2d.data_ptr(), in_2d.data_ptr(), optional_ptr(weight), optional_ptr(bias), rows,
-                                  (int)hidden, in_2d.stride(0), (float)eps, code, current_stream()));
+                                  to_int(hidden, "hidden"), in_2d.stride(0), (float)eps, code, current_stream()));
   } else {
     check_rc(arctic_speculator_add_ln_act(out_2d.data_ptr(), in_2d.data_ptr(), z_2d.defined() ? z_2d.data_ptr() : nullptr,
-                                          optional_ptr(weight), optional_ptr(bias), rows, (int)hidden, in_2d.stride(0),
+                                          optional_ptr(weight), optional_ptr(bias), rows, to_int(hidden, "hidden"), in_2d.stride(0),
                                           z_2d.defined() ? z_2d.stride(0) : 0, (float)alpha, (float)eps, act,
                                           (float)out_scale, code, current_stream()));
   }
@@ -406,13 +434,13 @@ std::tuple<at::Tensor, at::Tensor> sum_lstm(const at::Tensor &states_4d, const a
   if (given(token_ids)) {
     check_rc(arctic_sum_lstm_embedded(
         out_state.data_ptr(), out_cell.data_ptr(), s2.data_ptr(), z.data_ptr(), (const int64_t *)token_ids->data_ptr(), pc,
-        optional_ptr(w_cell), optional_ptr(b_cell), optional_ptr(w_state), optional_ptr(b_state), rows, (int)d_gate,
+        optional_ptr(w_cell), optional_ptr(b_cell), optional_ptr(w_state), optional_ptr(b_state), rows, to_int(d_gate, "d_gate"),
         s2.stride(0), z.stride(0), pc_stride, out_cell.stride(0), z.size(0), (float)alpha, (float)eps_cell,
         (float)eps_state, use_fast_gelu ? 1 : 0, code, current_stream()));
   } else {
     const auto entry = shared_z ? arctic_sum_lstm_shared_z : arctic_sum_lstm;
     check_rc(entry(out_state.data_ptr(), out_cell.data_ptr(), s2.data_ptr(), z2.data_ptr(), pc, optional_ptr(w_cell),
-                   optional_ptr(b_cell), optional_ptr(w_state), optional_ptr(b_state), rows, (int)d_gate, s2.stride(0),
+                   optional_ptr(b_cell), optional_ptr(w_state), optional_ptr(b_state), rows, to_int(d_gate, "d_gate"), s2.stride(0),
                    z2.stride(0), pc_stride, out_cell.stride(0), (float)alpha, (float)eps_cell, (float)eps_state,
                    use_fast_gelu ? 1 : 0, code, current_stream()));
   }
@@ -456,7 +484,7 @@ void move_rows(const char *fn, const TensorList &sources, const at::Tensor &indi
     dst_ptr[k] = dst.data_ptr();
   }
   const DeviceGuard guard(indices.device());
-  check_rc(arctic_gather_rows((int)count, src_ptr.data(), dst_ptr.data(), row_bytes.data(), src_stride.data(),
+  check_rc(arctic_gather_rows(to_int(count, "count"), src_ptr.data(), dst_ptr.data(), row_bytes.data(), src_stride.data(),
                               dst_stride.data(), indices.data_ptr(), (int)indices.element_size(), n, indexed_rows,
                               scatter ? 1 : 0, current_stream()));
 }
@@ -479,9 +507,8 @@ at::Tensor argmax_clamp(const at::Tensor &logits, int64_t max_index) {
   const int64_t rows = in_2d.size(0);
   at::Tensor out = at::empty(logits.sizes().slice(0, logits.dim() - 1), logits.options().dtype(at::kLong));
   if (rows == 0) return out;
-  TORCH_CHECK(cols <= 0x7fffffff, "speculator_argmax: more than 2^31 columns");
   const DeviceGuard guard(logits.device());
-  check_rc(arctic_argmax_clamp((int64_t *)out.data_ptr(), in_2d.data_ptr(), rows, (int)cols, in_2d.stride(0), max_index,
+  check_rc(arctic_argmax_clamp((int64_t *)out.data_ptr(), in_2d.data_ptr(), rows, to_int(cols, "cols"), in_2d.stride(0), max_index,
                                code, current_stream()));
   return out;
 }

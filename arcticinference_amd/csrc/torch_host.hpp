@@ -8,6 +8,7 @@
 
 #include <string>
 #include <tuple>
+#include <vector>
 
 namespace arctic_host {
 
@@ -29,9 +30,24 @@ struct SelectRows {
   const at::Tensor &v_out;
 };
 
+// What a bulk write needs to know of its layers, after every layer has been compared with layer 0: the four pointer
+// tables of the C ABI and the geometry all layers share.  Holds addresses, not tensors: whoever keeps one beyond the
+// call that made it must keep the tensors alive and unchanged as well (PreparedLayers of host_ext.cpp does).
+struct CheckedLayers {
+  int64_t num_layers = 0, block_size = 0, block_stride = 0, num_blocks = 0, cache_element_size = 0;
+  c10::Device device = c10::Device(c10::kCPU);
+  const char *scales_problem = nullptr;   // why the scales cannot serve an fp8 write, or nullptr
+  std::vector<const void *> key_caches, value_caches;
+  std::vector<const float *> k_scales, v_scales;
+};
+CheckedLayers check_layers(const LayerLists &layers);
+
 // reshape_and_cache_flash_bulk (csrc/custom_ops/reshape_and_cache_flash_bulk.cu:77-144) and, with `select`, the
-// variant that also gathers the selected rows (llama_swiftkv.py:663-679).
+// variant that also gathers the selected rows (llama_swiftkv.py:663-679).  The first form checks the layers itself.
 void bulk_write(const at::Tensor &keys, const at::Tensor &values, const LayerLists &layers,
+                const at::Tensor &slot_mapping, const std::string &kv_cache_dtype, int64_t num_heads,
+                int64_t head_size, const SelectRows *select);
+void bulk_write(const at::Tensor &keys, const at::Tensor &values, const CheckedLayers &layers,
                 const at::Tensor &slot_mapping, const std::string &kv_cache_dtype, int64_t num_heads,
                 int64_t head_size, const SelectRows *select);
 

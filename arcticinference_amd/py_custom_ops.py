@@ -230,6 +230,22 @@ def reshape_and_cache_flash_bulk(
                                         kv_cache_dtype, k_scales, v_scales, num_heads, head_size)
 
 
+def prepare_bulk_kv_layers(key_caches: List[torch.Tensor], value_caches: List[torch.Tensor],
+                           k_scales: List[torch.Tensor], v_scales: List[torch.Tensor]):
+    """The per-layer arguments of ``reshape_and_cache_flash_bulk``, checked once and held, for a caller that writes
+    the same layers on every step.  The reference's caller rebuilds its four lists - two views of every layer's cache
+    tensor and two attribute reads - on every engine step (arctic_inference/vllm/swiftkv/llama_swiftkv.py:594-615),
+    which costs it several times the host time of the write itself; with the object returned here a step is
+    ``layers.write(k_states, v_states, slot_mapping, kv_cache_dtype, num_heads, head_size)`` (or ``write_select`` with
+    ``logits_indices, k_out, v_out`` behind), same checks of the per-call arguments, same launch.  The object keeps an
+    alias of every tensor, so what it checked stays allocated and keeps its geometry; scales updated in place are seen.
+    Make a new one whenever a cache or scale tensor is REPLACED (a pool rebuilt after sleep / wake, a scale
+    re-assigned): it cannot notice that.  Not in the reference; not a registered operator (eager callers only)."""
+    _ops()
+    from . import _host_ext
+    return _host_ext.BulkKVLayers(key_caches, value_caches, k_scales, v_scales)
+
+
 def reshape_and_cache_flash_bulk_select(
     keys: torch.Tensor,
     values: torch.Tensor,

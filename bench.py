@@ -676,6 +676,9 @@ def host_overhead_route(route, calls=3000):
         slots = torch.arange(T, device=dev)
         out[f"reshape_and_cache_flash_bulk_{L}_layers"] = per_call_us(
             lambda: bulk(keys, values, kc, vc, slots, "fp8", ks, vs, H, D))
+        if route == "py_custom_ops":   # the per-layer arguments checked once and held (prepare_bulk_kv_layers)
+            write = ops.prepare_bulk_kv_layers(kc, vc, ks, vs).write
+            out[f"prepared_layers_write_{L}_layers"] = per_call_us(lambda: write(keys, values, slots, "fp8", H, D))
 
         # what the caller itself spends per step on the four lists it passes (llama_swiftkv.py:594-615: two views of
         # every layer's cache tensor and two attribute reads), for scale

@@ -373,3 +373,55 @@ def test_rows_narrower_than_the_layers_as_in_the_reference_unit_test(ops):
     with pytest.raises(RuntimeError, match="128 columns"):
         ops.reshape_and_cache_flash_bulk(keys[:4].to(DEV), values.to(DEV), dkc, dvc, slots.to(DEV), "auto", dscales, dscales,
                                          H, D)
+
+
+def test_prepared_layers_write_the_same_bytes_and_keep_their_tensors(ops):
+    """prepare_bulk_kv_layers(...).write(...) against the plain operator and the oracle; the object holds its tensors
+    (the caller's lists and views may go), sees scales updated in place, and refuses at construction what the operator
+    refuses per call."""
+    case = make_bulk_case(T=300, L=6, H=8, D=128, bs=16, NB=32, kv_cache_dtype="fp8", seed=80, std=1.5, pad_fraction=0.1)
+    d = bulk_case_to(case, DEV)
+    a = bulk_args(d)
+    layers = ops.prepare_bulk_kv_layers(a[2], a[3], a[6], a[7])
+    assert layers.num_layers == 6
+    keep = [b.clone() for b in d["bufs"]]
+    d["key_caches"], d["value_caches"] = None, None          # only the pool's own tensors stay with the caller
+    del a
+    layers.write(d["keys"], d["values"], d["slot_mapping"], "fp8", 8, 128)
+    torch.cuda.synchronize()
+    oracle.reshape_and_cache_flash_bulk(*bulk_args(case))
+    assert_bulk_equal(d["bufs"], case["bufs"])
+    # a scale changed in place is read by the next write (the kernel reads scales on the device)
+    for b, k in zip(d["bufs"], keep):
+        b.copy_(k)
+    case2 = make_bulk_case(T=300, L=6, H=8, D=128, bs=16, NB=32, kv_cache_dtype="fp8", seed=80, std=1.5, pad_fraction=0.1)
+    d["k_scales"][2].mul_(2.0)
+    case2["k_scales"][2] = case2["k_scales"][2] * 2.0
+    layers.write(d["keys"], d["values"], d["slot_mapping"], "fp8", 8, 128)
+    torch.cuda.synchronize()
+    oracle.reshape_and_cache_flash_bulk(*bulk_args(case2))
+    assert_bulk_equal(d["bufs"], case2["bufs"])
+    # the per-call checks are the operator's
+    with pytest.raises(RuntimeError, match="element size"):
+        layers.write(d["keys"], d["values"], d["slot_mapping"], "auto", 8, 128)
+    with pytest.raises(RuntimeError, match="Long"):
+        layers.write(d["keys"], d["values"], d["slot_mapping"].int(), "fp8", 8, 128)
+    with pytest.raises(RuntimeError, match="at least 300 rows"):
+        layers.write(d["keys"][:10], d["values"], d["slot_mapping"], "fp8", 8, 128)
+    # and so are the per-layer ones, at construction
+    bufs = d["bufs"]
+    small = torch.zeros(2, 2, 16, 8, 128, dtype=torch.uint8, device=DEV)
+    with pytest.raises(RuntimeError, match="must share dtype, block stride, number of blocks"):
+        ops.prepare_bulk_kv_layers([bufs[0][0], small[0]], [bufs[0][1], small[1]], d["k_scales"][:2], d["v_scales"][:2])
+    with pytest.raises(RuntimeError, match="value_caches"):
+        ops.prepare_bulk_kv_layers([bufs[0][0]], [], d["k_scales"][:1], d["v_scales"][:1])
+    bad = ops.prepare_bulk_kv_layers([bufs[0][0]], [bufs[0][1]], [d["k_scales"][0].double()], d["v_scales"][:1])
+    with pytest.raises(RuntimeError, match="must be float32"):          # the scales only matter to an fp8 write
+        bad.write(d["keys"], d["values"], d["slot_mapping"], "fp8", 8, 128)
+    # with the selection folded in: the rows index_select would give
+    idx = torch.tensor([5, 299, 0, 5], device=DEV)
+    k_out = torch.zeros(4, 6 * 1024, dtype=torch.bfloat16, device=DEV)
+    v_out = torch.zeros_like(k_out)
+    layers.write_select(d["keys"], d["values"], d["slot_mapping"], "fp8", 8, 128, idx, k_out, v_out)
+    torch.cuda.synchronize()
+    assert torch.equal(k_out, d["keys"].index_select(0, idx)) and torch.equal(v_out, d["values"].index_select(0, idx))

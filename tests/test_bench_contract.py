@@ -57,3 +57,9 @@ def test_the_json_line_carries_the_contract():
     assert d["value"] <= roof["achieved"] * 1.02 and abs(d["value"] - nbytes / d["ms_per_step"] / 1e6) < 0.01 * d["value"]
     cpu = d["cpu_baseline"]
     assert cpu["kind"] in ("port", "reference") and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
+    # the same write as PyTorch CPU operations, beside the port
+    torch_cpu = d["cpu_baseline_pytorch"]
+    assert torch_cpu["kind"] == "pytorch" and torch_cpu["cores"] >= 1 and torch_cpu["value"] > 0 and torch_cpu["sample"]
+    # where the traffic figure comes from: a day and a commit, not just a file
+    assert "measured on 20" in roof["traffic_source"] and "commit" in roof["traffic_source"]
+    assert d["extras"]["box_reference"]["torch_copy_1GiB_GBps"] > 0

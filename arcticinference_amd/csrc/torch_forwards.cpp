@@ -135,6 +135,9 @@ void bulk_write(const at::Tensor &keys, const at::Tensor &values, const CheckedL
     }
   }
   if (num_layers == 0) return;   // reference :87-89; no layer, so no column to write or to select either
+  TORCH_CHECK(num_heads >= 1 && head_size >= 1 && num_heads <= (1 << 24) && head_size <= (1 << 24) &&
+                  num_heads * head_size <= (1 << 24),
+              "reshape_and_cache_flash_bulk: num_heads and head_size must be positive and num_heads * head_size at most 2^24");
   const int64_t width = num_layers * num_heads * head_size;
   const int64_t num_tokens = slot_mapping.size(0);
   at::Tensor idx;
@@ -265,12 +268,19 @@ void cache_write_fp4(const at::Tensor &key, const at::Tensor &value, const at::T
               "reshape_and_cache_flash_fp4: cache last dim must be head_size / 2 packed bytes");
   TORCH_CHECK(key_scale_cache.numel() * 8 >= key_cache.numel() && value_scale_cache.numel() * 8 >= value_cache.numel(),
               "reshape_and_cache_flash_fp4: scale cache too small (one byte per 16 elements)");
+  for (const at::Tensor *t : {&value, &key_cache, &value_cache, &slot_mapping, &key_scale_cache, &value_scale_cache})
+    TORCH_CHECK(key.is_cuda() && t->device() == key.device(),
+                "reshape_and_cache_flash_fp4: all tensors must be on one CUDA device");
+  TORCH_CHECK(slot_mapping.dim() == 1 && (slot_mapping.size(0) <= 1 || slot_mapping.stride(0) == 1) &&
+                  key.size(0) >= slot_mapping.size(0),
+              "reshape_and_cache_flash_fp4: slot_mapping must be 1-D, contiguous and no longer than key has tokens");
   const DeviceGuard guard(key.device());
   check_rc(arctic_reshape_and_cache_flash_fp4(
       key.data_ptr(), value.data_ptr(), key.stride(0), value.stride(0), key_cache.data_ptr(), value_cache.data_ptr(),
       key_scale_cache.data_ptr(), value_scale_cache.data_ptr(), (const int64_t *)slot_mapping.data_ptr(),
-      slot_mapping.size(0), to_int(num_heads, "num_heads"), to_int(head_size, "head_size"), to_int(block_size, "block_size"), block_stride, page_stride, head_stride,
-      key_cache.size(0), half_code(key), current_stream()));
+      slot_mapping.size(0), to_int(num_heads, "num_heads"), to_int(head_size, "head_size"),
+      to_int(block_size, "block_size"), block_stride, page_stride, head_stride, key_cache.size(0), half_code(key),
+      current_stream()));
 }
 
 namespace {
@@ -303,13 +313,13 @@ at::Tensor add_ln_act(const char *fn, const at::Tensor &input, const OptTensor &
   TORCH_CHECK(hidden > 0, fn, ": hidden size must be > 0");
   TORCH_CHECK(input.stride(-1) == 1, fn, ": last dimension must be contiguous (stride -1 == 1)");
   if (given(weight)) {
-    TORCH_CHECK(weight->is_cuda(), "weight must be CUDA");
+    TORCH_CHECK(weight->is_cuda() && weight->device() == input.device(), "weight must be CUDA");
     TORCH_CHECK(weight->scalar_type() == dtype, "weight dtype must match input dtype");
     TORCH_CHECK(weight->dim() == 1 && weight->numel() == hidden, "weight must be 1D of size hidden");
     TORCH_CHECK(weight->is_contiguous(), "weight must be contiguous");
   }
   if (given(bias)) {
-    TORCH_CHECK(bias->is_cuda(), "bias must be CUDA");
+    TORCH_CHECK(bias->is_cuda() && bias->device() == input.device(), "bias must be CUDA");
     TORCH_CHECK(bias->scalar_type() == dtype, "bias dtype must match input dtype");
     TORCH_CHECK(bias->dim() == 1 && bias->numel() == hidden, "bias must be 1D of size hidden");
     TORCH_CHECK(bias->is_contiguous(), "bias must be contiguous");
@@ -342,16 +352,16 @@ at::Tensor add_ln_act(const char *fn, const at::Tensor &input, const OptTensor &
   if (given(token_ids)) {
     check_rc(arctic_speculator_embed_add_ln_act(
         out_2d.data_ptr(), in_2d.data_ptr(), z->data_ptr(), (const int64_t *)token_ids->data_ptr(), optional_ptr(weight),
-        optional_ptr(bias), rows, to_int(hidden, "hidden"), in_2d.stride(0), z->stride(0), z->size(0), (float)alpha, (float)eps, act,
-        (float)out_scale, code, current_stream()));
+        optional_ptr(bias), rows, to_int(hidden, "hidden"), in_2d.stride(0), z->stride(0), z->size(0), (float)alpha,
+        (float)eps, act, (float)out_scale, code, current_stream()));
   } else if (!z_2d.defined() && act == ARCTIC_ACT_NONE && out_scale == 1.0) {
     check_rc(arctic_speculator_ln(out_2d.data_ptr(), in_2d.data_ptr(), optional_ptr(weight), optional_ptr(bias), rows,
                                   to_int(hidden, "hidden"), in_2d.stride(0), (float)eps, code, current_stream()));
   } else {
     check_rc(arctic_speculator_add_ln_act(out_2d.data_ptr(), in_2d.data_ptr(), z_2d.defined() ? z_2d.data_ptr() : nullptr,
-                                          optional_ptr(weight), optional_ptr(bias), rows, to_int(hidden, "hidden"), in_2d.stride(0),
-                                          z_2d.defined() ? z_2d.stride(0) : 0, (float)alpha, (float)eps, act,
-                                          (float)out_scale, code, current_stream()));
+                                          optional_ptr(weight), optional_ptr(bias), rows, to_int(hidden, "hidden"),
+                                          in_2d.stride(0), z_2d.defined() ? z_2d.stride(0) : 0, (float)alpha, (float)eps,
+                                          act, (float)out_scale, code, current_stream()));
   }
   return out;
 }
@@ -367,6 +377,8 @@ std::tuple<at::Tensor, at::Tensor> sum_lstm(const at::Tensor &states_4d, const a
   const bool zero_cell = !given(prev_cell_d);
   TORCH_CHECK(states_4d.is_cuda() && z.is_cuda() && (zero_cell || prev_cell_d->is_cuda()),
               "sum_lstm: inputs must be CUDA tensors");
+  TORCH_CHECK(z.device() == states_4d.device() && (zero_cell || prev_cell_d->device() == states_4d.device()),
+              "sum_lstm: inputs must be on one device");
   TORCH_CHECK(z.scalar_type() == dtype && (zero_cell || prev_cell_d->scalar_type() == dtype),
               "sum_lstm: all input dtypes must match");
   const int64_t hidden4 = states_4d.size(-1);
@@ -386,7 +398,7 @@ std::tuple<at::Tensor, at::Tensor> sum_lstm(const at::Tensor &states_4d, const a
   for (int i = 0; i < 4; ++i) {
     if (!given(*vecs[i])) continue;
     const at::Tensor &t = **vecs[i];
-    TORCH_CHECK(t.is_cuda(), "sum_lstm: ", names[i], " must be CUDA");
+    TORCH_CHECK(t.is_cuda() && t.device() == states_4d.device(), "sum_lstm: ", names[i], " must be CUDA");
     TORCH_CHECK(t.scalar_type() == dtype, "sum_lstm: ", names[i], " dtype mismatch");
     TORCH_CHECK(t.numel() >= d_gate, "sum_lstm: ", names[i], " must have length >= D_eff");
     TORCH_CHECK(t.is_contiguous(), "sum_lstm: ", names[i], " must be contiguous");
@@ -434,15 +446,15 @@ std::tuple<at::Tensor, at::Tensor> sum_lstm(const at::Tensor &states_4d, const a
   if (given(token_ids)) {
     check_rc(arctic_sum_lstm_embedded(
         out_state.data_ptr(), out_cell.data_ptr(), s2.data_ptr(), z.data_ptr(), (const int64_t *)token_ids->data_ptr(), pc,
-        optional_ptr(w_cell), optional_ptr(b_cell), optional_ptr(w_state), optional_ptr(b_state), rows, to_int(d_gate, "d_gate"),
-        s2.stride(0), z.stride(0), pc_stride, out_cell.stride(0), z.size(0), (float)alpha, (float)eps_cell,
-        (float)eps_state, use_fast_gelu ? 1 : 0, code, current_stream()));
+        optional_ptr(w_cell), optional_ptr(b_cell), optional_ptr(w_state), optional_ptr(b_state), rows,
+        to_int(d_gate, "d_gate"), s2.stride(0), z.stride(0), pc_stride, out_cell.stride(0), z.size(0), (float)alpha,
+        (float)eps_cell, (float)eps_state, use_fast_gelu ? 1 : 0, code, current_stream()));
   } else {
     const auto entry = shared_z ? arctic_sum_lstm_shared_z : arctic_sum_lstm;
     check_rc(entry(out_state.data_ptr(), out_cell.data_ptr(), s2.data_ptr(), z2.data_ptr(), pc, optional_ptr(w_cell),
-                   optional_ptr(b_cell), optional_ptr(w_state), optional_ptr(b_state), rows, to_int(d_gate, "d_gate"), s2.stride(0),
-                   z2.stride(0), pc_stride, out_cell.stride(0), (float)alpha, (float)eps_cell, (float)eps_state,
-                   use_fast_gelu ? 1 : 0, code, current_stream()));
+                   optional_ptr(b_cell), optional_ptr(w_state), optional_ptr(b_state), rows, to_int(d_gate, "d_gate"),
+                   s2.stride(0), z2.stride(0), pc_stride, out_cell.stride(0), (float)alpha, (float)eps_cell,
+                   (float)eps_state, use_fast_gelu ? 1 : 0, code, current_stream()));
   }
   return std::make_tuple(state_shaped, cell_shaped);
 }
@@ -484,9 +496,9 @@ void move_rows(const char *fn, const TensorList &sources, const at::Tensor &indi
     dst_ptr[k] = dst.data_ptr();
   }
   const DeviceGuard guard(indices.device());
-  check_rc(arctic_gather_rows(to_int(count, "count"), src_ptr.data(), dst_ptr.data(), row_bytes.data(), src_stride.data(),
-                              dst_stride.data(), indices.data_ptr(), (int)indices.element_size(), n, indexed_rows,
-                              scatter ? 1 : 0, current_stream()));
+  check_rc(arctic_gather_rows(to_int(count, "count"), src_ptr.data(), dst_ptr.data(), row_bytes.data(),
+                              src_stride.data(), dst_stride.data(), indices.data_ptr(), (int)indices.element_size(), n,
+                              indexed_rows, scatter ? 1 : 0, current_stream()));
 }
 
 at::Tensor argmax_clamp(const at::Tensor &logits, int64_t max_index) {

@@ -183,7 +183,7 @@ def test_direct_c_abi_calls(ops):
 
 
 def test_side_stream(ops):
-    """The shim launches on torch's current stream, whichever that is."""
+    """The host layer launches on torch's current stream, whichever that is."""
     g = torch.Generator().manual_seed(15)
     x = torch.randn(64, 2048, generator=g).to(torch.bfloat16)
     dx = x.to(DEV)
@@ -245,7 +245,7 @@ def test_operators_trace_under_torch_compile(ops, backend):
 
 def test_reference_schemas_through_the_dispatcher(ops):
     """One eager call of each of the reference's four operators as torch.ops.arctic_inference.<op> (schema parsing,
-    dispatch on the CUDA key, the shim), compared with the oracle."""
+    dispatch on the CUDA key, the host layer), compared with the oracle."""
     t = torch.ops.arctic_inference
     for kv in ("fp8", "auto"):
         case = make_bulk_case(T=130, L=5, H=8, D=128, bs=16, NB=16, kv_cache_dtype=kv, seed=80, std=1.5, pad_fraction=0.1)

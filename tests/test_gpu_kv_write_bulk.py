@@ -1,8 +1,8 @@
 """GPU parity of the bulk KV-cache write against the CPU oracle: bit-exact.
 
 The calls go through the module's wrapper functions, as the reference's callers do: for GPU tensors outside
-torch.compile those call the Python shim directly (shim -> C ABI of libarctic_mi355x.so); the same shim is what the
-dispatcher runs for torch.ops.arctic_inference.reshape_and_cache_flash_bulk, which
+torch.compile those call the C++ host layer directly (_host_ext -> C ABI of libarctic_mi355x.so); the same function is
+what the dispatcher runs for torch.ops.arctic_inference.reshape_and_cache_flash_bulk, which
 tests/test_gpu_graph_and_abi.py::test_reference_schemas_through_the_dispatcher calls explicitly.
 """
 import pytest

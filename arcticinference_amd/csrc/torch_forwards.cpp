@@ -189,6 +189,7 @@ void bulk_write(const at::Tensor &keys, const at::Tensor &values, const CheckedL
               layers.cache_element_size, " does not match kv_cache_dtype '", kv_cache_dtype, "' (expected ", want_elem, ")");
   TORCH_CHECK(layers.device == keys.device() && values.device() == keys.device() && slot_mapping.device() == keys.device(),
               "reshape_and_cache_flash_bulk: all tensors must be on the same device");
+  TORCH_CHECK(keys.is_cuda(), "reshape_and_cache_flash_bulk: the tensors must be CUDA tensors");
   // Row t is read at t * stride(0), `width` elements long.  The reference looks at stride(0) only, and its own unit
   // test (tests/unit_tests/test_custom_ops.py:79-80) passes keys of shape [L * T, H * D]; rows narrower than `width`
   // are therefore accepted as long as the last row read still ends inside the tensor's storage.

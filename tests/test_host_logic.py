@@ -106,6 +106,45 @@ def test_argument_checks_mirror_the_reference(loaded):
         bulk(x32, x32, [cache, cache.view(4, 2, 1, 64)], [cache, cache], slots, "auto", [x32] * 2, [x32] * 2, 1, 32)
 
 
+def test_no_host_pointer_reaches_a_launch(loaded):
+    """Called directly (past the dispatcher, which would turn CPU tensors away), every host-layer function refuses
+    tensors that are not on a GPU before it hands a pointer to the library."""
+    f = ops._IMPLS
+    x = torch.randn(4, 64).bfloat16()
+    slots = torch.zeros(4, dtype=torch.int64)
+    cache = torch.zeros(2, 4, 1, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="must be CUDA tensors"):
+        f["reshape_and_cache_flash_bulk"](x, x, [cache[0]], [cache[1]], slots, "auto", [x], [x], 1, 64)
+    layers = ops.prepare_bulk_kv_layers([cache[0]], [cache[1]], [x], [x])
+    assert layers.num_layers == 1
+    with pytest.raises(RuntimeError, match="must be CUDA tensors"):
+        layers.write(x, x, slots, "auto", 1, 64)
+    with pytest.raises(RuntimeError, match="logits_indices must be a 1-D int32 or int64 CUDA tensor"):
+        f["reshape_and_cache_flash_bulk_select"](x, x, [cache[0]], [cache[1]], slots, "auto", [x], [x], 1, 64, slots, x, x)
+    key = torch.zeros(4, 2, 32).bfloat16()
+    packed, scales = torch.zeros(4, 1, 2, 16, dtype=torch.uint8), torch.zeros(4, 1, 2, 2, dtype=torch.uint8)
+    with pytest.raises(RuntimeError, match="one CUDA device"):
+        f["reshape_and_cache_flash_fp4"](key, key, packed, packed, slots, "nvfp4", x, x, scales, scales)
+    with pytest.raises(RuntimeError, match="contiguous 1-D CUDA tensor"):
+        f["gather_rows"]([x], slots, [x])
+    with pytest.raises(RuntimeError, match="contiguous 1-D CUDA tensor"):
+        f["scatter_rows"]([x], slots, [x])
+    with pytest.raises(RuntimeError, match="logits must be CUDA"):
+        f["speculator_argmax_cuda"](x, 63)
+    with pytest.raises(RuntimeError, match="input must be CUDA"):
+        f["speculator_add_ln_act_cuda"](x, x, None, None, 1.0, 1e-6, "gelu", 1.0)
+    with pytest.raises(RuntimeError, match="input must be CUDA"):
+        f["speculator_embed_add_ln_act_cuda"](x, x, slots, None, None, 1.0, 1e-6, "gelu", 1.0)
+    s4 = torch.randn(4, 256).bfloat16()
+    for name, args in (("sum_lstm_zero_cell_cuda", (s4, s4)), ("sum_lstm_shared_z_cuda", (s4, x, x)),
+                       ("sum_lstm_embedded_cuda", (s4, x, slots, x))):
+        with pytest.raises(RuntimeError, match="inputs must be CUDA tensors"):
+            f[name](*args, None, None, None, None, 1.0, 1e-6, 1e-6, False)
+    # sizes that do not fit the library's ints are an error, not a wrapped value
+    with pytest.raises(RuntimeError, match="num_heads and head_size must be positive"):
+        f["reshape_and_cache_flash_bulk"](x, x, [cache[0]], [cache[1]], slots, "auto", [x], [x], 1 << 40, 64)
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     """Without the shared object: try_load returns False (as the reference does) and the
     operators raise; nothing falls back to another implementation."""

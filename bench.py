@@ -357,6 +357,24 @@ def bench_decode_sizes(ops, dev, mem, steps):
     return out
 
 
+def bench_block_contiguous_slots(ops, dev, w, steps):
+    """The headline launch with the slot pattern a paged allocator produces for a prefill chunk instead of the
+    benchmark's random distinct slots: the chunk's tokens fill whole blocks in order (16 consecutive tokens = 16
+    consecutive slots = 16 KiB of one layer's K cache), the blocks themselves lie anywhere in the pool; the same
+    10 % of the tokens are padding.  Same source, same caches, same bytes."""
+    g = torch.Generator().manual_seed(12)
+    blocks = torch.randperm(w.NB, generator=g)[: (w.T + w.bs - 1) // w.bs]
+    slots = (blocks[:, None] * w.bs + torch.arange(w.bs)[None, :]).reshape(-1)[: w.T].clone()
+    slots[w.slots_cpu < 0] = -1
+    slots_dev = slots.to(dev)
+    args = list(w.args())
+    args[4] = slots_dev
+    f = lambda: ops.reshape_and_cache_flash_bulk(*args)
+    for _ in range(5):
+        f()
+    return kernel_stats(f, steps, w.bytes)
+
+
 def load_floor_kernels():
     """bench_floor.so: bare kernels that move the same bytes as the library's and compute nothing
     (built by __graft_entry__.build()).  None when it has not been built."""
@@ -1449,6 +1467,7 @@ def main():
 
     us = event_times_us(fn, args.steps)   # per launch, for the spread (a host hiccup between a launch's events shows here)
     if not args.no_extras:
+        extras["bulk_fp8_70b_block_contiguous_slots_serving_map"] = bench_block_contiguous_slots(ops, dev, w, args.steps)
         extras["bulk_fp8_70b_decode_sizes_serving_map"] = bench_decode_sizes(ops, dev, mem, args.steps)
         # The speculator's operators and the decode step are measured here, while the serving map is held: their
         # tensors (activations of a few GB at most) are then allocated behind weights and KV pool, as in a serving

@@ -63,7 +63,7 @@ def make_slots(num_tokens, num_slots, gen, pad_fraction):
 class BulkWorkload:
     """One bulk KV-write configuration, resident on the GPU."""
 
-    def __init__(self, name, T, L, H, D, bs, NB, kv, pad_fraction, seed, std, dev, bufs=None):
+    def __init__(self, name, T, L, H, D, bs, NB, kv, pad_fraction, seed, std, dev, bufs=None, make_bufs=None):
         self.name, self.T, self.L, self.H, self.D, self.bs, self.NB, self.kv = name, T, L, H, D, bs, NB, kv
         n = H * D
         self.n = n
@@ -81,8 +81,11 @@ class BulkWorkload:
         self.valid = int((self.slots_cpu >= 0).sum())
         quant = kv != "auto"
         cdt = torch.uint8 if quant else torch.bfloat16
-        # bufs: the layers' [2, NB, bs, H, D] cache tensors when they already exist (a serving pool)
-        self.bufs = bufs if bufs is not None else [torch.zeros(2, NB, bs, H, D, dtype=cdt, device=dev) for _ in range(L)]
+        # bufs: the layers' [2, NB, bs, H, D] cache tensors when they already exist (a serving pool); make_bufs: a
+        # function that allocates them now, behind the source
+        if bufs is None:
+            bufs = make_bufs() if make_bufs else [torch.zeros(2, NB, bs, H, D, dtype=cdt, device=dev) for _ in range(L)]
+        self.bufs = bufs
         assert len(self.bufs) == L and tuple(self.bufs[0].shape) == (2, NB, bs, H, D) and self.bufs[0].dtype == cdt
         self.key_caches = [b[0] for b in self.bufs]
         self.value_caches = [b[1] for b in self.bufs]
@@ -996,6 +999,34 @@ def bench_bulk_tp_heads(ops, dev, steps):
     return out
 
 
+def bench_source_before_pool(ops, dev, steps):
+    """The headline launch with the K/V source allocated BETWEEN the weights and the KV pool instead of behind the
+    pool.  A vLLM worker profiles a forward pass of its largest batch before it sizes and allocates the pool, and
+    torch's caching allocator keeps those activation blocks, so the k_states / v_states of an eager prefill chunk come
+    out of memory that lies in front of the pool; the loads of the launch (two thirds of its traffic) then come from
+    another HBM region than most of its stores.  Meant for a process of its own on an idle GPU (--only), where
+    allocation order is physical order."""
+    weights = torch.empty(66 << 30, dtype=torch.uint8, device=dev)
+    pool = []
+
+    def written_layers_of_a_new_pool():
+        torch.cuda.empty_cache()      # the source generator's temporaries go back; keys and values stay where they are
+        pool.extend(torch.empty(2, 65536, 16, 8, 128, dtype=torch.uint8, device=dev) for _ in range(80))
+        return pool[40:]
+
+    w = BulkWorkload("70B-SwiftKV-source-first", 16384, 40, 8, 128, 16, 65536, "fp8", 0.10, 2, 1.5, dev,
+                     make_bufs=written_layers_of_a_new_pool)
+    f = lambda: ops.reshape_and_cache_flash_bulk(*w.args())
+    box_reference(dev)                # the GPU out of its idle state, as in front of the headline
+    for _ in range(20):
+        f()
+    out = dict(kernel_stats(f, max(steps, 50), w.bytes),
+               memory_map="66 GiB resident weights (placeholder), then the K/V source (2.5 GiB), then the paged KV pool of "
+                          "all 80 layers, 65536 blocks = 2 GiB per layer; layers 40-79 are written")
+    del weights
+    return out
+
+
 def bench_lstm_rows(ops, dev, steps):
     """sum_lstm at 4096 against the number of rows (tokens) per call: the fixed cost of a launch against the
     90 112 bytes per row.  Enough buffer sets rotate inside one HIP graph that every call reads from HBM (at least
@@ -1348,6 +1379,7 @@ ONLY = {
     "swiftkv_select_decode_70b": lambda ops, dev, a: bench_row_gather(ops, dev, a.steps),
     "bulk_fp8_70b_tp_sharded_heads_compact_pool": lambda ops, dev, a: bench_bulk_tp_heads(ops, dev, a.steps),
     "host_us_per_call": lambda ops, dev, a: bench_host_overhead(),
+    "bulk_fp8_70b_source_before_pool": lambda ops, dev, a: bench_source_before_pool(ops, dev, a.steps),
 }
 
 

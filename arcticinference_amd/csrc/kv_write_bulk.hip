@@ -675,9 +675,9 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
 
       // A token's layers are split over `groups` workgroups.  Measured best on gfx950 (sweeps over the group count and
       // both shapes at 64 to 16384 tokens, 16 and 40 layers):
-      //  - above 8192 tokens, the 512-lane shape with up to five batches of 1024 chunks per workgroup (20 layers of
-      //    8 x 128 bf16) and at least about 1024 workgroups; a workgroup that would get less than two batches takes
-      //    the 256-lane shape instead;
+      //  - above 8192 tokens, the wide shape (batches of 1024 chunks by 1024 lanes, by 512 lanes when rows are
+      //    selected as well) with up to five batches per workgroup (20 layers of 8 x 128 bf16) and at least about
+      //    1024 workgroups; a workgroup that would get less than two batches takes the 256-lane shape instead;
       //  - below that, the 256-lane shape with about two batches of 1024 chunks per workgroup (8 such layers), more
       //    and smaller workgroups when fewer than about 2048 would exist otherwise, but never less than one batch each.
       int groups = 1;
@@ -707,7 +707,7 @@ static int bulk_entry(const char *fn, const void *keys, const void *values, int6
       }
       p.layers_per_group = (count + groups - 1) / groups;
       p.groups_per_token = (count + p.layers_per_group - 1) / p.layers_per_group;
-      // lanes of the shape launched below
+      // lanes of the shape launched below when rows are selected (the only case with index workgroups)
       const int lanes = !vec ? kScalarThreads : (wide && p.chunk_shift >= 0) ? 512 : 256;
       const int64_t index_blocks = p.indices ? (p.num_out_rows + lanes - 1) / lanes : 0;
       const int64_t grid = num_tokens * p.groups_per_token + index_blocks;

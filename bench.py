@@ -378,6 +378,78 @@ def bench_block_contiguous_slots(ops, dev, w, steps):
     return kernel_stats(f, steps, w.bytes)
 
 
+def bench_reference_decomposition(ops, dev, w, mem, steps, library_us):
+    """The same fp8 write in the launch decomposition of the reference's kernel (one workgroup per (layer, token), one
+    element per lane per step, reshape_and_cache_flash_bulk.cu:12-60,133-135), written for this GPU in bench_floor.hip:
+    what that decomposition costs on an MI355X, next to the library's kernel, on the same tensors.  First its bytes
+    are compared with the library's on two of the written caches; then the headline launch is timed, and the launch
+    of a 512-token decode batch with the K/V rows of 8 source sets in rotation inside a HIP graph (as
+    bulk_fp8_70b_decode_sizes_serving_map measures the library)."""
+    floor = load_floor_kernels()
+    if floor is None:
+        return "bench_floor.so is not built"
+
+    def tables(v):
+        table = lambda ts: torch.tensor([t.data_ptr() for t in ts], dtype=torch.int64, device=dev)
+        return table(v.key_caches), table(v.value_caches), table(v.k_scales), table(v.v_scales)
+
+    def launch(v, tabs):
+        rc = floor.floor_write_per_layer_and_token(
+            v.keys.data_ptr(), v.values.data_ptr(), tabs[0].data_ptr(), tabs[1].data_ptr(), v.slots.data_ptr(), v.T, v.L,
+            v.key_caches[0].stride(0), v.keys.stride(0), v.values.stride(0), v.H, v.D, v.bs, tabs[2].data_ptr(),
+            tabs[3].data_ptr(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, rc
+
+    tabs = tables(w)
+    # two of the caches, cleared (the pool is uninitialised memory), written by the library and kept; cleared again,
+    # written by the other kernel and compared
+    w.key_caches[0].zero_()
+    w.value_caches[w.L - 1].zero_()
+    ops.reshape_and_cache_flash_bulk(*w.args())
+    want_k, want_v = w.key_caches[0].clone(), w.value_caches[w.L - 1].clone()
+    w.key_caches[0].zero_()
+    w.value_caches[w.L - 1].zero_()
+    launch(w, tabs)
+    identical = bool(torch.equal(w.key_caches[0], want_k) and torch.equal(w.value_caches[w.L - 1], want_v))
+    del want_k, want_v
+    out = {"identical_bytes": identical}
+    for _ in range(3):
+        launch(w, tabs)
+    ref = kernel_stats(lambda: launch(w, tabs), max(5, steps // 4), w.bytes)
+    out["70b_prefill_16384_tokens_serving_map"] = {"reference_decomposition": ref, "library_kernel_us": round(library_us, 2),
+                                                   "library_is_faster_by": round(ref["kernel_us"] / library_us, 2)}
+    T, sets = 512, 8
+    ws = [BulkWorkload(f"decode-{T}", T, 40, 8, 128, 16, mem.NB, "fp8", 0.0, 20 + k, 1.5, dev, bufs=mem.written_layers())
+          for k in range(sets)]
+    per_set = [tables(v) for v in ws]
+    rounds = 2
+    times = {}
+    for name, call in (("library", lambda v, t: ops.reshape_and_cache_flash_bulk(*v.args())),
+                       ("reference_decomposition", launch)):
+        def run():
+            for _ in range(rounds):
+                for v, t in zip(ws, per_set):
+                    call(v, t)
+        run()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            run()
+        warm_replays(graph.replay)
+        times[name] = statistics.median(event_times_us(graph.replay, max(10, steps // 2))) / (sets * rounds)
+        del graph
+    out["decode_512_tokens_40_layers_serving_map"] = {
+        "reference_decomposition": {"us_per_call_graph": round(times["reference_decomposition"], 2),
+                                    "GBps": round(ws[0].bytes / times["reference_decomposition"] / 1e3, 1),
+                                    "hbm_frac": round(ws[0].bytes / times["reference_decomposition"] / 1e3 / HBM_PEAK_GBS, 4)},
+        "library_us_per_call_graph": round(times["library"], 2),
+        "library_is_faster_by": round(times["reference_decomposition"] / times["library"], 2)}
+    out["note"] = ("kernel time only: the reference's launcher also copies four pointer tables to the device with a "
+                   "synchronous copy each on every call (reshape_and_cache_flash_bulk.cu:121-131), which this comparison "
+                   "leaves out")
+    return out
+
+
 def load_floor_kernels():
     """bench_floor.so: bare kernels that move the same bytes as the library's and compute nothing
     (built by __graft_entry__.build()).  None when it has not been built."""
@@ -396,6 +468,9 @@ def load_floor_kernels():
     lib.floor_valu_rate.argtypes = [i32, i32, i32, vp, vp]
     lib.floor_node.argtypes = [vp, vp, i32, i32, i32, vp]
     lib.floor_row_read.argtypes = [vp, i64, i64, i32, vp, vp]
+    lib.floor_write_per_layer_and_token.argtypes = [vp, vp, vp, vp, vp, i64, i32, i64, i64, i64, i32, i32, i32, vp, vp, vp]
+    f32 = ctypes.c_float
+    lib.floor_sum_lstm_three_passes.argtypes = [vp] * 9 + [i64, i32, i64, i64, i64, i64, f32, f32, f32, vp]
     return lib
 
 
@@ -475,6 +550,20 @@ def bench_speculator(ops, dev, steps, warmup):
             floor.floor_lstm_traffic_staged(S[i % sets][k].data_ptr(), Z[i % sets][k].data_ptr(), C0[i % sets].data_ptr(),
                                             OS[0].data_ptr(), OS[1].data_ptr(), T, Hd, stream)
 
+    OC = [torch.empty(T, Hd, dtype=torch.bfloat16, device=dev) for _ in range(3)]
+
+    def lstm3_three_passes(i, state_out=None):
+        # the reference's kernel decomposition written for this GPU (bench_floor.hip): 128 lanes per row, three passes
+        stream = torch.cuda.current_stream().cuda_stream
+        cell = C0[i % sets]
+        for k in range(3):
+            rc = floor.floor_sum_lstm_three_passes(
+                (state_out if state_out is not None else OS[0]).data_ptr(), OC[k].data_ptr(), S[i % sets][k].data_ptr(),
+                Z[i % sets][k].data_ptr(), cell.data_ptr(), w_cell.data_ptr(), b_cell.data_ptr(), w_state.data_ptr(),
+                b_state.data_ptr(), T, Hd, 4 * Hd, 4 * Hd, Hd, Hd, alpha, 1e-6, 1e-6, stream)
+            assert rc == 0, rc
+            cell = OC[k]
+
     def ln_traffic_only(i):
         floor.floor_ln_traffic(X[i % sets].data_ptr(), OS[0].data_ptr(), T, Hd, torch.cuda.current_stream().cuda_stream)
 
@@ -489,6 +578,7 @@ def bench_speculator(ops, dev, steps, warmup):
         cases.insert(1, ("sum_lstm_traffic_only_floor", lstm3_traffic_only, 22 * Hd * T, 3))
         cases.insert(2, ("sum_lstm_traffic_only_in_stages", lstm3_traffic_staged, 22 * Hd * T, 3))
         cases.append(("speculator_ln_traffic_only_floor", ln_traffic_only, 4 * Hd * T, 1))
+        cases.insert(3, ("sum_lstm_reference_decomposition", lstm3_three_passes, 22 * Hd * T, 3))
     out = {}
     for name, fn, per_call, calls in cases:
         for i in range(warmup):
@@ -510,6 +600,17 @@ def bench_speculator(ops, dev, steps, warmup):
         out[name].update({"us_per_call_graph": round(med, 2),
                           "GBps_graph": round(per_call / med / 1e3, 1),
                           "hbm_frac_graph": round(per_call / med / 1e3 / HBM_PEAK_GBS, 4)})
+    if floor is not None:
+        # the comparison kernel computes the same function: third step's state and cell against the library's, within
+        # the operators' tolerance (1e-2 relative + 2e-2 absolute)
+        cell = C0[0]
+        for k in range(3):
+            state, cell = ops.sum_lstm(S[0][k], Z[0][k], cell, w_cell, b_cell, w_state, b_state, alpha, 1e-6, 1e-6, False)
+        lstm3_three_passes(0, state_out=OS[1])
+        close = lambda a, b: bool(torch.allclose(a.float(), b.float(), rtol=1e-2, atol=2e-2))
+        out["sum_lstm_reference_decomposition"]["within_tolerance_of_the_library"] = close(OS[1], state) and close(OC[2], cell)
+        out["sum_lstm_reference_decomposition"]["library_is_faster_by"] = round(
+            out["sum_lstm_reference_decomposition"]["us_per_call_graph"] / out["sum_lstm"]["us_per_call_graph"], 2)
     return out
 
 
@@ -1501,6 +1602,7 @@ def main():
     if not args.no_extras:
         extras["bulk_fp8_70b_block_contiguous_slots_serving_map"] = bench_block_contiguous_slots(ops, dev, w, args.steps)
         extras["bulk_fp8_70b_decode_sizes_serving_map"] = bench_decode_sizes(ops, dev, mem, args.steps)
+        extras["bulk_fp8_reference_decomposition"] = bench_reference_decomposition(ops, dev, w, mem, args.steps, kernel_us)
         # The speculator's operators and the decode step are measured here, while the serving map is held: their
         # tensors (activations of a few GB at most) are then allocated behind weights and KV pool, as in a serving
         # process, and in the physical order of a fresh process.  Allocated late, after the map has been handed back

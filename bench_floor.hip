@@ -1,5 +1,6 @@
-// Bare kernels that bench.py times next to the library's kernels: what the same bytes cost on this GPU
-// when nothing is computed.  Measurement aid only; nothing in the package uses it.
+// Kernels that bench.py times next to the library's: what the same bytes cost on this GPU when nothing is
+// computed, and what the reference's own launch decompositions of two operators cost on it.  Measurement aid only;
+// nothing in the package uses it.
 //
 //   floor_lstm_traffic   the loads and stores of sum_lstm (nine 16-byte loads per lane from the rows of
 //                        states, z4 and prev_cell, two 16-byte stores), one workgroup per row, no arithmetic
@@ -12,12 +13,21 @@
 //   floor_stream         load-only, store-only or a 2:1 load:store stream in 64 KiB pieces, the pieces dealt
 //                        round robin over up to three buffers (which the caller places in different regions
 //                        of the HBM); the 2:1 stream also with its stores scattered as rows of 1 KiB
+//   floor_write_per_layer_and_token  the bf16 -> e4m3 bulk write in the launch decomposition of the reference's kernel
+//                        (csrc/custom_ops/reshape_and_cache_flash_bulk.cu:12-60, 133-135), written for this GPU: what
+//                        that decomposition costs here, next to the library's
+//   floor_sum_lstm_three_passes  sum_lstm (bf16, exact GELU) in the decomposition of the reference's kernel
+//                        (csrc/custom_ops/sum_lstm.cu:28-191, launched :401-418): 128 lanes per row, three passes over
+//                        global memory, two block sums, the C library's expf and erff
 //   floor_stream_resident the scattered 2:1 stream once more, shaped for bandwidth alone: as many workgroups of 1024
 //                        lanes as stay resident (one or two per CU), each looping over pieces with all of a piece's
 //                        loads (4 or 8 per lane) requested before the first store
 #include <hip/hip_runtime.h>
+#include <hipcub/hipcub.hpp>
 
 #include <cstdint>
+
+#include "arcticinference_amd/csrc/common.hpp"   // 16-byte chunks of bf16 and their conversion to and from fp32
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
@@ -336,5 +346,173 @@ extern "C" int floor_stream(void *const *src, int nsrc, void *const *dst, int nd
   const int scatter_bits = __builtin_ctzll((unsigned long long)(pieces * 32));
   hipLaunchKernelGGL(stream_kernel, dim3(8192), dim3(256), 0, (hipStream_t)stream, a, nsrc, b, ndst, pieces, mode,
                      scatter_bits, (unsigned *)sink);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+// The bulk write as the reference decomposes it (csrc/custom_ops/reshape_and_cache_flash_bulk.cu:12-60): one workgroup
+// per (layer, token) of min(n, 512) lanes; a lane moves one element per step - a 2-byte load of K and of V, an fp32
+// division by the layer's scale, a conversion, a 1-byte store each - and finds its place in the cache row with a
+// division and a remainder by head_size per element; the slot, the two cache pointers and the two scale pointers are
+// read from device memory by every workgroup.  bf16 source, e4m3 cache.  Same bytes out as the library's kernel
+// (bench.py compares them); a measurement aid, not a code path of the package.
+__device__ __forceinline__ unsigned char e4m3_of(float q) {
+  if (q != q) return (unsigned char)(0x7fu | ((__float_as_uint(q) >> 24) & 0x80u));
+  const float c = __builtin_amdgcn_fmed3f(q, -448.0f, 448.0f);
+  return (unsigned char)(__builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false) & 0xff);
+}
+
+__global__ void write_per_layer_and_token_kernel(const unsigned short *keys, const unsigned short *values,
+                                                 const int64_t *key_cache_ptrs, const int64_t *value_cache_ptrs,
+                                                 const int64_t *slot_mapping, int64_t block_stride, int64_t key_stride,
+                                                 int64_t value_stride, int num_heads, int head_size, int block_size,
+                                                 const int64_t *k_scale_ptrs, const int64_t *v_scale_ptrs) {
+  const int64_t layer = blockIdx.x, token = blockIdx.y;
+  const int64_t slot = slot_mapping[token];
+  if (slot < 0) return;   // a padding token
+  const int64_t block = slot / block_size, in_block = slot % block_size;
+  const int n = num_heads * head_size;
+  unsigned char *key_cache = (unsigned char *)key_cache_ptrs[layer];
+  unsigned char *value_cache = (unsigned char *)value_cache_ptrs[layer];
+  const float *k_scale = (const float *)k_scale_ptrs[layer];
+  const float *v_scale = (const float *)v_scale_ptrs[layer];
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int head = i / head_size, in_head = i % head_size;
+    const int64_t dst = block * block_stride + in_block * n + (int64_t)head * head_size + in_head;
+    const float k = __uint_as_float((unsigned)keys[token * key_stride + layer * n + i] << 16);
+    const float v = __uint_as_float((unsigned)values[token * value_stride + layer * n + i] << 16);
+    key_cache[dst] = e4m3_of(k / *k_scale);
+    value_cache[dst] = e4m3_of(v / *v_scale);
+  }
+}
+
+// The four pointer tables are int64[num_layers] in DEVICE memory (the reference's launcher copies them there on
+// every call, :104-131).  Strides in elements.
+extern "C" int floor_write_per_layer_and_token(const void *keys, const void *values, const void *key_cache_ptrs,
+                                               const void *value_cache_ptrs, const void *slot_mapping,
+                                               int64_t num_tokens, int num_layers, int64_t block_stride,
+                                               int64_t key_stride, int64_t value_stride, int num_heads, int head_size,
+                                               int block_size, const void *k_scale_ptrs, const void *v_scale_ptrs,
+                                               void *stream) {
+  if (num_tokens <= 0 || num_tokens > 65535 || num_layers <= 0 || num_heads <= 0 || head_size <= 0 || block_size <= 0 ||
+      (int64_t)num_heads * head_size > (1 << 24))
+    return 1;
+  const int n = num_heads * head_size;
+  hipLaunchKernelGGL(write_per_layer_and_token_kernel, dim3((unsigned)num_layers, (unsigned)num_tokens),
+                     dim3((unsigned)(n < 512 ? n : 512)), 0, (hipStream_t)stream, (const unsigned short *)keys,
+                     (const unsigned short *)values, (const int64_t *)key_cache_ptrs, (const int64_t *)value_cache_ptrs,
+                     (const int64_t *)slot_mapping, block_stride, key_stride, value_stride, num_heads, head_size,
+                     block_size, (const int64_t *)k_scale_ptrs, (const int64_t *)v_scale_ptrs);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+// sum_lstm as the reference decomposes it (csrc/custom_ops/sum_lstm.cu:28-191): one workgroup of 128 lanes per row,
+// 16 bytes per lane and step, and three passes over global memory - the cell's pre-activation alone for its sum of
+// squares; then the forget, input and cell pre-activations with the previous cell, for the new cell, which is stored;
+// then the stored cell read back, with the output gate's pre-activation, for the state - with a block-wide sum after
+// each of the first two, and sigmoid and GELU through the C library's expf and erff.  bf16, all four vectors given.
+// Results agree with the library's kernel within the operators' tolerance (bench.py checks); a measurement aid.
+namespace three_passes {
+
+constexpr int kLanes = 128;
+
+__device__ __forceinline__ float sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float gelu(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
+
+__device__ __forceinline__ void load8(const char *p, int chunk, float (&f)[8]) {
+  arctic::Chunk::load(p + (int64_t)chunk * 16).unpack<arctic::BF16>(f);
+}
+// s + alpha * z of gate g (0 forget, 1 input, 2 output, 3 cell), chunk i
+__device__ __forceinline__ void pre_activation(const char *s, const char *z, int64_t gate_bytes, int g, int i,
+                                               float alpha, float (&f)[8]) {
+  float a[8], b[8];
+  load8(s + g * gate_bytes, i, a);
+  load8(z + g * gate_bytes, i, b);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) f[k] = a[k] + alpha * b[k];
+}
+
+__global__ __launch_bounds__(kLanes) void sum_lstm_kernel(char *out_state, char *out_cell, const char *states,
+                                                          const char *z4, const char *prev_cell, const char *w_cell,
+                                                          const char *b_cell, const char *w_state, const char *b_state,
+                                                          int64_t s_pitch, int64_t z_pitch, int64_t c_pitch,
+                                                          int64_t o_pitch, int D, float alpha, float eps_cell,
+                                                          float eps_state) {
+  typedef hipcub::BlockReduce<float, kLanes> Reduce;
+  __shared__ typename Reduce::TempStorage scratch0, scratch1;
+  __shared__ float inv_rms_pre, inv_rms_cell;
+  const int64_t row = blockIdx.x;
+  const char *s = states + row * s_pitch, *z = z4 + row * z_pitch, *pc = prev_cell + row * c_pitch;
+  char *cell_row = out_cell + row * o_pitch, *state_row = out_state + row * o_pitch;
+  const int chunks = D / 8;
+  const int64_t gate_bytes = (int64_t)D * 2;
+
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < chunks; i += kLanes) {
+    float c[8];
+    pre_activation(s, z, gate_bytes, 3, i, alpha, c);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) ss += c[k] * c[k];
+  }
+  float total = Reduce(scratch0).Sum(ss);
+  if (threadIdx.x == 0) inv_rms_pre = rsqrtf(total / (float)D + eps_cell);
+  __syncthreads();
+
+  ss = 0.f;
+  for (int i = threadIdx.x; i < chunks; i += kLanes) {
+    float f[8], in[8], c[8], p[8], w[8], b[8], cell[8];
+    pre_activation(s, z, gate_bytes, 0, i, alpha, f);
+    pre_activation(s, z, gate_bytes, 1, i, alpha, in);
+    pre_activation(s, z, gate_bytes, 3, i, alpha, c);
+    load8(pc, i, p);
+    load8(w_cell, i, w);
+    load8(b_cell, i, b);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      float normed = c[k] * inv_rms_pre;
+      normed *= w[k];
+      normed += b[k];
+      cell[k] = p[k] * sigmoid(f[k]) + gelu(normed) * sigmoid(in[k]);
+      ss += cell[k] * cell[k];
+    }
+    arctic::Chunk::pack<arctic::BF16>(cell).store(cell_row + (int64_t)i * 16);
+  }
+  total = Reduce(scratch1).Sum(ss);
+  if (threadIdx.x == 0) inv_rms_cell = rsqrtf(total / (float)D + eps_state);
+  __syncthreads();
+
+  for (int i = threadIdx.x; i < chunks; i += kLanes) {
+    float c[8], o[8], w[8], b[8], state[8];
+    load8(cell_row, i, c);   // the rounded cell this lane stored above
+    pre_activation(s, z, gate_bytes, 2, i, alpha, o);
+    load8(w_state, i, w);
+    load8(b_state, i, b);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      float normed = c[k] * inv_rms_cell;
+      normed *= w[k];
+      normed += b[k];
+      state[k] = gelu(normed) * sigmoid(o[k]);
+    }
+    arctic::Chunk::pack<arctic::BF16>(state).store(state_row + (int64_t)i * 16);
+  }
+}
+
+}  // namespace three_passes
+
+// bf16 rows; pitches in elements; D a multiple of 8; every pointer 16-byte aligned and none null.
+extern "C" int floor_sum_lstm_three_passes(void *out_state, void *out_cell, const void *states, const void *z4,
+                                           const void *prev_cell, const void *w_cell, const void *b_cell,
+                                           const void *w_state, const void *b_state, int64_t rows, int D, int64_t s_pitch,
+                                           int64_t z_pitch, int64_t c_pitch, int64_t o_pitch, float alpha, float eps_cell,
+                                           float eps_state, void *stream) {
+  if (rows <= 0 || rows > 0x7fffffffLL || D <= 0 || D % 8 || (s_pitch | z_pitch | c_pitch | o_pitch) % 8) return 1;
+  const void *all[9] = {out_state, out_cell, states, z4, prev_cell, w_cell, b_cell, w_state, b_state};
+  for (const void *p : all)
+    if (!p || ((uintptr_t)p & 15)) return 1;
+  hipLaunchKernelGGL(three_passes::sum_lstm_kernel, dim3((unsigned)rows), dim3(three_passes::kLanes), 0,
+                     (hipStream_t)stream, (char *)out_state, (char *)out_cell, (const char *)states, (const char *)z4,
+                     (const char *)prev_cell, (const char *)w_cell, (const char *)b_cell, (const char *)w_state,
+                     (const char *)b_state, s_pitch * 2, z_pitch * 2, c_pitch * 2, o_pitch * 2, D, alpha, eps_cell,
+                     eps_state);
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }

@@ -471,6 +471,7 @@ def load_floor_kernels():
     lib.floor_write_per_layer_and_token.argtypes = [vp, vp, vp, vp, vp, i64, i32, i64, i64, i64, i32, i32, i32, vp, vp, vp]
     f32 = ctypes.c_float
     lib.floor_sum_lstm_three_passes.argtypes = [vp] * 9 + [i64, i32, i64, i64, i64, i64, f32, f32, f32, vp]
+    lib.floor_ln_two_passes.argtypes = [vp, vp, vp, vp, i64, i32, i64, f32, vp]
     return lib
 
 
@@ -564,6 +565,13 @@ def bench_speculator(ops, dev, steps, warmup):
             assert rc == 0, rc
             cell = OC[k]
 
+    def ln_two_passes(i, out=None):
+        # the reference's kernel decomposition written for this GPU (bench_floor.hip): 256 lanes per row, two passes
+        rc = floor.floor_ln_two_passes((out if out is not None else OS[0]).data_ptr(), X[i % sets].data_ptr(),
+                                       w_cell.data_ptr(), b_cell.data_ptr(), T, Hd, Hd, 1e-6,
+                                       torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, rc
+
     def ln_traffic_only(i):
         floor.floor_ln_traffic(X[i % sets].data_ptr(), OS[0].data_ptr(), T, Hd, torch.cuda.current_stream().cuda_stream)
 
@@ -579,6 +587,7 @@ def bench_speculator(ops, dev, steps, warmup):
         cases.insert(2, ("sum_lstm_traffic_only_in_stages", lstm3_traffic_staged, 22 * Hd * T, 3))
         cases.append(("speculator_ln_traffic_only_floor", ln_traffic_only, 4 * Hd * T, 1))
         cases.insert(3, ("sum_lstm_reference_decomposition", lstm3_three_passes, 22 * Hd * T, 3))
+        cases.append(("speculator_ln_reference_decomposition", ln_two_passes, 4 * Hd * T, 1))
     out = {}
     for name, fn, per_call, calls in cases:
         for i in range(warmup):
@@ -611,6 +620,11 @@ def bench_speculator(ops, dev, steps, warmup):
         out["sum_lstm_reference_decomposition"]["within_tolerance_of_the_library"] = close(OS[1], state) and close(OC[2], cell)
         out["sum_lstm_reference_decomposition"]["library_is_faster_by"] = round(
             out["sum_lstm_reference_decomposition"]["us_per_call_graph"] / out["sum_lstm"]["us_per_call_graph"], 2)
+        ln_two_passes(0, out=OS[1])
+        out["speculator_ln_reference_decomposition"]["within_tolerance_of_the_library"] = close(
+            OS[1], ops.speculator_ln(X[0], w_cell, b_cell, 1e-6))
+        out["speculator_ln_reference_decomposition"]["library_is_faster_by"] = round(
+            out["speculator_ln_reference_decomposition"]["us_per_call_graph"] / out["speculator_ln"]["us_per_call_graph"], 2)
     return out
 
 

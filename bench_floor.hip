@@ -19,6 +19,9 @@
 //   floor_sum_lstm_three_passes  sum_lstm (bf16, exact GELU) in the decomposition of the reference's kernel
 //                        (csrc/custom_ops/sum_lstm.cu:28-191, launched :401-418): 128 lanes per row, three passes over
 //                        global memory, two block sums, the C library's expf and erff
+//   floor_ln_two_passes  speculator_ln (bf16, weight and bias) in the reference's decomposition
+//                        (csrc/custom_ops/speculator_ln.cu:21-107, launched :203-207): 256 lanes per row, the row read
+//                        twice from global memory with a block sum between
 //   floor_stream_resident the scattered 2:1 stream once more, shaped for bandwidth alone: as many workgroups of 1024
 //                        lanes as stay resident (one or two per CU), each looping over pieces with all of a piece's
 //                        loads (4 or 8 per lane) requested before the first store
@@ -514,5 +517,59 @@ extern "C" int floor_sum_lstm_three_passes(void *out_state, void *out_cell, cons
                      (const char *)prev_cell, (const char *)w_cell, (const char *)b_cell, (const char *)w_state,
                      (const char *)b_state, s_pitch * 2, z_pitch * 2, c_pitch * 2, o_pitch * 2, D, alpha, eps_cell,
                      eps_state);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+// speculator_ln as the reference decomposes it (csrc/custom_ops/speculator_ln.cu:21-107; 256 lanes per row from 256
+// rows on, :203-207): a first pass over the row for its sum of squares, a block sum, a second pass that reads the row
+// again, scales it, applies weight and bias and stores.  bf16, weight and bias given, output rows dense.
+namespace two_passes {
+
+constexpr int kLanes = 256;
+
+__global__ __launch_bounds__(kLanes) void ln_kernel(char *out, const char *in, const char *weight, const char *bias,
+                                                    int64_t in_pitch, int hidden, float eps) {
+  typedef hipcub::BlockReduce<float, kLanes> Reduce;
+  __shared__ typename Reduce::TempStorage scratch;
+  __shared__ float inv_rms;
+  const char *row_in = in + (int64_t)blockIdx.x * in_pitch;
+  char *row_out = out + (int64_t)blockIdx.x * hidden * 2;
+  const int chunks = hidden / 8;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < chunks; i += kLanes) {
+    float x[8];
+    three_passes::load8(row_in, i, x);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) ss += x[k] * x[k];
+  }
+  const float total = Reduce(scratch).Sum(ss);
+  if (threadIdx.x == 0) inv_rms = rsqrtf(total / (float)hidden + eps);
+  __syncthreads();
+  for (int i = threadIdx.x; i < chunks; i += kLanes) {
+    float x[8], w[8], b[8], y[8];
+    three_passes::load8(row_in, i, x);
+    three_passes::load8(weight, i, w);
+    three_passes::load8(bias, i, b);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      y[k] = x[k] * inv_rms;
+      y[k] *= w[k];
+      y[k] += b[k];
+    }
+    arctic::Chunk::pack<arctic::BF16>(y).store(row_out + (int64_t)i * 16);
+  }
+}
+
+}  // namespace two_passes
+
+// bf16; in_pitch in elements; hidden a multiple of 8; every pointer 16-byte aligned and none null.
+extern "C" int floor_ln_two_passes(void *out, const void *in, const void *weight, const void *bias, int64_t rows,
+                                   int hidden, int64_t in_pitch, float eps, void *stream) {
+  if (rows <= 0 || rows > 0x7fffffffLL || hidden <= 0 || hidden % 8 || in_pitch % 8) return 1;
+  const void *all[4] = {out, in, weight, bias};
+  for (const void *p : all)
+    if (!p || ((uintptr_t)p & 15)) return 1;
+  hipLaunchKernelGGL(two_passes::ln_kernel, dim3((unsigned)rows), dim3(two_passes::kLanes), 0, (hipStream_t)stream,
+                     (char *)out, (const char *)in, (const char *)weight, (const char *)bias, in_pitch * 2, hidden, eps);
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }

@@ -78,6 +78,42 @@ def test_every_finite_sixteen_bit_value(ops, dtype):
     run_both(ops, key, value, kc, vc, ksc, vsc, slots)
 
 
+@pytest.mark.parametrize("nhd,bs", [(True, 16), (False, 8)])
+def test_dequantised_cache_against_the_fp16_rows_as_in_the_reference_test(ops, nhd, bs):
+    """The check of the reference's own test (tests/unit_tests/test_reshape_and_cache_flash_nvfp4.py:77-196) on the
+    kernel's output, with its sizes and inputs (64 tokens, 16 heads x 128, blocks of 16, randn * 0.5 in fp16,
+    slot t = t, zeroed caches): the cache is decoded with the test's formulas (e2m1 nibbles times the e4m3 group
+    scale) and compared with the rows an fp16 cache would hold.  The reference prints the error; here it is bounded:
+    the e2m1 grid has gaps of at most 2 and the scale is within 1/16 of amax / 6, so |x - decoded| <= 1.07 * scale,
+    and the relative RMS error is that of a 4-bit code.  (Heads-first caches with blocks of 8: with as many heads as
+    slots per block the operator, like the reference's, takes a cache for tokens-first.)"""
+    T, H, D = 64, 16, 128
+    NB = T // bs
+    g = torch.Generator().manual_seed(0)
+    key = (torch.randn(T, H, D, generator=g) * 0.5).to(torch.float16)
+    value = (torch.randn(T, H, D, generator=g) * 0.5).to(torch.float16)
+    slots = torch.arange(T, dtype=torch.int64)
+    shape = (NB, bs, H) if nhd else (NB, H, bs)
+    kc, vc = (torch.zeros(*shape, D // 2, dtype=torch.uint8, device=DEV) for _ in range(2))
+    ksc, vsc = (torch.zeros(*shape, D // 16, dtype=torch.uint8, device=DEV) for _ in range(2))
+    ops.reshape_and_cache_flash_fp4(key.to(DEV), value.to(DEV), kc, vc, ksc, vsc, slots.to(DEV), "fp4", ZERO.to(DEV),
+                                    ZERO.to(DEV))
+    torch.cuda.synchronize()
+    for src, cache, scales in ((key, kc.cpu(), ksc.cpu()), (value, vc.cpu(), vsc.cpu())):
+        if not nhd:   # [blocks, heads, block, bytes] -> [blocks, block, heads, bytes]
+            cache, scales = cache.transpose(1, 2), scales.transpose(1, 2)
+        packed = cache.reshape(T, H, D // 2)              # slot t = t: token t sits in block t / bs at offset t % bs
+        group_scale = oracle.e4m3fn_decode(scales.reshape(T, H, D // 16)).repeat_interleave(16, dim=-1)
+        nibbles = torch.stack((packed & 0xF, packed >> 4), dim=-1).reshape(T, H, D)
+        decoded = oracle.e2m1_decode(nibbles) * group_scale
+        x = src.float()
+        assert bool(((x - decoded).abs() <= 1.07 * group_scale + 1e-6).all())
+        assert float(((x - decoded).pow(2).mean() / x.pow(2).mean()).sqrt()) < 0.12
+        # what the reference's test prints: mean and largest absolute error against the fp16 rows
+        assert float((x - decoded.to(torch.float16).float()).abs().mean()) < 0.05
+        assert float((x - decoded.to(torch.float16).float()).abs().max()) < 0.5
+
+
 def test_rounding_ties(ops):
     """Groups whose scale is an exact power of two, holding every e2m1 tie and its neighbours."""
     ties = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0])
